@@ -1,0 +1,117 @@
+/* C ABI of the MI355X int4-KV GQA attention library (libyka.so).
+ *
+ * Conventions follow the reference's include/yskn_abi.h and src/c_api.cpp:
+ *   - opaque handle, created by an open call and released by a close call (yskn_abi.h:21-24);
+ *   - every call returns int: 0 = ok, -1 = error; the message of the last error of the calling thread is
+ *     returned by yka_last_error() (c_api.cpp:17,33,49);
+ *   - the stream is passed as void* (yskn_abi.h:19 "void* cuda_stream"); here it is a hipStream_t;
+ *   - the position of the pass lives on the device (const int* d_pos) and is read by the kernels, never by the
+ *     host, so a captured graph replays at new positions (engine35.cpp:2365-2375, q35_atxpk3.cuh:183);
+ *   - the launch path (yka_append / yka_attend / yka_append_attend) allocates nothing, synchronises nothing and
+ *     sets no function attribute: everything is reserved in yka_kv_open (engine35.cpp:323-326);
+ *   - hooks that take host pointers allocate, copy, launch, synchronise and free inside (src/kvx_probe.cu).
+ * One caller at a time per handle; any host thread may call (the device of the handle is made current first,
+ * as on_gpu does in c_api.cpp:22-31).
+ *
+ * Fixed format: head_dim 128; symmetric signed int4 codes stored as q+8, two per byte, even channel in the low
+ * nibble; one fp16 scale per (token, kv head, 32-channel group); Q, new K/V and outputs are fp16 bit patterns.
+ */
+#ifndef YKA_ABI_H
+#define YKA_ABI_H
+#include <stddef.h>
+#include <stdint.h>
+#define YKA_API __attribute__((visibility("default")))
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct yka_kv yka_kv;
+
+typedef struct yka_kv_config {
+  int32_t n_layers;    /* KV containers (the reference keeps one per full-attention layer, engine35.cpp:303-329) */
+  int32_t n_heads;     /* query heads (24) */
+  int32_t n_kv_heads;  /* KV heads (4); n_heads / n_kv_heads must be 6 */
+  int32_t head_dim;    /* 128 */
+  int32_t max_ctx;     /* tokens reserved per layer; multiple of 256 */
+  int32_t max_rows;    /* most query rows one call may carry (64 = kVerifyMax, engine35.hpp:157; up to 2048 = PM_ for prefill) */
+  int32_t paged;       /* 0: token t of a KV head lives in page t/256; 1: pages go through a per-layer page table */
+  int32_t device;      /* HIP device ordinal */
+} yka_kv_config;
+
+/* replaces the KV reservation of yskn_open (yskn_abi.h:22; engine35.cpp:303-329). NULL on error. */
+YKA_API yka_kv* yka_kv_open(const yka_kv_config* cfg);
+/* replaces yskn_close (yskn_abi.h:23) for the KV containers */
+YKA_API void yka_kv_close(yka_kv* kv);
+/* replaces yskn_last_error (yskn_abi.h:30): thread-local message of the last failed call */
+YKA_API const char* yka_last_error(void);
+/* replaces yskn_build_info (yskn_abi.h:84): "hip=<version>;arch=gfx950;..." */
+YKA_API const char* yka_build_info(void);
+/* replaces yskn_set_opt (yskn_abi.h:87) for the options of this path.
+ * key 1: split count of the narrow kernel (decode, rows of at most 2 tokens); key 2: split count of the wide kernel;
+ * key 3: 1 forces the narrow kernel for every width (cross-check of the wide kernel), 0 = automatic. */
+YKA_API int yka_set_opt(yka_kv* kv, int key, int value);
+
+/* Paged mode: logical page p of `layer` (-1 = every layer) lives in physical page h_table[p]; n_pages = max_ctx/256
+ * entries forming a permutation.  No counterpart in the reference (rows are addressed (kvh*max_ctx+pos)*row_bytes,
+ * q35_atxpk3.cuh:196-200); added for the 256-token shuffled-page configuration. Synchronous. */
+YKA_API int yka_kv_set_page_table(yka_kv* kv, int layer, const int32_t* h_table, int n_pages);
+
+/* Quantize-on-append: rows *d_pos .. *d_pos+M-1 of every KV head of `layer` are overwritten with the int4 codes and
+ * fp16 scales of d_k16 / d_v16 ([M][n_kv_heads][128] fp16, device).  Replaces the KV store of launch_q35_attn_post
+ * followed by launch_tb_requant (q35_kernels.cu:1038,1064,1084-1092; call site engine35.cpp:911-913) and, for the
+ * v1 engine, the K/V part of launch_qkv_post (post_kernels.cu:55-81). */
+YKA_API int yka_append(yka_kv* kv, int layer, const uint16_t* d_k16, const uint16_t* d_v16, int M,
+                       const int* d_pos, void* hip_stream);
+
+/* Attention over the cache: row t of d_q16 ([M][n_heads][128] fp16) attends to keys [0, *d_pos + depth(t) + 1),
+ * depth(t) = d_depth ? d_depth[t] : t (q35_atx.cu:110-118); writes d_out16 [M][n_heads][128] fp16.
+ * Replaces launch_q35_prefill_atx_pk / launch_q35_atx_pk + launch_q35_combine (q35_atxpk.hpp:15-24, q35.hpp:153-156;
+ * call site engine35.cpp:921-934) and launch_attention + launch_attn_combine of the v1 engine (args.hpp:36-37). */
+YKA_API int yka_attend(yka_kv* kv, int layer, const uint16_t* d_q16, int M, const int* d_pos,
+                       const uint8_t* d_depth, uint16_t* d_out16, void* hip_stream);
+
+/* One layer call = yka_append then yka_attend on the same stream: the sequence of Engine35::attn_block
+ * (engine35.cpp:911-934).  M may be as large as max_rows; passes wider than 64 rows are cut into 64-row slices
+ * inside, as attn_block does (engine35.cpp:935-947). */
+YKA_API int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16_t* d_k16,
+                              const uint16_t* d_v16, int M, const int* d_pos, const uint8_t* d_depth,
+                              uint16_t* d_out16, void* hip_stream);
+
+/* ---- hooks with host pointers (model: src/kvx_probe.cu) ---- */
+
+/* Codec round trip on the GPU, replaces yskn_kvx_probe (kvx_probe.cu:22-36): x16 [rows][128] fp16 ->
+ * codes [rows][64], scales [rows][4] fp16, y [rows][128] fp32 dequantized. */
+YKA_API int yka_codec_probe(const uint16_t* x16, int rows, uint8_t* codes, uint16_t* scales, float* y);
+
+/* Canonical image of rows [pos0, pos0+n) of one layer, independent of the physical layout:
+ * kc/vc [n_kv_heads][n][64], ks/vs [n_kv_heads][n][4].  export = device -> host, import = host -> device.
+ * (The reference reads its containers back only inside its hooks, e.g. kvx_probe.cu:369.) Synchronous. */
+YKA_API int yka_kv_export_rows(yka_kv* kv, int layer, int pos0, int n, uint8_t* kc, uint16_t* ks, uint8_t* vc, uint16_t* vs);
+YKA_API int yka_kv_import_rows(yka_kv* kv, int layer, int pos0, int n, const uint8_t* kc, const uint16_t* ks,
+                               const uint8_t* vc, const uint16_t* vs);
+/* dequantize rows on the GPU (decoder probe, replaces tba_unpack_kernel's use in yskn_tbp_pack_unpack,
+ * kvx_probe.cu:123-170): k, v [n_kv_heads][n][128] fp32 */
+YKA_API int yka_kv_dequant_rows(yka_kv* kv, int layer, int pos0, int n, float* k, float* v);
+/* copy the content of layer `src` into every other layer (device to device), as the bench hook tiles one set of
+ * encoded rows over `nlayers` containers (kvx_probe.cu:373-386). Synchronous. */
+YKA_API int yka_kv_replicate_layer(yka_kv* kv, int src);
+
+/* Host-pointer form of one layer call: uploads q/k/v ([M][..][128] fp16; k16/v16 may be NULL = attend only),
+ * sets the device position to `pos`, runs append + attend on an internal stream, downloads out16.
+ * depth may be NULL.  The single-call analogue of the run/combine lambda of yskn_atxpk_bench (kvx_probe.cu:388-401). */
+YKA_API int yka_layer_call_host(yka_kv* kv, int layer, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16,
+                                int M, int pos, const uint8_t* depth, uint16_t* out16);
+
+/* Timed sweeps, replaces yskn_atxpk_bench (kvx_probe.cu:322-449): with q/k/v uploaded once and the device position
+ * fixed at `pos`, runs one warm sweep over all layers and then `reps` timed sweeps (hipEvents on the internal
+ * stream), each sweep = one layer call per layer on distinct containers.  mode 0 = append + attend, 1 = attend only,
+ * 2 = the dominant attention kernel alone (no append, no combine).  ms[r] = time of sweep r in milliseconds.
+ * use_graph != 0 replays the sweep from a captured hipGraph (the reference replays captured passes,
+ * engine35.cpp:1977-1988). */
+YKA_API int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, int pos,
+                           int mode, int use_graph, int reps, float* ms, uint16_t* out16_last);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,89 @@
+/* CPU oracle for the int4-KV GQA attention path.  TEST INFRASTRUCTURE ONLY.
+ *
+ * This library is the checker: tests, the smoke run and the cpu_baseline leg of
+ * the benchmark may call it.  The product (the HIP library) never links, loads
+ * or calls anything declared here.
+ *
+ * Every function is a plain-C restatement of the reference's arithmetic for the
+ * path, adapted to the measured format (24 query heads / 4 KV heads /
+ * head_dim 128, symmetric signed int4 with one fp16 scale per 32-channel
+ * group).  Each cites the reference lines it follows.  Pinning status:
+ *
+ *   yko_h2f / yko_f2h        pinned: exhaustive / dense comparison with numpy float16
+ *   yko_quant_group32        pinned: closed-form properties, ties-to-even cases,
+ *                            exhaustive 1-value groups, independent fp64/numpy
+ *                            restatement on random groups
+ *   yko_dequant_group32      pinned: exact product, all 15 codes x all fp16 scales
+ *   yko_pack / yko_unpack    pinned: all 256 byte values, v1 nibble order
+ *   yko_attend_f32           pinned: fp64 textbook softmax(QK^T/sqrt(d))V (numpy),
+ *                            split-count independence, uniform-V / dominant-key
+ *                            closed forms, window == single rows
+ *   yko_attend_f64           pinned: same closed forms + numpy
+ *   yko_combine              pinned: algebraic identity vs unsplit evaluation,
+ *                            empty-split sentinel
+ *
+ * The reference holds no golden vectors or known-answer tests for this path, so
+ * none are replayed here; the checks above are what the mathematics fixes.
+ */
+#ifndef YKO_H
+#define YKO_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define YKO_GROUP 32 /* channels per scale group */
+
+/* ---- fp16 helpers (reference: src/a8_prologue.cuh:36-38, __float2half_rn / __half2float) ---- */
+float yko_h2f(uint16_t h);
+uint16_t yko_f2h(float f); /* round to nearest even, IEEE overflow to inf, subnormals kept */
+
+/* ---- codec (reference: src/kvq_fast.cuh:194-198, src/kvq_gpu.cuh:85-86, decode src/kvq_attn.cuh:52-54,
+ *      nibble order src/post_kernels.cu:77-80) ----
+ * x16: 32 fp16 bit patterns.  codes: 16 bytes, element 2j in the low nibble of byte j,
+ * element 2j+1 in the high nibble, each stored as q+8 (1..15).  scale16: fp16 bit pattern. */
+void yko_quant_group32(const uint16_t* x16, uint8_t* codes16, uint16_t* scale16);
+void yko_dequant_group32(const uint8_t* codes16, uint16_t scale16, float* y32);
+/* rows of `dim` channels (dim % 32 == 0): codes [rows][dim/2], scales [rows][dim/32] */
+void yko_quant_rows(const uint16_t* x16, int rows, int dim, uint8_t* codes, uint16_t* scales);
+void yko_dequant_rows(const uint8_t* codes, const uint16_t* scales, int rows, int dim, float* y);
+void yko_pack_nibbles(const uint8_t* fields, int n, uint8_t* bytes); /* n even; fields 0..15 */
+void yko_unpack_nibbles(const uint8_t* bytes, int n, uint8_t* fields);
+
+/* ---- canonical cache image used by the oracle and by the export/import hooks of the product ----
+ * One layer: kc/vc [kvh][max_ctx][dim/2] bytes, ks/vs [kvh][max_ctx][dim/32] fp16 bit patterns. */
+typedef struct {
+  int n_heads, n_kv_heads, head_dim, max_ctx;
+  uint8_t* kc; uint16_t* ks; uint8_t* vc; uint16_t* vs;
+} yko_cache;
+
+/* quantize-on-append (reference ordering: src/engine35.cpp:911-913 - rows are written before attention reads them;
+ * row placement src/q35_kernels.cu:1038,1064): k16/v16 [M][kvh][dim] -> rows pos..pos+M-1 */
+void yko_append(yko_cache* c, const uint16_t* k16, const uint16_t* v16, int M, int pos);
+
+/* ---- attention ----
+ * q16 [M][n_heads][dim]; row t of the window sees keys [0, pos + depth(t) + 1) with depth(t) = depth ? depth[t] : t
+ * (reference: src/q35_atx.cu:110-118).  out16 [M][n_heads][dim] fp16.
+ * splits <= 0 selects the reference policy (31 below 4096 keys, else 42: src/q35_atxpk.cu:404-409).
+ * fp32 streaming form follows src/attention_kv4q.cu:19-31,71-146 (online softmax per split, sentinels m=-1e30,l=0)
+ * and the combiner src/attention_kv4q.cu:325-332.  threads <= 1: scalar single thread (the oracle proper);
+ * threads > 1: same loop nest spread over (kv head x split) with OpenMP (the timed CPU baseline). */
+void yko_attend_f32(const yko_cache* c, const uint16_t* q16, int M, int pos, const uint8_t* depth,
+                    int splits, int threads, uint16_t* out16, float* out32 /* optional, pre-rounding */);
+/* textbook two-pass softmax in double on the dequantized tensors; out64 [M][n_heads][dim] */
+void yko_attend_f64(const yko_cache* c, const uint16_t* q16, int M, int pos, const uint8_t* depth, double* out64);
+/* combiner alone: pm,pl [S][rows], pacc [S][rows][dim] -> y [rows][dim] (src/attention_kv4q.cu:325-332) */
+void yko_combine(const float* pm, const float* pl, const float* pacc, int S, int rows, int dim, float* y);
+
+/* ---- seeded synthetic inputs (counter based: value i of stream `seed` does not depend on any other) ---- */
+uint64_t yko_splitmix64(uint64_t x);
+double yko_normal(uint64_t seed, uint64_t i);            /* N(0,1) */
+void yko_outlier_channels(uint64_t seed, int dim, int* ch4); /* 4 distinct channel indices */
+/* fills fp16 bit patterns of N(0,1) * (mult on the 4 outlier channels, 1 elsewhere); n = rows*dim */
+void yko_fill_normal_f16(uint64_t seed, uint64_t first, uint64_t n, int dim, const int* ch4, float mult, uint16_t* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,187 @@
+"""ctypes wrapper of the CPU oracle libyko.so.  TEST INFRASTRUCTURE ONLY.
+
+Only tests, the smoke run and the cpu_baseline leg of the benchmark import this module; the product package
+(yasakani_amd) never does.
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_SO = os.path.join(_HERE, "libyko.so")
+D, GROUP = 128, 32
+NG = D // GROUP
+
+
+def build(force=False):
+    if force:
+        subprocess.run(["make", "-C", _HERE, "clean"], check=True, stdout=subprocess.DEVNULL)
+    p = subprocess.run(["make", "-C", _HERE], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if p.returncode != 0:
+        raise RuntimeError("building libyko.so failed:\n" + p.stdout[-4000:])
+    return _SO
+
+
+class _Cache(C.Structure):
+    _fields_ = [("n_heads", C.c_int), ("n_kv_heads", C.c_int), ("head_dim", C.c_int), ("max_ctx", C.c_int),
+                ("kc", C.c_void_p), ("ks", C.c_void_p), ("vc", C.c_void_p), ("vs", C.c_void_p)]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_SO):
+            build()
+        L = C.CDLL(_SO)
+        vp = C.c_void_p
+        L.yko_h2f.restype = C.c_float; L.yko_h2f.argtypes = [C.c_uint16]
+        L.yko_f2h.restype = C.c_uint16; L.yko_f2h.argtypes = [C.c_float]
+        L.yko_quant_rows.argtypes = [vp, C.c_int, C.c_int, vp, vp]
+        L.yko_dequant_rows.argtypes = [vp, vp, C.c_int, C.c_int, vp]
+        L.yko_pack_nibbles.argtypes = [vp, C.c_int, vp]
+        L.yko_unpack_nibbles.argtypes = [vp, C.c_int, vp]
+        L.yko_append.argtypes = [C.POINTER(_Cache), vp, vp, C.c_int, C.c_int]
+        L.yko_attend_f32.argtypes = [C.POINTER(_Cache), vp, C.c_int, C.c_int, vp, C.c_int, C.c_int, vp, vp]
+        L.yko_attend_f64.argtypes = [C.POINTER(_Cache), vp, C.c_int, C.c_int, vp, vp]
+        L.yko_combine.argtypes = [vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]
+        L.yko_normal.restype = C.c_double; L.yko_normal.argtypes = [C.c_uint64, C.c_uint64]
+        L.yko_splitmix64.restype = C.c_uint64; L.yko_splitmix64.argtypes = [C.c_uint64]
+        L.yko_outlier_channels.argtypes = [C.c_uint64, C.c_int, vp]
+        L.yko_fill_normal_f16.argtypes = [C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, vp, C.c_float, vp]
+        _lib = L
+    return _lib
+
+
+def _p(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _as_u16(a):
+    a = np.ascontiguousarray(a)
+    return a.view(np.uint16) if a.dtype == np.float16 else a.astype(np.uint16, copy=False)
+
+
+def h2f_all():
+    """fp32 value of every fp16 bit pattern (65536 entries)."""
+    L = lib()
+    return np.array([L.yko_h2f(i) for i in range(65536)], np.float32)
+
+
+def f2h(x):
+    L = lib()
+    x = np.asarray(x, np.float32).ravel()
+    return np.array([L.yko_f2h(float(v)) for v in x], np.uint16)
+
+
+def quant_rows(x16, dim=D):
+    """x16 [rows, dim] fp16 -> codes [rows, dim/2] u8, scales [rows, dim/32] u16."""
+    x = _as_u16(x16).reshape(-1, dim)
+    rows = x.shape[0]
+    codes = np.empty((rows, dim // 2), np.uint8)
+    scales = np.empty((rows, dim // GROUP), np.uint16)
+    lib().yko_quant_rows(_p(x), rows, dim, _p(codes), _p(scales))
+    return codes, scales
+
+
+def dequant_rows(codes, scales, dim=D):
+    codes = np.ascontiguousarray(codes, np.uint8).reshape(-1, dim // 2)
+    scales = _as_u16(scales).reshape(-1, dim // GROUP)
+    y = np.empty((codes.shape[0], dim), np.float32)
+    lib().yko_dequant_rows(_p(codes), _p(scales), codes.shape[0], dim, _p(y))
+    return y
+
+
+def pack_nibbles(fields):
+    f = np.ascontiguousarray(fields, np.uint8)
+    out = np.empty(f.size // 2, np.uint8)
+    lib().yko_pack_nibbles(_p(f), f.size, _p(out))
+    return out
+
+
+def unpack_nibbles(bytes_):
+    b = np.ascontiguousarray(bytes_, np.uint8)
+    out = np.empty(b.size * 2, np.uint8)
+    lib().yko_unpack_nibbles(_p(b), b.size * 2, _p(out))
+    return out
+
+
+class Cache:
+    """Canonical cache image of one layer: kc/vc [kvh, max_ctx, 64] u8, ks/vs [kvh, max_ctx, 4] u16."""
+
+    def __init__(self, max_ctx, n_heads=24, n_kv_heads=4, head_dim=D):
+        self.n_heads, self.n_kv_heads, self.head_dim, self.max_ctx = n_heads, n_kv_heads, head_dim, max_ctx
+        self.kc = np.zeros((n_kv_heads, max_ctx, head_dim // 2), np.uint8)
+        self.vc = np.zeros_like(self.kc)
+        self.ks = np.zeros((n_kv_heads, max_ctx, head_dim // GROUP), np.uint16)
+        self.vs = np.zeros_like(self.ks)
+
+    def _c(self):
+        return _Cache(self.n_heads, self.n_kv_heads, self.head_dim, self.max_ctx,
+                      self.kc.ctypes.data, self.ks.ctypes.data, self.vc.ctypes.data, self.vs.ctypes.data)
+
+    def append(self, k16, v16, pos):
+        k = _as_u16(k16); v = _as_u16(v16)
+        M = k.shape[0]
+        assert k.shape == (M, self.n_kv_heads, self.head_dim) and v.shape == k.shape
+        assert pos + M <= self.max_ctx
+        c = self._c()
+        lib().yko_append(C.byref(c), _p(k), _p(v), M, pos)
+
+    def attend_f32(self, q16, pos, depth=None, splits=0, threads=1, want_f32=False):
+        q = _as_u16(q16)
+        M = q.shape[0]
+        assert q.shape == (M, self.n_heads, self.head_dim)
+        dep = None if depth is None else np.ascontiguousarray(depth, np.uint8)
+        out = np.empty(q.shape, np.uint16)
+        o32 = np.empty(q.shape, np.float32) if want_f32 else None
+        c = self._c()
+        lib().yko_attend_f32(C.byref(c), _p(q), M, pos, _p(dep), splits, threads, _p(out), _p(o32))
+        return (out.view(np.float16), o32) if want_f32 else out.view(np.float16)
+
+    def attend_f64(self, q16, pos, depth=None):
+        q = _as_u16(q16)
+        M = q.shape[0]
+        dep = None if depth is None else np.ascontiguousarray(depth, np.uint8)
+        out = np.empty(q.shape, np.float64)
+        c = self._c()
+        lib().yko_attend_f64(C.byref(c), _p(q), M, pos, _p(dep), _p(out))
+        return out
+
+
+def combine(pm, pl, pacc):
+    pm = np.ascontiguousarray(pm, np.float32); pl = np.ascontiguousarray(pl, np.float32)
+    pacc = np.ascontiguousarray(pacc, np.float32)
+    S, rows = pm.shape
+    dim = pacc.shape[-1]
+    y = np.empty((rows, dim), np.float32)
+    lib().yko_combine(_p(pm), _p(pl), _p(pacc), S, rows, dim, _p(y))
+    return y
+
+
+def outlier_channels(seed, dim=D):
+    ch = np.zeros(4, np.int32)
+    lib().yko_outlier_channels(seed, dim, _p(ch))
+    return ch
+
+
+def fill_normal_f16(seed, n_rows, dim=D, outliers=None, mult=8.0, first=0):
+    """fp16 array [n_rows, dim] of N(0,1); channels in `outliers` (4 ints) multiplied by `mult` before rounding."""
+    out = np.empty((n_rows, dim), np.uint16)
+    ch = None if outliers is None else np.ascontiguousarray(outliers, np.int32)
+    lib().yko_fill_normal_f16(seed, first, n_rows * dim, dim, _p(ch), mult, _p(out))
+    return out.view(np.float16)
+
+
+def make_inputs(seed, ctx, M, n_heads=24, n_kv_heads=4, dim=D):
+    """Seeded inputs of the measured configurations: Q [M,NH,D], cached K/V [ctx,KVH,D], new K/V [M,KVH,D], all fp16;
+    K carries 4 fixed outlier channels scaled x8."""
+    ch = outlier_channels(seed, dim)
+    q = fill_normal_f16(seed + 1, M * n_heads, dim).reshape(M, n_heads, dim)
+    k = fill_normal_f16(seed + 2, (ctx + M) * n_kv_heads, dim, ch, 8.0).reshape(ctx + M, n_kv_heads, dim)
+    v = fill_normal_f16(seed + 3, (ctx + M) * n_kv_heads, dim).reshape(ctx + M, n_kv_heads, dim)
+    return q, k[:ctx], v[:ctx], k[ctx:], v[ctx:], ch

@@ -1,0 +1,165 @@
+"""GPU attention through the C ABI vs the oracle: max-abs 2e-3 and relative L2 1e-3 (tests/tolerances.py)."""
+import numpy as np
+import pytest
+
+from tests.tolerances import assert_attn_close, attn_errors
+
+pytestmark = pytest.mark.gpu
+
+
+def _fill(native, oracle, seed, ctx, M, max_ctx=None, **kw):
+    """Cache with `ctx` rows quantized by the oracle and imported, plus seeded q and new k/v for an M-row window."""
+    q, k, v, kn, vn, ch = oracle.make_inputs(seed, ctx, M)
+    max_ctx = max_ctx or ((ctx + M + 255) // 256) * 256
+    oc = oracle.Cache(max_ctx)
+    kv = native.KvCache(max_ctx=max_ctx, **kw)
+    if ctx:
+        oc.append(k, v, 0)
+        kv.import_rows(0, 0, oc.kc[:, :ctx], oc.ks[:, :ctx], oc.vc[:, :ctx], oc.vs[:, :ctx])
+    return kv, oc, q, kn, vn
+
+
+@pytest.mark.parametrize("ctx", [0, 1, 31, 32, 33, 255, 256, 1000, 4096])
+def test_decode_matches_oracle(native, oracle, ctx):
+    kv, oc, q, kn, vn = _fill(native, oracle, 300 + ctx, ctx, 1)
+    with kv:
+        out = kv.layer_call(0, q, kn, vn, ctx)
+        oc.append(kn, vn, ctx)
+        ref16, ref32 = oc.attend_f32(q, ctx, want_f32=True)
+        assert_attn_close(out, ref32, f"decode ctx={ctx} vs fp32")
+        assert_attn_close(out, ref16, f"decode ctx={ctx} vs fp16")
+
+
+@pytest.mark.parametrize("M", [2, 3, 7, 16, 33, 64])
+def test_window_matches_oracle(native, oracle, M):
+    ctx = 1500
+    kv, oc, q, kn, vn = _fill(native, oracle, 400 + M, ctx, M)
+    with kv:
+        out = kv.layer_call(0, q, kn, vn, ctx)
+        oc.append(kn, vn, ctx)
+        ref16, ref32 = oc.attend_f32(q, ctx, threads=8, want_f32=True)
+        assert_attn_close(out, ref32, f"window M={M}")
+        # appended rows are in the cache, bit-exact
+        got = kv.export_rows(0, ctx, M)
+        assert (got[0] == oc.kc[:, ctx:ctx + M]).all() and (got[3] == oc.vs[:, ctx:ctx + M]).all()
+
+
+def test_window_equals_single_row_calls(native, oracle):
+    # reference invariant (src/kvx_probe.cu:425-436): an M-row pass equals M one-row passes
+    ctx, M = 900, 9
+    kv, oc, q, kn, vn = _fill(native, oracle, 500, ctx, M)
+    with kv:
+        full = kv.layer_call(0, q, kn, vn, ctx)
+        for t in range(M):
+            one = kv.layer_call(0, q[t:t + 1], None, None, ctx + t)
+            ma, rl = attn_errors(one, full[t:t + 1])
+            assert ma <= 2e-3 and rl <= 1e-3, (t, ma, rl)
+
+
+def test_split_count_does_not_matter(native, oracle):
+    ctx = 3000
+    kv, oc, q, kn, vn = _fill(native, oracle, 501, ctx, 2)
+    with kv:
+        oc.append(kn, vn, ctx)
+        ref = oc.attend_f32(q, ctx, want_f32=True)[1]
+        outs = []
+        for S in (1, 2, 7, 32, 128):
+            kv.set_opt(1, S)
+            outs.append(kv.layer_call(0, q, kn, vn, ctx))
+            assert_attn_close(outs[-1], ref, f"splits={S}")
+
+
+def test_depth_table(native, oracle):
+    ctx, M = 700, 6
+    kv, oc, q, kn, vn = _fill(native, oracle, 502, ctx, M)
+    depth = np.array([0, 1, 1, 2, 2, 3], np.uint8)
+    with kv:
+        out = kv.layer_call(0, q, kn, vn, ctx, depth=depth)
+        oc.append(kn, vn, ctx)
+        assert_attn_close(out, oc.attend_f32(q, ctx, depth, want_f32=True)[1], "depth table")
+
+
+def test_paged_layout_is_bit_identical_to_contiguous(native, oracle):
+    ctx, M = 2000, 5
+    q, k, v, kn, vn, ch = oracle.make_inputs(503, ctx, M)
+    oc = oracle.Cache(2304); oc.append(k, v, 0)
+    rng = np.random.default_rng(503)
+    outs = []
+    for paged in (False, True):
+        with native.KvCache(max_ctx=2304, paged=paged) as kv:
+            if paged:
+                kv.set_page_table(rng.permutation(9).astype(np.int32))
+            kv.import_rows(0, 0, oc.kc[:, :ctx], oc.ks[:, :ctx], oc.vc[:, :ctx], oc.vs[:, :ctx])
+            outs.append(kv.layer_call(0, q, kn, vn, ctx))
+    assert (outs[0].view(np.uint16) == outs[1].view(np.uint16)).all()
+    oc.append(kn, vn, ctx)
+    assert_attn_close(outs[1], oc.attend_f32(q, ctx, want_f32=True)[1], "paged")
+
+
+def test_uniform_v_and_dominant_key(native, oracle):
+    ctx = 1200
+    kv, oc, q, kn, vn = _fill(native, oracle, 504, ctx, 1)
+    with kv:
+        vc = np.repeat(oc.vc[:, :1], ctx, axis=1); vs = np.repeat(oc.vs[:, :1], ctx, axis=1)
+        kv.import_rows(0, 0, oc.kc[:, :ctx], oc.ks[:, :ctx], vc, vs)
+        out = kv.layer_call(0, q, None, None, ctx - 1).astype(np.float32)
+        vrow = np.repeat(oracle.dequant_rows(oc.vc[:, 0], oc.vs[:, 0]), 6, axis=0)
+        assert np.abs(out[0] - vrow).max() <= 2e-3 * max(1.0, np.abs(vrow).max())
+
+
+def test_multi_layer_containers_are_independent(native, oracle):
+    ctx = 400
+    q, k, v, kn, vn, ch = oracle.make_inputs(505, ctx, 1)
+    q2, k2, v2, kn2, vn2, _ = oracle.make_inputs(506, ctx, 1)
+    with native.KvCache(n_layers=3, max_ctx=512) as kv:
+        oa, ob = oracle.Cache(512), oracle.Cache(512)
+        oa.append(k, v, 0); ob.append(k2, v2, 0)
+        kv.import_rows(0, 0, oa.kc[:, :ctx], oa.ks[:, :ctx], oa.vc[:, :ctx], oa.vs[:, :ctx])
+        kv.import_rows(2, 0, ob.kc[:, :ctx], ob.ks[:, :ctx], ob.vc[:, :ctx], ob.vs[:, :ctx])
+        o0 = kv.layer_call(0, q, kn, vn, ctx); o2 = kv.layer_call(2, q, kn, vn, ctx)
+        oa.append(kn, vn, ctx); ob.append(kn, vn, ctx)
+        assert_attn_close(o0, oa.attend_f32(q, ctx, want_f32=True)[1], "layer 0")
+        assert_attn_close(o2, ob.attend_f32(q, ctx, want_f32=True)[1], "layer 2")
+        kv.replicate_layer(0)
+        o2b = kv.layer_call(2, q, None, None, ctx)
+        assert (o2b.view(np.uint16) == o0.view(np.uint16)).all()
+
+
+def test_wide_pass_is_cut_into_slices(native, oracle):
+    # passes wider than 64 rows are cut into 64-row slices (src/engine35.cpp:935-947)
+    ctx, M = 300, 150
+    kv, oc, q, kn, vn = _fill(native, oracle, 507, ctx, M, max_rows=256)
+    with kv:
+        out = kv.layer_call(0, q, kn, vn, ctx)
+        oc.append(kn, vn, ctx)
+        assert_attn_close(out, oc.attend_f32(q, ctx, threads=8, want_f32=True)[1], "150-row pass")
+
+
+def test_errors_are_reported_not_thrown(native):
+    with native.KvCache(max_ctx=256, max_rows=4) as kv:
+        q = np.zeros((5, 24, 128), np.float16)
+        with pytest.raises(native.YkaError, match="max_rows"):
+            kv.layer_call(0, q, None, None, 0)
+        with pytest.raises(native.YkaError, match="layer"):
+            kv.layer_call(3, q[:1], None, None, 0)
+        with pytest.raises(native.YkaError, match="max_ctx"):
+            kv.layer_call(0, q[:4], None, None, 254)
+        with pytest.raises(native.YkaError, match="contiguous"):
+            kv.set_page_table(np.zeros(1, np.int32))
+    with native.KvCache(max_ctx=512, paged=True) as kv:
+        with pytest.raises(native.YkaError, match="permutation"):
+            kv.set_page_table(np.array([0, 0], np.int32))
+
+
+def test_bench_hook_runs_and_agrees_with_single_call(native, oracle):
+    ctx = 2048
+    q, k, v, kn, vn, ch = oracle.make_inputs(508, ctx, 1)
+    with native.KvCache(n_layers=4, max_ctx=2304) as kv:
+        oc = oracle.Cache(2304); oc.append(k, v, 0)
+        kv.import_rows(0, 0, oc.kc[:, :ctx], oc.ks[:, :ctx], oc.vc[:, :ctx], oc.vs[:, :ctx])
+        kv.replicate_layer(0)
+        one = kv.layer_call(3, q, kn, vn, ctx)
+        for graph in (False, True):
+            ms, out = kv.bench(q, kn, vn, ctx, mode=0, use_graph=graph, reps=3)
+            assert (ms > 0).all()
+            assert (out.view(np.uint16) == one.view(np.uint16)).all()

@@ -1,0 +1,379 @@
+// C ABI of libyka.so: handle, validation, launch sequencing, host-pointer hooks.
+// Error convention of the reference's C layer (src/c_api.cpp:17,33,49): catch everything, keep a thread-local
+// message, return -1.
+#include "../../include/yka_abi.h"
+#include "yka_internal.h"
+#include <algorithm>
+#include <cstdio>
+#include <cstring>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+using namespace yka;
+
+static thread_local std::string g_err;
+
+#define HIPCHK(expr)                                                                                  \
+  do {                                                                                                \
+    hipError_t rc_ = (expr);                                                                          \
+    if (rc_ != hipSuccess) throw std::runtime_error(std::string(#expr) + ": " + hipGetErrorString(rc_)); \
+  } while (0)
+
+struct yka_kv {
+  yka_kv_config cfg{};
+  int n_pages = 0;
+  size_t layer_bytes = 0;
+  uint8_t* pool = nullptr;
+  int32_t* tables = nullptr;       // [n_layers][n_pages], paged mode only
+  float *pm = nullptr, *pl = nullptr, *pacc = nullptr;
+  size_t ws_rows = 0;              // capacity of the partial workspace in (token, split) pairs
+  int* d_pos = nullptr;            // position used by the host-pointer hooks
+  hipStream_t stream = nullptr;    // stream of the host-pointer hooks
+  int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0;
+  KvView view(int layer) const {
+    return KvView{pool + (size_t)layer * layer_bytes, tables ? tables + (size_t)layer * n_pages : nullptr, cfg.n_kv_heads, cfg.max_ctx};
+  }
+};
+
+namespace {
+
+struct DevBuf {  // device buffer that frees itself (hooks only; the launch path never allocates)
+  void* p = nullptr;
+  explicit DevBuf(size_t n) { HIPCHK(hipMalloc(&p, n ? n : 1)); }
+  ~DevBuf() { if (p) (void)hipFree(p); }
+  DevBuf(const DevBuf&) = delete;
+  DevBuf& operator=(const DevBuf&) = delete;
+  template <class T> T* as() const { return static_cast<T*>(p); }
+};
+
+void on_device(const yka_kv* kv) {
+  if (!kv) throw std::runtime_error("null handle");
+  HIPCHK(hipSetDevice(kv->cfg.device));
+}
+
+constexpr int kMaxSplits = 128;
+constexpr size_t kWsPairs = 512;  // (token, split) pairs the partial workspace holds: 512 * 24 * 130 floats = 6.4 MB
+
+// splits for the narrow kernel: enough workgroups (n_kv * S * ceil(M/2)) to cover 256 CUs about twice over
+int narrow_splits(const yka_kv* kv, int M) {
+  if (kv->opt_splits_narrow > 0) return std::min(kv->opt_splits_narrow, (int)(kWsPairs / (size_t)M));
+  const int tiles = (M + 1) / 2;
+  int S = 512 / (kv->cfg.n_kv_heads * tiles);
+  S = std::max(2, std::min(kMaxSplits, S));
+  return std::min(S, (int)(kWsPairs / (size_t)M));
+}
+
+void check_layer(const yka_kv* kv, int layer) {
+  if (layer < 0 || layer >= kv->cfg.n_layers) throw std::runtime_error("layer out of range");
+}
+void check_rows(const yka_kv* kv, int M) {
+  if (M < 1 || M > kv->cfg.max_rows) throw std::runtime_error("M must be in [1, max_rows]");
+}
+
+void do_append(yka_kv* kv, int layer, const uint16_t* k16, const uint16_t* v16, int M, const int* d_pos, hipStream_t st) {
+  launch_append(AppendArgs{kv->view(layer), k16, v16, d_pos, M}, st);
+}
+
+// mode 0: attention + combine; 2: attention kernel alone
+void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_pos, const uint8_t* depth, uint16_t* out16,
+               hipStream_t st, int mode = 0) {
+  const int NH = kv->cfg.n_heads;
+  for (int s0 = 0; s0 < M; s0 += kMaxSlice) {   // 64-row slices, as attn_block cuts wide passes (engine35.cpp:935-947)
+    const int Ms = std::min(kMaxSlice, M - s0);
+    const int S = narrow_splits(kv, Ms);
+    AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * kD, d_pos, depth, Ms, s0, NH, S, kv->pm, kv->pl, kv->pacc};
+    if (Ms <= 2 || kv->opt_force_narrow) launch_attend_narrow(A, st); else launch_attend_wide(A, st);
+    if (mode != 2) launch_combine(CombineArgs{kv->pm, kv->pl, kv->pacc, S, Ms, NH, out16 + (size_t)s0 * NH * kD}, st);
+  }
+}
+
+}  // namespace
+
+#define YKA_TRY try {
+#define YKA_CATCH_INT                                                   \
+  return 0; }                                                           \
+  catch (const std::exception& e) { g_err = e.what(); return -1; }      \
+  catch (...) { g_err = "unknown error"; return -1; }
+
+extern "C" {
+
+const char* yka_last_error(void) { return g_err.c_str(); }
+
+const char* yka_build_info(void) {
+  static const std::string s = [] {
+    char b[128];
+    snprintf(b, sizeof b, "hip=%d;arch=gfx950;page_bytes=%d;page_tokens=%d", HIP_VERSION, kPageBytes, kPageTok);
+    return std::string(b);
+  }();
+  return s.c_str();
+}
+
+yka_kv* yka_kv_open(const yka_kv_config* cfg) {
+  yka_kv* kv = nullptr;
+  try {
+    if (!cfg) throw std::runtime_error("null config");
+    if (cfg->head_dim != kD) throw std::runtime_error("head_dim must be 128");
+    if (cfg->n_kv_heads < 1 || cfg->n_heads != cfg->n_kv_heads * kG) throw std::runtime_error("n_heads must be 6 * n_kv_heads");
+    if (cfg->n_layers < 1) throw std::runtime_error("n_layers must be >= 1");
+    if (cfg->max_ctx < kPageTok || cfg->max_ctx % kPageTok) throw std::runtime_error("max_ctx must be a positive multiple of 256");
+    if (cfg->max_rows < 1 || cfg->max_rows > 8192) throw std::runtime_error("max_rows must be in [1, 8192]");
+    int ndev = 0;
+    HIPCHK(hipGetDeviceCount(&ndev));
+    if (cfg->device < 0 || cfg->device >= ndev) throw std::runtime_error("device out of range");
+    HIPCHK(hipSetDevice(cfg->device));
+    kv = new yka_kv();
+    kv->cfg = *cfg;
+    kv->n_pages = cfg->max_ctx / kPageTok;
+    kv->layer_bytes = (size_t)kv->n_pages * kv_page_bytes(cfg->n_kv_heads);
+    HIPCHK(hipMalloc((void**)&kv->pool, kv->layer_bytes * cfg->n_layers));
+    HIPCHK(hipMemset(kv->pool, 0, kv->layer_bytes * cfg->n_layers));   // zero scales: unwritten rows decode to finite values
+    if (cfg->paged) {
+      std::vector<int32_t> ident((size_t)cfg->n_layers * kv->n_pages);
+      for (size_t i = 0; i < ident.size(); ++i) ident[i] = (int32_t)(i % kv->n_pages);
+      HIPCHK(hipMalloc((void**)&kv->tables, ident.size() * 4));
+      HIPCHK(hipMemcpy(kv->tables, ident.data(), ident.size() * 4, hipMemcpyHostToDevice));
+    }
+    kv->ws_rows = kWsPairs;
+    const size_t np = kv->ws_rows * cfg->n_heads;
+    HIPCHK(hipMalloc((void**)&kv->pm, np * 4));
+    HIPCHK(hipMalloc((void**)&kv->pl, np * 4));
+    HIPCHK(hipMalloc((void**)&kv->pacc, np * kD * 4));
+    HIPCHK(hipMalloc((void**)&kv->d_pos, 4));
+    HIPCHK(hipMemset(kv->d_pos, 0, 4));
+    HIPCHK(hipStreamCreateWithFlags(&kv->stream, hipStreamNonBlocking));
+    HIPCHK(hipDeviceSynchronize());
+    return kv;
+  } catch (const std::exception& e) {
+    g_err = e.what();
+  } catch (...) { g_err = "unknown error"; }
+  if (kv) yka_kv_close(kv);
+  return nullptr;
+}
+
+void yka_kv_close(yka_kv* kv) {
+  if (!kv) return;
+  (void)hipSetDevice(kv->cfg.device);
+  (void)hipDeviceSynchronize();
+  if (kv->stream) (void)hipStreamDestroy(kv->stream);
+  (void)hipFree(kv->pool); (void)hipFree(kv->tables); (void)hipFree(kv->pm); (void)hipFree(kv->pl); (void)hipFree(kv->pacc); (void)hipFree(kv->d_pos);
+  delete kv;
+}
+
+int yka_set_opt(yka_kv* kv, int key, int value) {
+  YKA_TRY
+  if (!kv) throw std::runtime_error("null handle");
+  switch (key) {
+    case 1: if (value < 0 || value > kMaxSplits) throw std::runtime_error("splits must be in [0, 128]"); kv->opt_splits_narrow = value; break;
+    case 2: if (value < 0 || value > kMaxSplits) throw std::runtime_error("splits must be in [0, 128]"); kv->opt_splits_wide = value; break;
+    case 3: kv->opt_force_narrow = value != 0; break;
+    default: throw std::runtime_error("unknown option key");
+  }
+  YKA_CATCH_INT
+}
+
+int yka_kv_set_page_table(yka_kv* kv, int layer, const int32_t* h_table, int n_pages) {
+  YKA_TRY
+  on_device(kv);
+  if (!kv->cfg.paged) throw std::runtime_error("handle was opened in contiguous mode");
+  if (!h_table || n_pages != kv->n_pages) throw std::runtime_error("page table must have max_ctx/256 entries");
+  if (layer < -1 || layer >= kv->cfg.n_layers) throw std::runtime_error("layer out of range");
+  std::vector<char> seen((size_t)n_pages, 0);
+  for (int p = 0; p < n_pages; ++p) {
+    if (h_table[p] < 0 || h_table[p] >= n_pages || seen[(size_t)h_table[p]]) throw std::runtime_error("page table is not a permutation");
+    seen[(size_t)h_table[p]] = 1;
+  }
+  HIPCHK(hipDeviceSynchronize());
+  for (int l = 0; l < kv->cfg.n_layers; ++l)
+    if (layer < 0 || l == layer) HIPCHK(hipMemcpy(kv->tables + (size_t)l * n_pages, h_table, (size_t)n_pages * 4, hipMemcpyHostToDevice));
+  YKA_CATCH_INT
+}
+
+int yka_append(yka_kv* kv, int layer, const uint16_t* d_k16, const uint16_t* d_v16, int M, const int* d_pos, void* hip_stream) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); check_rows(kv, M);
+  if (!d_k16 || !d_v16 || !d_pos) throw std::runtime_error("null pointer");
+  do_append(kv, layer, d_k16, d_v16, M, d_pos, (hipStream_t)hip_stream);
+  HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_attend(yka_kv* kv, int layer, const uint16_t* d_q16, int M, const int* d_pos, const uint8_t* d_depth,
+               uint16_t* d_out16, void* hip_stream) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); check_rows(kv, M);
+  if (!d_q16 || !d_pos || !d_out16) throw std::runtime_error("null pointer");
+  do_attend(kv, layer, d_q16, M, d_pos, d_depth, d_out16, (hipStream_t)hip_stream);
+  HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16_t* d_k16, const uint16_t* d_v16, int M,
+                      const int* d_pos, const uint8_t* d_depth, uint16_t* d_out16, void* hip_stream) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); check_rows(kv, M);
+  if (!d_q16 || !d_k16 || !d_v16 || !d_pos || !d_out16) throw std::runtime_error("null pointer");
+  do_append(kv, layer, d_k16, d_v16, M, d_pos, (hipStream_t)hip_stream);
+  do_attend(kv, layer, d_q16, M, d_pos, d_depth, d_out16, (hipStream_t)hip_stream);
+  HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_codec_probe(const uint16_t* x16, int rows, uint8_t* codes, uint16_t* scales, float* y) {
+  YKA_TRY
+  if (!x16 || !codes || !scales || !y || rows < 1) throw std::runtime_error("bad argument");
+  const size_t n = (size_t)rows * kD;
+  DevBuf dx(n * 2), dc(n / 2), ds((size_t)rows * kNG * 2), dy(n * 4);
+  HIPCHK(hipMemcpy(dx.p, x16, n * 2, hipMemcpyHostToDevice));
+  launch_codec_probe(dx.as<uint16_t>(), rows, dc.as<uint8_t>(), ds.as<uint16_t>(), dy.as<float>(), nullptr);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipDeviceSynchronize());
+  HIPCHK(hipMemcpy(codes, dc.p, n / 2, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(scales, ds.p, (size_t)rows * kNG * 2, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(y, dy.p, n * 4, hipMemcpyDeviceToHost));
+  YKA_CATCH_INT
+}
+
+static void check_range(const yka_kv* kv, int pos0, int n) {
+  if (pos0 < 0 || n < 1 || (long long)pos0 + n > kv->cfg.max_ctx) throw std::runtime_error("row range outside the container");
+}
+
+int yka_kv_export_rows(yka_kv* kv, int layer, int pos0, int n, uint8_t* kc, uint16_t* ks, uint8_t* vc, uint16_t* vs) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); check_range(kv, pos0, n);
+  if (!kc || !ks || !vc || !vs) throw std::runtime_error("null pointer");
+  const size_t rows = (size_t)kv->cfg.n_kv_heads * n;
+  DevBuf dkc(rows * 64), dvc(rows * 64), dks(rows * kNG * 2), dvs(rows * kNG * 2);
+  HIPCHK(hipDeviceSynchronize());
+  launch_export_rows(kv->view(layer), pos0, n, dkc.as<uint8_t>(), dks.as<uint16_t>(), dvc.as<uint8_t>(), dvs.as<uint16_t>(), nullptr);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipDeviceSynchronize());
+  HIPCHK(hipMemcpy(kc, dkc.p, rows * 64, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(vc, dvc.p, rows * 64, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(ks, dks.p, rows * kNG * 2, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(vs, dvs.p, rows * kNG * 2, hipMemcpyDeviceToHost));
+  YKA_CATCH_INT
+}
+
+int yka_kv_import_rows(yka_kv* kv, int layer, int pos0, int n, const uint8_t* kc, const uint16_t* ks, const uint8_t* vc, const uint16_t* vs) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); check_range(kv, pos0, n);
+  if (!kc || !ks || !vc || !vs) throw std::runtime_error("null pointer");
+  const size_t rows = (size_t)kv->cfg.n_kv_heads * n;
+  DevBuf dkc(rows * 64), dvc(rows * 64), dks(rows * kNG * 2), dvs(rows * kNG * 2);
+  HIPCHK(hipMemcpy(dkc.p, kc, rows * 64, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dvc.p, vc, rows * 64, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dks.p, ks, rows * kNG * 2, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dvs.p, vs, rows * kNG * 2, hipMemcpyHostToDevice));
+  HIPCHK(hipDeviceSynchronize());
+  launch_import_rows(kv->view(layer), pos0, n, dkc.as<uint8_t>(), dks.as<uint16_t>(), dvc.as<uint8_t>(), dvs.as<uint16_t>(), nullptr);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipDeviceSynchronize());
+  YKA_CATCH_INT
+}
+
+int yka_kv_dequant_rows(yka_kv* kv, int layer, int pos0, int n, float* k, float* v) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); check_range(kv, pos0, n);
+  if (!k || !v) throw std::runtime_error("null pointer");
+  const size_t ne = (size_t)kv->cfg.n_kv_heads * n * kD;
+  DevBuf dk(ne * 4), dv(ne * 4);
+  HIPCHK(hipDeviceSynchronize());
+  launch_dequant_rows(kv->view(layer), pos0, n, dk.as<float>(), dv.as<float>(), nullptr);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipDeviceSynchronize());
+  HIPCHK(hipMemcpy(k, dk.p, ne * 4, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(v, dv.p, ne * 4, hipMemcpyDeviceToHost));
+  YKA_CATCH_INT
+}
+
+int yka_kv_replicate_layer(yka_kv* kv, int src) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, src);
+  HIPCHK(hipDeviceSynchronize());
+  for (int l = 0; l < kv->cfg.n_layers; ++l) {
+    if (l == src) continue;
+    HIPCHK(hipMemcpy(kv->pool + (size_t)l * kv->layer_bytes, kv->pool + (size_t)src * kv->layer_bytes, kv->layer_bytes, hipMemcpyDeviceToDevice));
+    if (kv->tables) HIPCHK(hipMemcpy(kv->tables + (size_t)l * kv->n_pages, kv->tables + (size_t)src * kv->n_pages, (size_t)kv->n_pages * 4, hipMemcpyDeviceToDevice));
+  }
+  HIPCHK(hipDeviceSynchronize());
+  YKA_CATCH_INT
+}
+
+int yka_layer_call_host(yka_kv* kv, int layer, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, int pos,
+                        const uint8_t* depth, uint16_t* out16) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); check_rows(kv, M);
+  if (!q16 || !out16 || ((k16 == nullptr) != (v16 == nullptr))) throw std::runtime_error("bad pointer arguments");
+  if (pos < 0 || (long long)pos + M > kv->cfg.max_ctx) throw std::runtime_error("pos + M exceeds max_ctx");
+  const size_t nq = (size_t)M * kv->cfg.n_heads * kD, nk = (size_t)M * kv->cfg.n_kv_heads * kD;
+  DevBuf dq(nq * 2), dk(nk * 2), dv(nk * 2), dout(nq * 2), dd((size_t)M);
+  hipStream_t st = kv->stream;
+  HIPCHK(hipMemcpy(dq.p, q16, nq * 2, hipMemcpyHostToDevice));
+  if (k16) { HIPCHK(hipMemcpy(dk.p, k16, nk * 2, hipMemcpyHostToDevice)); HIPCHK(hipMemcpy(dv.p, v16, nk * 2, hipMemcpyHostToDevice)); }
+  if (depth) HIPCHK(hipMemcpy(dd.p, depth, (size_t)M, hipMemcpyHostToDevice));
+  HIPCHK(hipDeviceSynchronize());
+  launch_set_int(kv->d_pos, pos, st);
+  if (k16) do_append(kv, layer, dk.as<uint16_t>(), dv.as<uint16_t>(), M, kv->d_pos, st);
+  do_attend(kv, layer, dq.as<uint16_t>(), M, kv->d_pos, depth ? dd.as<uint8_t>() : nullptr, dout.as<uint16_t>(), st);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipStreamSynchronize(st));
+  HIPCHK(hipMemcpy(out16, dout.p, nq * 2, hipMemcpyDeviceToHost));
+  YKA_CATCH_INT
+}
+
+int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, int pos, int mode,
+                   int use_graph, int reps, float* ms, uint16_t* out16_last) {
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  hipGraph_t graph = nullptr; hipGraphExec_t gexec = nullptr;
+  int rc = 0;
+  try {
+    on_device(kv); check_rows(kv, M);
+    if (!q16 || !ms || reps < 1 || mode < 0 || mode > 2) throw std::runtime_error("bad argument");
+    if (mode == 0 && (!k16 || !v16)) throw std::runtime_error("mode 0 needs k16 and v16");
+    if (pos < 0 || (long long)pos + M > kv->cfg.max_ctx) throw std::runtime_error("pos + M exceeds max_ctx");
+    const size_t nq = (size_t)M * kv->cfg.n_heads * kD, nk = (size_t)M * kv->cfg.n_kv_heads * kD;
+    DevBuf dq(nq * 2), dk(nk * 2), dv(nk * 2), dout(nq * 2);
+    hipStream_t st = kv->stream;
+    HIPCHK(hipMemcpy(dq.p, q16, nq * 2, hipMemcpyHostToDevice));
+    if (k16) { HIPCHK(hipMemcpy(dk.p, k16, nk * 2, hipMemcpyHostToDevice)); HIPCHK(hipMemcpy(dv.p, v16, nk * 2, hipMemcpyHostToDevice)); }
+    HIPCHK(hipMemset(dout.p, 0, nq * 2));
+    HIPCHK(hipDeviceSynchronize());
+    launch_set_int(kv->d_pos, pos, st);
+    auto sweep = [&]() {
+      for (int l = 0; l < kv->cfg.n_layers; ++l) {
+        if (mode == 0) do_append(kv, l, dk.as<uint16_t>(), dv.as<uint16_t>(), M, kv->d_pos, st);
+        do_attend(kv, l, dq.as<uint16_t>(), M, kv->d_pos, nullptr, dout.as<uint16_t>(), st, mode == 2 ? 2 : 0);
+      }
+    };
+    if (use_graph) {
+      HIPCHK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+      sweep();
+      HIPCHK(hipStreamEndCapture(st, &graph));
+      HIPCHK(hipGraphInstantiate(&gexec, graph, nullptr, nullptr, 0));
+    }
+    auto run = [&]() { if (use_graph) HIPCHK(hipGraphLaunch(gexec, st)); else sweep(); };
+    HIPCHK(hipEventCreate(&e0));
+    HIPCHK(hipEventCreate(&e1));
+    run();                                       // warm sweep
+    HIPCHK(hipGetLastError());
+    HIPCHK(hipStreamSynchronize(st));
+    for (int r = 0; r < reps; ++r) {
+      HIPCHK(hipEventRecord(e0, st));
+      run();
+      HIPCHK(hipEventRecord(e1, st));
+      HIPCHK(hipEventSynchronize(e1));
+      HIPCHK(hipEventElapsedTime(&ms[r], e0, e1));
+    }
+    HIPCHK(hipGetLastError());
+    if (out16_last) HIPCHK(hipMemcpy(out16_last, dout.p, nq * 2, hipMemcpyDeviceToHost));
+  } catch (const std::exception& e) { g_err = e.what(); rc = -1; }
+  catch (...) { g_err = "unknown error"; rc = -1; }
+  if (gexec) (void)hipGraphExecDestroy(gexec);
+  if (graph) (void)hipGraphDestroy(graph);
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  return rc;
+}
+
+}  // extern "C"

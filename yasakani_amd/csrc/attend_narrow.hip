@@ -1,0 +1,226 @@
+// Split-KV attention over the int4 cache for row tiles of at most 2 tokens x 6 heads (single-token decode and the
+// building block for any window), plus the split combiner.  gfx950 (wave64, MFMA 16x16x32 f16).
+//
+// What it computes is the reference's split-KV pass (src/attention_kv4q.cu:71-146, production form
+// src/q35_atxpk3.cuh:131-477): for every query row, an online softmax over the keys of one split, written as
+// (m, l, acc) partials, merged by a combiner (src/attention_kv4q.cu:325-332).  How it computes it is specific to
+// CDNA4:
+//   * one wave owns a 32-key tile.  K rows are read as one 16-byte chunk per lane; the page layout puts one dword of
+//     every scale group into that chunk, so MFMA step m contracts exactly the 32 channels of group m.  V is read as
+//     one dword per (lane, token) so that a lane ends up with 8 tokens of the same 8 channels - the operand shape
+//     the token-contracting MFMA needs;
+//   * codes become fp16 without integer conversion: a nibble OR-ed into the mantissa of 1024.0 is 1024+n (or
+//     1024+16n for the odd nibble of a byte); subtracting 1032 (1152) gives n-8 (16(n-8)) exactly;
+//   * K stays exact: the MFMA multiplies Q by the integer codes, and the fp16 group scale is applied to the fp32
+//     partial sum of each group (rounding q*scale to fp16 first costs 7e-4 relative L2 on inputs with outlier
+//     channels, most of the 1e-3 budget).  V is scaled in fp16 (one rounding, 2e-4);
+//   * scores S^T = K Q^T come out of the MFMA with one query row per lane column, which is already the B-operand
+//     layout of O^T += V^T P^T: probabilities never move between lanes;
+//   * running maxima are shared by the 4 lane groups of a row through two cross-lane exchanges per tile.
+#include "yka_internal.h"
+#include <hip/hip_fp16.h>
+
+namespace yka {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ h2 as_h2(uint32_t u) { return __builtin_bit_cast(h2, u); }
+__device__ __forceinline__ uint32_t as_u32(h2 h) { return __builtin_bit_cast(uint32_t, h); }
+
+constexpr uint32_t kMagic = 0x64006400u;  // two fp16 1024.0
+constexpr float kLog2e = 1.4426950408889634f;
+
+// 8 codes of one dword -> 4 half2 in element order [n0,n4 | n1,n5 | n2,n6 | n3,n7] holding n-8 for even nibbles and
+// 16(n-8) for odd ones, all exact.  The factor 16 is undone by the query fragment.
+__device__ __forceinline__ void dq_dword_int(uint32_t w, h2* out) {
+  const h2 c1032 = {(_Float16)1032.f, (_Float16)1032.f}, c1152 = {(_Float16)1152.f, (_Float16)1152.f};
+  const uint32_t t = w >> 8;
+  out[0] = as_h2((w & 0x000f000fu) | kMagic) - c1032;
+  out[1] = as_h2((w & 0x00f000f0u) | kMagic) - c1152;
+  out[2] = as_h2((t & 0x000f000fu) | kMagic) - c1032;
+  out[3] = as_h2((t & 0x00f000f0u) | kMagic) - c1152;
+}
+
+struct RawTile {       // what one lane holds of a 32-key tile before dequantization
+  uint4 kw[2];         // K codes: key 16*kt + (lane&15), dword m = channels 32m + 8*(lane>>4) .. +7
+  uint4 ks[2][2];      // K scales of the 4 keys whose scores this lane receives: [kt][..] = keys 16kt+4g+r, 4 fp16 each
+  uint32_t vw[8];      // V codes: token tau(e), channels 8*(lane&15) .. +7
+  uint2 vs[2];         // V scales, group (lane&15)/4, tokens 16h+4g .. +3 (4 fp16)
+};
+// token slot e of lane group g inside a 32-key tile: the keys whose scores this lane receives from the two score MFMAs
+__device__ __forceinline__ int tau(int g, int e) { return 16 * (e >> 2) + 4 * g + (e & 3); }
+
+// pg = start of the (page, kv head) block, tp = index of the tile's first token inside the page
+__device__ __forceinline__ void load_tile(const uint8_t* pg, int tp, int i, int g, RawTile& R) {
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt) {
+    R.kw[kt] = *reinterpret_cast<const uint4*>(pg + kPageKc + (size_t)(tp + 16 * kt + i) * 64 + 16 * g);
+    const uint4* sp = reinterpret_cast<const uint4*>(pg + kPageKs + (size_t)(tp + 16 * kt + 4 * g) * 8);
+    R.ks[kt][0] = sp[0]; R.ks[kt][1] = sp[1];
+    R.vs[kt] = *reinterpret_cast<const uint2*>(pg + kPageVs + ((size_t)(i >> 2) * kPageTok + tp + 16 * kt + 4 * g) * 2);
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e)
+    R.vw[e] = *reinterpret_cast<const uint32_t*>(pg + kPageVc + (size_t)(tp + tau(g, e)) * 64 + 4 * i);
+}
+
+// grid (S, n_kv, ceil(M/2)), block 256 (4 waves).  Workgroup = (split, kv head, row tile of 2 tokens x 6 heads).
+__global__ void __launch_bounds__(256) attend_narrow_kernel(AttnArgs A) {
+  __shared__ float s_m[4][16], s_l[4][16];
+  __shared__ float s_acc[4][16][kD + 4];
+  const int split = blockIdx.x, kvh = blockIdx.y, rt = blockIdx.z;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
+  const int pos = *A.d_pos;
+
+  // query row of this lane column: j = i -> (token 2*rt + i/6, head kvh*6 + i%6); columns 12..15 are padding
+  const int tl = 2 * rt + i / kG;                  // token index inside the slice
+  const bool vrow = i < 2 * kG && tl < A.M;
+  const int head = kvh * kG + i % kG;
+  int len = 0;
+  if (vrow) { const int tg = A.tok0 + tl; len = pos + (A.depth ? (int)A.depth[tg] : tg) + 1; len = min(len, A.kv.max_ctx); }
+  int maxlen = len;
+#pragma unroll
+  for (int o = 1; o < 16; o <<= 1) maxlen = max(maxlen, __shfl_xor(maxlen, o, 64));
+  const int ntiles = (maxlen + 31) >> 5, tps = (ntiles + A.S - 1) / A.S;
+  const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
+
+  // Q fragments: B operand of S^T = K Q^T.  MFMA step m (= scale group m), lane (row i, lane group g), element e
+  // <-> channel 32m + 8g + pi(e), pi = [0,4,1,5,2,6,3,7] (the order dq_dword_int produces); odd channels carry 1/16.
+  h8 qf[4];
+  {
+    const uint16_t* qrow = A.q16 + ((size_t)tl * A.n_heads + head) * kD + 8 * g;
+    const _Float16 sx = (_Float16)0.0625f;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      uint4 u = vrow ? *reinterpret_cast<const uint4*>(qrow + 32 * m) : make_uint4(0, 0, 0, 0);
+      const h8 c = __builtin_bit_cast(h8, u);
+      qf[m] = h8{c[0], c[4], c[1] * sx, c[5] * sx, c[2], c[6], c[3] * sx, c[7] * sx};
+    }
+  }
+  const float sc_log2 = kLog2e / sqrtf((float)kD);
+
+  float m_run = -1e30f, l_run = 0.f;
+  f4 o[8];
+#pragma unroll
+  for (int b = 0; b < 8; ++b) o[b] = f4{0.f, 0.f, 0.f, 0.f};
+
+  RawTile cur, nxt;
+  int T = tile0 + wave;
+  if (T < tile1) load_tile(kv_page(A.kv, kvh, T << 5), (T << 5) % kPageTok, i, g, cur);
+  for (; T < tile1; T += 4) {
+    if (T + 4 < tile1) load_tile(kv_page(A.kv, kvh, (T + 4) << 5), ((T + 4) << 5) % kPageTok, i, g, nxt);
+    const int t0 = T << 5;
+    // ---- scores: two 16-key MFMA tiles; step m contracts scale group m, its fp32 sum is scaled afterwards ----
+    float s[8];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      const uint32_t w[4] = {cur.kw[kt].x, cur.kw[kt].y, cur.kw[kt].z, cur.kw[kt].w};
+      f4 part[4];
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        h2 k4[4];
+        dq_dword_int(w[m], k4);
+        const h8 kf = h8{k4[0][0], k4[0][1], k4[1][0], k4[1][1], k4[2][0], k4[2][1], k4[3][0], k4[3][1]};
+        part[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[m], f4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+      }
+      // part[m][r] = sum over group m of q * code for key t0 + 16kt + 4g + r and row i
+      const uint32_t sw[8] = {cur.ks[kt][0].x, cur.ks[kt][0].y, cur.ks[kt][0].z, cur.ks[kt][0].w,
+                              cur.ks[kt][1].x, cur.ks[kt][1].y, cur.ks[kt][1].z, cur.ks[kt][1].w};
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const h2 s01 = as_h2(sw[2 * r]), s23 = as_h2(sw[2 * r + 1]);
+        const float dot = part[0][r] * (float)s01[0] + part[1][r] * (float)s01[1] + part[2][r] * (float)s23[0] + part[3][r] * (float)s23[1];
+        const int key = t0 + 16 * kt + 4 * g + r;
+        s[4 * kt + r] = key < len ? dot * sc_log2 : -INFINITY;
+      }
+    }
+    // ---- online softmax (one running maximum per row, shared by its 4 lane groups) ----
+    float tmax = s[0];
+#pragma unroll
+    for (int e = 1; e < 8; ++e) tmax = fmaxf(tmax, s[e]);
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax);
+    const float alpha = exp2f(m_run - m_new);
+    m_run = m_new;
+    if (__any(alpha != 1.f)) {
+      l_run *= alpha;
+#pragma unroll
+      for (int b = 0; b < 8; ++b) { o[b][0] *= alpha; o[b][1] *= alpha; o[b][2] *= alpha; o[b][3] *= alpha; }
+    }
+    h8 pf;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { const float p = exp2f(s[e] - m_new); l_run += p; pf[e] = (_Float16)p; }
+    // ---- O^T += V^T P^T : 8 MFMAs, MFMA b covers channels 8*i' + b ----
+    h2 va[8][4];
+#pragma unroll
+    for (int pe = 0; pe < 4; ++pe) {
+      const uint32_t spk = (pe & 1) ? cur.vs[pe >> 1].y : cur.vs[pe >> 1].x;   // scales of tokens (2pe, 2pe+1) of this lane
+      const h2 s2 = as_h2(spk), s2q = s2 * h2{(_Float16)0.0625f, (_Float16)0.0625f};
+      const h2 c1032 = {(_Float16)1032.f, (_Float16)1032.f}, c1152 = {(_Float16)1152.f, (_Float16)1152.f};
+      const uint32_t w0 = cur.vw[2 * pe], w1 = cur.vw[2 * pe + 1];
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) {
+        // byte bb of both tokens side by side: low half = token 2pe, high half = token 2pe+1
+        const uint32_t x = ((w0 >> (8 * bb)) & 0xffu) | (((w1 >> (8 * bb)) & 0xffu) << 16);
+        va[2 * bb][pe] = (as_h2((x & 0x000f000fu) | kMagic) - c1032) * s2;
+        va[2 * bb + 1][pe] = (as_h2((x & 0x00f000f0u) | kMagic) - c1152) * s2q;
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < 8; ++b) {
+      const h8 vf = h8{va[b][0][0], va[b][0][1], va[b][1][0], va[b][1][1], va[b][2][0], va[b][2][1], va[b][3][0], va[b][3][1]};
+      o[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[b], 0, 0, 0);
+    }
+    cur = nxt;
+  }
+  // ---- merge the 4 waves of the workgroup, write one partial per (row, split) ----
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+  if (g == 0) { s_m[wave][i] = m_run; s_l[wave][i] = l_run; }
+#pragma unroll
+  for (int b = 0; b < 8; ++b)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) s_acc[wave][i][8 * (4 * g + r) + b] = o[b][r];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < 2 * kG * kD; idx += 256) {
+    const int j = idx >> 7, d = idx & (kD - 1);
+    const int tj = 2 * rt + j / kG;
+    if (tj >= A.M) continue;
+    const float m0 = s_m[0][j], m1 = s_m[1][j], m2 = s_m[2][j], m3 = s_m[3][j];
+    const float M2 = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
+    const float w0 = exp2f(m0 - M2), w1 = exp2f(m1 - M2), w2 = exp2f(m2 - M2), w3 = exp2f(m3 - M2);
+    const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
+    A.pacc[p * kD + d] = w0 * s_acc[0][j][d] + w1 * s_acc[1][j][d] + w2 * s_acc[2][j][d] + w3 * s_acc[3][j][d];
+    if (d == 0) { A.pm[p] = M2; A.pl[p] = w0 * s_l[0][j] + w1 * s_l[1][j] + w2 * s_l[2][j] + w3 * s_l[3][j]; }
+  }
+}
+
+void launch_attend_narrow(const AttnArgs& A, hipStream_t st) {
+  hipLaunchKernelGGL(attend_narrow_kernel, dim3(A.S, A.kv.n_kv, (A.M + 1) / 2), dim3(256), 0, st, A);
+}
+
+// combiner (reference: src/attention_kv4q.cu:325-332): M2 = max pm; w = pm > -1e29 ? 2^(pm-M2) : 0; y = sum w acc / sum w l.
+// grid (n_heads, M), block 128 (thread = channel)
+__global__ void __launch_bounds__(128) combine_kernel(CombineArgs A) {
+  const int head = blockIdx.x, tok = blockIdx.y, d = threadIdx.x;
+  float M2 = -1e30f;
+  for (int s = 0; s < A.S; ++s) M2 = fmaxf(M2, A.pm[((size_t)tok * A.S + s) * A.n_heads + head]);
+  float L = 0.f, o = 0.f;
+  for (int s = 0; s < A.S; ++s) {
+    const size_t p = ((size_t)tok * A.S + s) * A.n_heads + head;
+    const float pmv = A.pm[p];
+    const float w = pmv > -1e29f ? exp2f(pmv - M2) : 0.f;
+    L += w * A.pl[p]; o += w * A.pacc[p * kD + d];
+  }
+  A.out16[((size_t)tok * A.n_heads + head) * kD + d] = __half_as_ushort(__float2half_rn(o / L));
+}
+void launch_combine(const CombineArgs& A, hipStream_t st) {
+  hipLaunchKernelGGL(combine_kernel, dim3(A.n_heads, A.M), dim3(128), 0, st, A);
+}
+
+void launch_attend_wide(const AttnArgs& A, hipStream_t st) { launch_attend_narrow(A, st); }
+
+}  // namespace yka

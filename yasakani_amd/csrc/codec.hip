@@ -1,0 +1,119 @@
+// Quantize-on-append and the codec probes.  Compiled with -ffp-contract=off: the codec is bit-exact by contract,
+// and the reference builds with --fmad=false (CMakeLists.txt:60-63).
+//
+// Arithmetic per 32-channel group (reference: src/kvq_fast.cuh:194-198, src/kvq_gpu.cuh:85-86):
+//   am = max|x|; s = fp16(am / 7); if (s == 0) s = 1; q = clamp(rint(x / s), -7, 7); stored nibble = q + 8.
+// The division is by the stored (fp16-rounded) scale, as the reference divides by the scale it stores.
+#include "yka_internal.h"
+#include <hip/hip_fp16.h>
+
+namespace yka {
+
+__device__ __forceinline__ float h2f_bits(uint16_t b) { return __half2float(__ushort_as_half(b)); }
+// physical byte of a K row that holds logical byte j (channels 2j, 2j+1)
+__device__ __forceinline__ int k_code_byte(int j) { return 4 * k_phys_dword(j >> 2) + (j & 3); }
+
+// one lane = one channel; lanes of a 32-lane half-wave form one scale group
+__device__ __forceinline__ void quant_lane(float x, int& code, uint16_t& s16) {
+  float am = fabsf(x);
+#pragma unroll
+  for (int o = 16; o; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, 32));
+  const float s32 = __fdiv_rn(am, 7.0f);
+  s16 = __half_as_ushort(__float2half_rn(s32));
+  if ((s16 & 0x7fffu) == 0) s16 = 0x3c00u;
+  const float sd = h2f_bits(s16);
+  float q = rintf(__fdiv_rn(x, sd));
+  q = fminf(fmaxf(q, -7.f), 7.f);
+  code = (int)q + 8;
+}
+
+// grid (M, n_kv * 2), block 128: blockIdx.y = kvh * 2 + (0: K, 1: V); thread = channel.
+// Rows land at *d_pos + tok (reference: q35_kernels.cu:1038,1064 write the pass's rows before attention reads them).
+__global__ void __launch_bounds__(128) append_kernel(AppendArgs A) {
+  const int tok = blockIdx.x, kvh = blockIdx.y >> 1, isv = blockIdx.y & 1, d = threadIdx.x;
+  const int pos = *A.d_pos + tok;
+  if (pos < 0 || pos >= A.kv.max_ctx) return;
+  const uint16_t* src = (isv ? A.v16 : A.k16) + ((size_t)tok * A.kv.n_kv + kvh) * kD;
+  const float x = h2f_bits(src[d]);
+  int code; uint16_t s16;
+  quant_lane(x, code, s16);
+  const int nb = __shfl_xor(code, 1, 64);
+  uint8_t* pg = kv_page(A.kv, kvh, pos);
+  const int tp = pos % kPageTok;
+  if ((d & 1) == 0) {
+    const uint8_t byte = (uint8_t)((code & 15) | ((nb & 15) << 4));
+    if (isv) pg[kPageVc + tp * 64 + (d >> 1)] = byte;
+    else pg[kPageKc + tp * 64 + k_code_byte(d >> 1)] = byte;
+  }
+  if ((d & 31) == 0) {
+    if (isv) reinterpret_cast<uint16_t*>(pg + kPageVs)[(d >> 5) * kPageTok + tp] = s16;
+    else reinterpret_cast<uint16_t*>(pg + kPageKs)[tp * kNG + (d >> 5)] = s16;
+  }
+}
+void launch_append(const AppendArgs& A, hipStream_t st) {
+  hipLaunchKernelGGL(append_kernel, dim3(A.M, A.kv.n_kv * 2), dim3(128), 0, st, A);
+}
+
+// codec round trip: x16 [rows][128] -> codes [rows][64], scales [rows][4], y [rows][128] fp32
+__global__ void __launch_bounds__(128) codec_probe_kernel(const uint16_t* x16, int rows, uint8_t* codes, uint16_t* scales, float* y) {
+  const int row = blockIdx.x, d = threadIdx.x;
+  if (row >= rows) return;
+  const float x = h2f_bits(x16[(size_t)row * kD + d]);
+  int code; uint16_t s16;
+  quant_lane(x, code, s16);
+  const int nb = __shfl_xor(code, 1, 64);
+  if ((d & 1) == 0) codes[(size_t)row * (kD / 2) + (d >> 1)] = (uint8_t)((code & 15) | ((nb & 15) << 4));
+  if ((d & 31) == 0) scales[(size_t)row * kNG + (d >> 5)] = s16;
+  // decode: (nib - 8) * s, exact in fp32 (reference: src/kvq_attn.cuh:52-54)
+  y[(size_t)row * kD + d] = __fmul_rn((float)(code - 8), h2f_bits(s16));
+}
+void launch_codec_probe(const uint16_t* x16, int rows, uint8_t* codes, uint16_t* scales, float* y, hipStream_t st) {
+  hipLaunchKernelGGL(codec_probe_kernel, dim3(rows), dim3(128), 0, st, x16, rows, codes, scales, y);
+}
+
+// canonical image <-> physical pages.  grid (n, n_kv), block 64: lane j moves byte j of K and V codes; lanes 0..3 the scales.
+template <bool IMPORT>
+__global__ void __launch_bounds__(64) xfer_rows_kernel(KvView kv, int pos0, int n, uint8_t* kc, uint16_t* ks, uint8_t* vc, uint16_t* vs) {
+  const int t = blockIdx.x, kvh = blockIdx.y, j = threadIdx.x;
+  uint8_t* pg = kv_page(kv, kvh, pos0 + t);
+  const int tp = (pos0 + t) % kPageTok;
+  uint8_t* pk = pg + kPageKc + tp * 64 + k_code_byte(j);
+  uint8_t* pv = pg + kPageVc + tp * 64 + j;
+  uint16_t* pks = reinterpret_cast<uint16_t*>(pg + kPageKs) + tp * kNG + j;      // j < 4 only
+  uint16_t* pvs = reinterpret_cast<uint16_t*>(pg + kPageVs) + j * kPageTok + tp; // j < 4 only
+  const size_t row = (size_t)kvh * n + t;
+  if (IMPORT) {
+    *pk = kc[row * 64 + j]; *pv = vc[row * 64 + j];
+    if (j < kNG) { *pks = ks[row * kNG + j]; *pvs = vs[row * kNG + j]; }
+  } else {
+    kc[row * 64 + j] = *pk; vc[row * 64 + j] = *pv;
+    if (j < kNG) { ks[row * kNG + j] = *pks; vs[row * kNG + j] = *pvs; }
+  }
+}
+void launch_export_rows(const KvView& kv, int pos0, int n, uint8_t* kc, uint16_t* ks, uint8_t* vc, uint16_t* vs, hipStream_t st) {
+  hipLaunchKernelGGL(xfer_rows_kernel<false>, dim3(n, kv.n_kv), dim3(64), 0, st, kv, pos0, n, kc, ks, vc, vs);
+}
+void launch_import_rows(const KvView& kv, int pos0, int n, const uint8_t* kc, const uint16_t* ks, const uint8_t* vc, const uint16_t* vs, hipStream_t st) {
+  hipLaunchKernelGGL(xfer_rows_kernel<true>, dim3(n, kv.n_kv), dim3(64), 0, st, kv, pos0, n,
+                     const_cast<uint8_t*>(kc), const_cast<uint16_t*>(ks), const_cast<uint8_t*>(vc), const_cast<uint16_t*>(vs));
+}
+
+// decoder probe: k, v [n_kv][n][128] fp32 = (nib - 8) * scale
+__global__ void __launch_bounds__(128) dequant_rows_kernel(KvView kv, int pos0, int n, float* k, float* v) {
+  const int t = blockIdx.x, kvh = blockIdx.y, d = threadIdx.x;
+  const uint8_t* pg = kv_page(kv, kvh, pos0 + t);
+  const int tp = (pos0 + t) % kPageTok;
+  const size_t o = ((size_t)kvh * n + t) * kD + d;
+  const int kb = pg[kPageKc + tp * 64 + k_code_byte(d >> 1)], vb = pg[kPageVc + tp * 64 + (d >> 1)];
+  const int kn = (d & 1) ? (kb >> 4) : (kb & 15), vn = (d & 1) ? (vb >> 4) : (vb & 15);
+  k[o] = __fmul_rn((float)(kn - 8), h2f_bits(reinterpret_cast<const uint16_t*>(pg + kPageKs)[tp * kNG + (d >> 5)]));
+  v[o] = __fmul_rn((float)(vn - 8), h2f_bits(reinterpret_cast<const uint16_t*>(pg + kPageVs)[(d >> 5) * kPageTok + tp]));
+}
+void launch_dequant_rows(const KvView& kv, int pos0, int n, float* k, float* v, hipStream_t st) {
+  hipLaunchKernelGGL(dequant_rows_kernel, dim3(n, kv.n_kv), dim3(128), 0, st, kv, pos0, n, k, v);
+}
+
+__global__ void set_int_kernel(int* p, int v) { *p = v; }
+void launch_set_int(int* p, int v, hipStream_t st) { hipLaunchKernelGGL(set_int_kernel, dim3(1), dim3(1), 0, st, p, v); }
+
+}  // namespace yka

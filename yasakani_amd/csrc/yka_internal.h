@@ -1,0 +1,68 @@
+// Internal declarations shared by the translation units of libyka.so (gfx950 only).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace yka {
+
+// ---- fixed shape of the path ----
+constexpr int kD = 128;          // head_dim
+constexpr int kG = 6;            // query heads per KV head
+constexpr int kGroup = 32;       // channels per scale group
+constexpr int kNG = kD / kGroup; // scale groups per row (4)
+constexpr int kPageTok = 256;    // tokens per page
+// ---- physical page of one (page, kv head): 256 tokens, 36864 bytes, four planes ----
+//   +0      K codes  [256][64]  byte j of a row: channel 2j low nibble, 2j+1 high nibble, value q+8; the 16 dwords of a
+//                                row are stored in the order physical 4g+m = logical 4m+g, so that the 16-byte chunk g
+//                                holds channels {32m + 8g .. 32m + 8g + 7 : m = 0..3} - one dword of every scale group
+//   +16384  V codes  [256][64]  plain channel order
+//   +32768  K scales [256][4]   fp16, token major
+//   +34816  V scales [4][256]   fp16, group major (4 consecutive tokens of one group are 8 contiguous bytes)
+constexpr int kPageKc = 0, kPageVc = 16384, kPageKs = 32768, kPageVs = 34816, kPageBytes = 36864;
+__host__ __device__ inline int k_phys_dword(int logical) { return 4 * (logical & 3) + (logical >> 2); }
+constexpr int kMaxSlice = 64;    // rows per attention slice (kVerifyMax of the reference, engine35.hpp:157)
+
+// One layer's container.  The page of token t of kv head h starts at
+//   base + (p * n_kv + h) * 36864,   p = table ? table[t / 256] : t / 256
+struct KvView {
+  uint8_t* base;
+  const int32_t* table;  // nullptr in contiguous mode
+  int n_kv;
+  int max_ctx;
+};
+__host__ __device__ inline size_t kv_page_bytes(int n_kv) { return (size_t)n_kv * kPageBytes; }
+
+struct AppendArgs { KvView kv; const uint16_t* k16; const uint16_t* v16; const int* d_pos; int M; };
+
+// partial results of the split-KV kernels (same roles as pm/pl/pacc of the reference, args.hpp:10):
+//   pm, pl [rows_tok][S][n_heads]; pacc [rows_tok][S][n_heads][128].  pm is in log2 units; empty split: pm=-1e30, pl=0.
+struct AttnArgs {
+  KvView kv; const uint16_t* q16; const int* d_pos; const uint8_t* depth;
+  int M;        // rows (tokens) of this slice
+  int tok0;     // index of the slice's first row inside the pass (row t sees keys [0, *d_pos + depth(tok0+t) + 1))
+  int n_heads;
+  int S;        // splits
+  float* pm; float* pl; float* pacc;
+};
+struct CombineArgs { const float* pm; const float* pl; const float* pacc; int S; int M; int n_heads; uint16_t* out16; };
+
+// launchers (each checks nothing: the C layer validates shapes first)
+void launch_append(const AppendArgs&, hipStream_t);
+void launch_attend_narrow(const AttnArgs&, hipStream_t);   // 16-row tiles: 2 tokens x 6 heads per workgroup column
+void launch_attend_wide(const AttnArgs&, hipStream_t);     // 3..64 tokens
+void launch_combine(const CombineArgs&, hipStream_t);
+// canonical <-> physical
+void launch_export_rows(const KvView&, int pos0, int n, uint8_t* kc, uint16_t* ks, uint8_t* vc, uint16_t* vs, hipStream_t);
+void launch_import_rows(const KvView&, int pos0, int n, const uint8_t* kc, const uint16_t* ks, const uint8_t* vc, const uint16_t* vs, hipStream_t);
+void launch_dequant_rows(const KvView&, int pos0, int n, float* k, float* v, hipStream_t);
+void launch_codec_probe(const uint16_t* x16, int rows, uint8_t* codes, uint16_t* scales, float* y, hipStream_t);
+void launch_set_int(int* p, int v, hipStream_t);
+
+// start of the (page, kv head) block that holds token t
+__device__ __forceinline__ uint8_t* kv_page(const KvView& kv, int kvh, int t) {
+  const int lp = t / kPageTok;
+  const int pp = kv.table ? kv.table[lp] : lp;
+  return kv.base + (size_t)(pp * kv.n_kv + kvh) * kPageBytes;
+}
+
+}  // namespace yka

@@ -1,0 +1,212 @@
+"""ctypes binding of libyka.so - one Python method per entry point of include/yka_abi.h.
+
+Mirrors the reference's binding style (python/yasakani/_native.py:1-5): argtypes/restype declared once, every int
+return checked, the library's thread-local error string raised as RuntimeError.  Host-pointer hooks take numpy
+arrays; launch-path calls take raw device addresses (ints), e.g. torch.Tensor.data_ptr().
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+from .build import library_path
+
+D = 128          # head_dim
+GROUP = 32       # channels per scale group
+NG = D // GROUP
+PAGE = 256       # tokens per page
+
+
+class YkaError(RuntimeError):
+    pass
+
+
+class KvConfig(C.Structure):
+    _fields_ = [(n, C.c_int32) for n in
+                ("n_layers", "n_heads", "n_kv_heads", "head_dim", "max_ctx", "max_rows", "paged", "device")]
+
+
+def _load():
+    path = library_path()
+    if not os.path.exists(path):
+        raise YkaError(f"{path} is not built: run `python -c 'import __graft_entry__ as g; g.build()'` "
+                       "(there is no CPU fallback for this path)")
+    lib = C.CDLL(path)
+    vp, i32 = C.c_void_p, C.c_int
+    sig = {
+        "yka_kv_open": (vp, [C.POINTER(KvConfig)]),
+        "yka_kv_close": (None, [vp]),
+        "yka_last_error": (C.c_char_p, []),
+        "yka_build_info": (C.c_char_p, []),
+        "yka_set_opt": (i32, [vp, i32, i32]),
+        "yka_kv_set_page_table": (i32, [vp, i32, vp, i32]),
+        "yka_append": (i32, [vp, i32, vp, vp, i32, vp, vp]),
+        "yka_attend": (i32, [vp, i32, vp, i32, vp, vp, vp, vp]),
+        "yka_append_attend": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
+        "yka_codec_probe": (i32, [vp, i32, vp, vp, vp]),
+        "yka_kv_export_rows": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
+        "yka_kv_import_rows": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
+        "yka_kv_dequant_rows": (i32, [vp, i32, i32, i32, vp, vp]),
+        "yka_kv_replicate_layer": (i32, [vp, i32]),
+        "yka_layer_call_host": (i32, [vp, i32, vp, vp, vp, i32, i32, vp, vp]),
+        "yka_attn_bench": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp, vp]),
+    }
+    for name, (res, args) in sig.items():
+        fn = getattr(lib, name)
+        fn.restype, fn.argtypes = res, args
+    return lib
+
+
+EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "yka_set_opt", "yka_kv_set_page_table",
+           "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kv_export_rows",
+           "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
+           "yka_attn_bench")
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        _lib = _load()
+    return _lib
+
+
+def _chk(rc):
+    if rc != 0:
+        raise YkaError(lib().yka_last_error().decode("utf-8", "replace"))
+
+
+def _ptr(a):
+    return None if a is None else a.ctypes.data_as(C.c_void_p)
+
+
+def _u16(a, shape):
+    a = np.ascontiguousarray(a)
+    if a.dtype == np.float16:
+        a = a.view(np.uint16)
+    if a.dtype != np.uint16 or a.shape != tuple(shape):
+        raise ValueError(f"expected fp16/uint16 array of shape {tuple(shape)}, got {a.dtype} {a.shape}")
+    return a
+
+
+def build_info() -> str:
+    return lib().yka_build_info().decode()
+
+
+def codec_probe(x16):
+    """x16 [rows,128] fp16 -> (codes [rows,64] u8, scales [rows,4] u16 bit patterns, y [rows,128] f32)."""
+    x16 = np.ascontiguousarray(x16)
+    rows = x16.shape[0]
+    x = _u16(x16, (rows, D))
+    codes = np.empty((rows, D // 2), np.uint8)
+    scales = np.empty((rows, NG), np.uint16)
+    y = np.empty((rows, D), np.float32)
+    _chk(lib().yka_codec_probe(_ptr(x), rows, _ptr(codes), _ptr(scales), _ptr(y)))
+    return codes, scales, y
+
+
+class KvCache:
+    """Owns the int4 KV containers of `n_layers` layers on one GPU (the role Engine35 plays for its KV, engine35.cpp:303-329)."""
+
+    def __init__(self, n_layers=1, n_heads=24, n_kv_heads=4, head_dim=D, max_ctx=4096, max_rows=64, paged=False, device=0):
+        self.cfg = KvConfig(n_layers, n_heads, n_kv_heads, head_dim, max_ctx, max_rows, int(bool(paged)), device)
+        self._h = lib().yka_kv_open(C.byref(self.cfg))
+        if not self._h:
+            raise YkaError(lib().yka_last_error().decode("utf-8", "replace"))
+
+    # -- lifetime --
+    def close(self):
+        if getattr(self, "_h", None):
+            lib().yka_kv_close(self._h)
+            self._h = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def n_heads(self):
+        return self.cfg.n_heads
+
+    @property
+    def n_kv_heads(self):
+        return self.cfg.n_kv_heads
+
+    @property
+    def max_ctx(self):
+        return self.cfg.max_ctx
+
+    # -- options / layout --
+    def set_opt(self, key, value):
+        _chk(lib().yka_set_opt(self._h, key, value))
+
+    def set_page_table(self, table, layer=-1):
+        t = np.ascontiguousarray(table, dtype=np.int32)
+        _chk(lib().yka_kv_set_page_table(self._h, layer, _ptr(t), t.size))
+
+    # -- launch path: device addresses --
+    def append(self, layer, d_k16, d_v16, M, d_pos, stream=0):
+        _chk(lib().yka_append(self._h, layer, d_k16, d_v16, M, d_pos, stream))
+
+    def attend(self, layer, d_q16, M, d_pos, d_out16, d_depth=None, stream=0):
+        _chk(lib().yka_attend(self._h, layer, d_q16, M, d_pos, d_depth, d_out16, stream))
+
+    def append_attend(self, layer, d_q16, d_k16, d_v16, M, d_pos, d_out16, d_depth=None, stream=0):
+        _chk(lib().yka_append_attend(self._h, layer, d_q16, d_k16, d_v16, M, d_pos, d_depth, d_out16, stream))
+
+    # -- hooks: host arrays --
+    def export_rows(self, layer, pos0, n):
+        kvh = self.cfg.n_kv_heads
+        kc = np.empty((kvh, n, D // 2), np.uint8); vc = np.empty_like(kc)
+        ks = np.empty((kvh, n, NG), np.uint16); vs = np.empty_like(ks)
+        _chk(lib().yka_kv_export_rows(self._h, layer, pos0, n, _ptr(kc), _ptr(ks), _ptr(vc), _ptr(vs)))
+        return kc, ks, vc, vs
+
+    def import_rows(self, layer, pos0, kc, ks, vc, vs):
+        kvh = self.cfg.n_kv_heads
+        n = kc.shape[1]
+        kc = np.ascontiguousarray(kc, np.uint8); vc = np.ascontiguousarray(vc, np.uint8)
+        ks = _u16(ks, (kvh, n, NG)); vs = _u16(vs, (kvh, n, NG))
+        if kc.shape != (kvh, n, D // 2) or vc.shape != kc.shape:
+            raise ValueError("codes must be [n_kv_heads, n, 64]")
+        _chk(lib().yka_kv_import_rows(self._h, layer, pos0, n, _ptr(kc), _ptr(ks), _ptr(vc), _ptr(vs)))
+
+    def dequant_rows(self, layer, pos0, n):
+        kvh = self.cfg.n_kv_heads
+        k = np.empty((kvh, n, D), np.float32); v = np.empty_like(k)
+        _chk(lib().yka_kv_dequant_rows(self._h, layer, pos0, n, _ptr(k), _ptr(v)))
+        return k, v
+
+    def replicate_layer(self, src=0):
+        _chk(lib().yka_kv_replicate_layer(self._h, src))
+
+    def layer_call(self, layer, q16, k16, v16, pos, depth=None):
+        """One layer call with host arrays: q16 [M,n_heads,128], k16/v16 [M,n_kv_heads,128] fp16 (or None = attend only)."""
+        M = q16.shape[0]
+        q = _u16(q16, (M, self.cfg.n_heads, D))
+        k = None if k16 is None else _u16(k16, (M, self.cfg.n_kv_heads, D))
+        v = None if v16 is None else _u16(v16, (M, self.cfg.n_kv_heads, D))
+        dep = None if depth is None else np.ascontiguousarray(depth, np.uint8)
+        out = np.empty((M, self.cfg.n_heads, D), np.uint16)
+        _chk(lib().yka_layer_call_host(self._h, layer, _ptr(q), _ptr(k), _ptr(v), M, pos, _ptr(dep), _ptr(out)))
+        return out.view(np.float16)
+
+    def bench(self, q16, k16, v16, pos, mode=0, use_graph=True, reps=20):
+        """Timed sweeps over all layers; returns (ms per sweep [reps], out of the last layer call)."""
+        M = q16.shape[0]
+        q = _u16(q16, (M, self.cfg.n_heads, D))
+        k = None if k16 is None else _u16(k16, (M, self.cfg.n_kv_heads, D))
+        v = None if v16 is None else _u16(v16, (M, self.cfg.n_kv_heads, D))
+        ms = np.zeros(reps, np.float32)
+        out = np.empty((M, self.cfg.n_heads, D), np.uint16)
+        _chk(lib().yka_attn_bench(self._h, _ptr(q), _ptr(k), _ptr(v), M, pos, mode, int(bool(use_graph)), reps, _ptr(ms), _ptr(out)))
+        return ms, out.view(np.float16)
