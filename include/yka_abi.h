@@ -102,6 +102,22 @@ YKA_API int yka_kv_replicate_layer(yka_kv* kv, int src);
 YKA_API int yka_layer_call_host(yka_kv* kv, int layer, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16,
                                 int M, int pos, const uint8_t* depth, uint16_t* out16);
 
+/* Host-pointer form of yka_append alone (fills a container from fp16 rows; model: the encode step of
+ * yskn_atxpk_bench, kvx_probe.cu:361-369). */
+YKA_API int yka_append_host(yka_kv* kv, int layer, const uint16_t* k16, const uint16_t* v16, int M, int pos);
+
+/* Captured passes.  The reference replays each pass shape from a CUDA graph (Engine35::run_pass, engine35.cpp:1977-1988;
+ * decode loop engine35.cpp:2365-2375).  yka_pass_capture records, for each of the n listed layers in order, one layer
+ * call (mode 0: append + attend, 1: attend only, 2: attention kernel alone) with the given device buffers into a
+ * hipGraph; yka_pass_launch replays it on `hip_stream`.  Positions are read from d_pos at replay time.  All layer
+ * calls of one graph share d_out16 and the handle's partial workspace, so they run in order. */
+typedef struct yka_pass yka_pass;
+YKA_API yka_pass* yka_pass_capture(yka_kv* kv, const int32_t* layers, int n, const uint16_t* d_q16, const uint16_t* d_k16,
+                                   const uint16_t* d_v16, int M, const int* d_pos, const uint8_t* d_depth,
+                                   uint16_t* d_out16, int mode);
+YKA_API int yka_pass_launch(yka_pass* p, void* hip_stream);
+YKA_API void yka_pass_destroy(yka_pass* p);
+
 /* Timed sweeps, replaces yskn_atxpk_bench (kvx_probe.cu:322-449): with q/k/v uploaded once and the device position
  * fixed at `pos`, runs one warm sweep over all layers and then `reps` timed sweeps (hipEvents on the internal
  * stream), each sweep = one layer call per layer on distinct containers.  mode 0 = append + attend, 1 = attend only,

@@ -322,6 +322,69 @@ int yka_layer_call_host(yka_kv* kv, int layer, const uint16_t* q16, const uint16
   YKA_CATCH_INT
 }
 
+int yka_append_host(yka_kv* kv, int layer, const uint16_t* k16, const uint16_t* v16, int M, int pos) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer);
+  if (!k16 || !v16 || M < 1) throw std::runtime_error("bad argument");
+  if (pos < 0 || (long long)pos + M > kv->cfg.max_ctx) throw std::runtime_error("pos + M exceeds max_ctx");
+  const size_t nk = (size_t)M * kv->cfg.n_kv_heads * kD;
+  DevBuf dk(nk * 2), dv(nk * 2);
+  HIPCHK(hipMemcpy(dk.p, k16, nk * 2, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dv.p, v16, nk * 2, hipMemcpyHostToDevice));
+  HIPCHK(hipDeviceSynchronize());
+  launch_set_int(kv->d_pos, pos, kv->stream);
+  do_append(kv, layer, dk.as<uint16_t>(), dv.as<uint16_t>(), M, kv->d_pos, kv->stream);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipStreamSynchronize(kv->stream));
+  YKA_CATCH_INT
+}
+
+struct yka_pass { hipGraph_t graph = nullptr; hipGraphExec_t exec = nullptr; int device = 0; };
+
+yka_pass* yka_pass_capture(yka_kv* kv, const int32_t* layers, int n, const uint16_t* d_q16, const uint16_t* d_k16,
+                           const uint16_t* d_v16, int M, const int* d_pos, const uint8_t* d_depth, uint16_t* d_out16, int mode) {
+  yka_pass* p = nullptr;
+  bool capturing = false;
+  try {
+    on_device(kv); check_rows(kv, M);
+    if (!layers || n < 1 || !d_q16 || !d_pos || !d_out16 || mode < 0 || mode > 2) throw std::runtime_error("bad argument");
+    if (mode == 0 && (!d_k16 || !d_v16)) throw std::runtime_error("mode 0 needs d_k16 and d_v16");
+    for (int i = 0; i < n; ++i) check_layer(kv, layers[i]);
+    p = new yka_pass(); p->device = kv->cfg.device;
+    hipStream_t st = kv->stream;
+    HIPCHK(hipStreamSynchronize(st));
+    HIPCHK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+    capturing = true;
+    for (int i = 0; i < n; ++i) {
+      if (mode == 0) do_append(kv, layers[i], d_k16, d_v16, M, d_pos, st);
+      do_attend(kv, layers[i], d_q16, M, d_pos, d_depth, d_out16, st, mode == 2 ? 2 : 0);
+    }
+    capturing = false;
+    HIPCHK(hipStreamEndCapture(st, &p->graph));
+    HIPCHK(hipGraphInstantiate(&p->exec, p->graph, nullptr, nullptr, 0));
+    return p;
+  } catch (const std::exception& e) { g_err = e.what(); }
+  catch (...) { g_err = "unknown error"; }
+  if (capturing) { hipGraph_t g = nullptr; (void)hipStreamEndCapture(kv->stream, &g); if (g) (void)hipGraphDestroy(g); }
+  yka_pass_destroy(p);
+  return nullptr;
+}
+
+int yka_pass_launch(yka_pass* p, void* hip_stream) {
+  YKA_TRY
+  if (!p || !p->exec) throw std::runtime_error("null pass");
+  HIPCHK(hipSetDevice(p->device));
+  HIPCHK(hipGraphLaunch(p->exec, (hipStream_t)hip_stream));
+  YKA_CATCH_INT
+}
+
+void yka_pass_destroy(yka_pass* p) {
+  if (!p) return;
+  if (p->exec) (void)hipGraphExecDestroy(p->exec);
+  if (p->graph) (void)hipGraphDestroy(p->graph);
+  delete p;
+}
+
 int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, int pos, int mode,
                    int use_graph, int reps, float* ms, uint16_t* out16_last) {
   hipEvent_t e0 = nullptr, e1 = nullptr;

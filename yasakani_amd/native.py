@@ -49,6 +49,10 @@ def _load():
         "yka_kv_dequant_rows": (i32, [vp, i32, i32, i32, vp, vp]),
         "yka_kv_replicate_layer": (i32, [vp, i32]),
         "yka_layer_call_host": (i32, [vp, i32, vp, vp, vp, i32, i32, vp, vp]),
+        "yka_append_host": (i32, [vp, i32, vp, vp, i32, i32]),
+        "yka_pass_capture": (vp, [vp, vp, i32, vp, vp, vp, i32, vp, vp, vp, i32]),
+        "yka_pass_launch": (i32, [vp, vp]),
+        "yka_pass_destroy": (None, [vp]),
         "yka_attn_bench": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp, vp]),
     }
     for name, (res, args) in sig.items():
@@ -60,7 +64,7 @@ def _load():
 EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "yka_set_opt", "yka_kv_set_page_table",
            "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kv_export_rows",
            "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
-           "yka_attn_bench")
+           "yka_append_host", "yka_pass_capture", "yka_pass_launch", "yka_pass_destroy", "yka_attn_bench")
 
 _lib = None
 
@@ -200,6 +204,20 @@ class KvCache:
         _chk(lib().yka_layer_call_host(self._h, layer, _ptr(q), _ptr(k), _ptr(v), M, pos, _ptr(dep), _ptr(out)))
         return out.view(np.float16)
 
+    def append_host(self, layer, k16, v16, pos):
+        """Quantize host rows k16/v16 [M,n_kv_heads,128] into rows pos..pos+M-1."""
+        M = k16.shape[0]
+        k = _u16(k16, (M, self.cfg.n_kv_heads, D)); v = _u16(v16, (M, self.cfg.n_kv_heads, D))
+        _chk(lib().yka_append_host(self._h, layer, _ptr(k), _ptr(v), M, pos))
+
+    def capture_pass(self, layers, d_q16, d_k16, d_v16, M, d_pos, d_out16, d_depth=None, mode=0):
+        """Records one layer call per listed layer into a graph (device addresses); returns a Pass."""
+        ls = np.ascontiguousarray(layers, np.int32)
+        h = lib().yka_pass_capture(self._h, _ptr(ls), ls.size, d_q16, d_k16, d_v16, M, d_pos, d_depth, d_out16, mode)
+        if not h:
+            raise YkaError(lib().yka_last_error().decode("utf-8", "replace"))
+        return Pass(h)
+
     def bench(self, q16, k16, v16, pos, mode=0, use_graph=True, reps=20):
         """Timed sweeps over all layers; returns (ms per sweep [reps], out of the last layer call)."""
         M = q16.shape[0]
@@ -210,3 +228,24 @@ class KvCache:
         out = np.empty((M, self.cfg.n_heads, D), np.uint16)
         _chk(lib().yka_attn_bench(self._h, _ptr(q), _ptr(k), _ptr(v), M, pos, mode, int(bool(use_graph)), reps, _ptr(ms), _ptr(out)))
         return ms, out.view(np.float16)
+
+
+class Pass:
+    """A captured sequence of layer calls (the reference replays captured passes, engine35.cpp:1977-1988)."""
+
+    def __init__(self, handle):
+        self._h = handle
+
+    def launch(self, stream=0):
+        _chk(lib().yka_pass_launch(self._h, stream))
+
+    def close(self):
+        if self._h:
+            lib().yka_pass_destroy(self._h)
+            self._h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
