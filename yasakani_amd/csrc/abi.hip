@@ -26,7 +26,7 @@ struct yka_kv {
   size_t layer_bytes = 0;
   uint8_t* pool = nullptr;
   int32_t* tables = nullptr;       // [n_layers][n_pages], paged mode only
-  float *pm = nullptr, *pl = nullptr, *pacc = nullptr;
+  float *pm = nullptr, *pl = nullptr; uint16_t* pacc16 = nullptr;
   size_t ws_rows = 0;              // capacity of the partial workspace in (token, split) pairs
   int* d_pos = nullptr;            // position used by the host-pointer hooks
   hipStream_t stream = nullptr;    // stream of the host-pointer hooks
@@ -53,7 +53,7 @@ void on_device(const yka_kv* kv) {
 }
 
 constexpr int kMaxSplits = 128;
-constexpr size_t kWsPairs = 512;  // (token, split) pairs the partial workspace holds: 512 * 24 * 130 floats = 6.4 MB
+constexpr size_t kWsPairs = 4096;  // (token, split) pairs the partial workspace holds: 4096 * 24 * (256 + 8) bytes = 26 MB
 
 // splits for the narrow kernel: enough workgroups (n_kv * S * ceil(M/2)) to cover 256 CUs about twice over
 int narrow_splits(const yka_kv* kv, int M) {
@@ -62,6 +62,16 @@ int narrow_splits(const yka_kv* kv, int M) {
   int S = 512 / (kv->cfg.n_kv_heads * tiles);
   S = std::max(2, std::min(kMaxSplits, S));
   return std::min(S, (int)(kWsPairs / (size_t)M));
+}
+
+// Wide kernel geometry: a workgroup owns 128 query rows (4 waves x 32) and one split; two workgroups share a CU.
+// Splits: about two workgroups per CU; the partial sums (M * S * 24 * 264 bytes) stay below the KV stream they summarise.
+int wide_rows_per_block(int) { return 128; }
+int wide_splits(const yka_kv* kv, int M) {
+  const int rows = kG * M, rpb = wide_rows_per_block(M), rb = (rows + rpb - 1) / rpb;
+  int S = kv->opt_splits_wide > 0 ? kv->opt_splits_wide : 512 / (kv->cfg.n_kv_heads * rb);
+  S = std::max(1, std::min(kMaxSplits, S));
+  return std::min(S, std::max(1, (int)kWsPairs / M));
 }
 
 void check_layer(const yka_kv* kv, int layer) {
@@ -81,10 +91,11 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
   const int NH = kv->cfg.n_heads;
   for (int s0 = 0; s0 < M; s0 += kMaxSlice) {   // 64-row slices, as attn_block cuts wide passes (engine35.cpp:935-947)
     const int Ms = std::min(kMaxSlice, M - s0);
-    const int S = narrow_splits(kv, Ms);
-    AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * kD, d_pos, depth, Ms, s0, NH, S, kv->pm, kv->pl, kv->pacc};
-    if (Ms <= 2 || kv->opt_force_narrow) launch_attend_narrow(A, st); else launch_attend_wide(A, st);
-    if (mode != 2) launch_combine(CombineArgs{kv->pm, kv->pl, kv->pacc, S, Ms, NH, out16 + (size_t)s0 * NH * kD}, st);
+    const bool narrow = Ms <= 2 || kv->opt_force_narrow;
+    const int S = narrow ? narrow_splits(kv, Ms) : wide_splits(kv, Ms);
+    AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * kD, d_pos, depth, Ms, s0, NH, S, wide_rows_per_block(Ms), kv->pm, kv->pl, kv->pacc16};
+    if (narrow) launch_attend_narrow(A, st); else launch_attend_wide(A, st);
+    if (mode != 2) launch_combine(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD}, st);
   }
 }
 
@@ -138,7 +149,7 @@ yka_kv* yka_kv_open(const yka_kv_config* cfg) {
     const size_t np = kv->ws_rows * cfg->n_heads;
     HIPCHK(hipMalloc((void**)&kv->pm, np * 4));
     HIPCHK(hipMalloc((void**)&kv->pl, np * 4));
-    HIPCHK(hipMalloc((void**)&kv->pacc, np * kD * 4));
+    HIPCHK(hipMalloc((void**)&kv->pacc16, np * kD * 2));
     HIPCHK(hipMalloc((void**)&kv->d_pos, 4));
     HIPCHK(hipMemset(kv->d_pos, 0, 4));
     HIPCHK(hipStreamCreateWithFlags(&kv->stream, hipStreamNonBlocking));
@@ -156,7 +167,7 @@ void yka_kv_close(yka_kv* kv) {
   (void)hipSetDevice(kv->cfg.device);
   (void)hipDeviceSynchronize();
   if (kv->stream) (void)hipStreamDestroy(kv->stream);
-  (void)hipFree(kv->pool); (void)hipFree(kv->tables); (void)hipFree(kv->pm); (void)hipFree(kv->pl); (void)hipFree(kv->pacc); (void)hipFree(kv->d_pos);
+  (void)hipFree(kv->pool); (void)hipFree(kv->tables); (void)hipFree(kv->pm); (void)hipFree(kv->pl); (void)hipFree(kv->pacc16); (void)hipFree(kv->d_pos);
   delete kv;
 }
 

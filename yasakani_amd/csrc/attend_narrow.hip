@@ -193,8 +193,10 @@ __global__ void __launch_bounds__(256) attend_narrow_kernel(AttnArgs A) {
     const float M2 = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
     const float w0 = exp2f(m0 - M2), w1 = exp2f(m1 - M2), w2 = exp2f(m2 - M2), w3 = exp2f(m3 - M2);
     const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
-    A.pacc[p * kD + d] = w0 * s_acc[0][j][d] + w1 * s_acc[1][j][d] + w2 * s_acc[2][j][d] + w3 * s_acc[3][j][d];
-    if (d == 0) { A.pm[p] = M2; A.pl[p] = w0 * s_l[0][j] + w1 * s_l[1][j] + w2 * s_l[2][j] + w3 * s_l[3][j]; }
+    const float L = w0 * s_l[0][j] + w1 * s_l[1][j] + w2 * s_l[2][j] + w3 * s_l[3][j];
+    const float acc = w0 * s_acc[0][j][d] + w1 * s_acc[1][j][d] + w2 * s_acc[2][j][d] + w3 * s_acc[3][j][d];
+    A.pacc16[p * kD + d] = __half_as_ushort(__float2half_rn(L > 0.f ? acc / L : 0.f));
+    if (d == 0) { A.pm[p] = M2; A.pl[p] = L; }
   }
 }
 
@@ -202,25 +204,50 @@ void launch_attend_narrow(const AttnArgs& A, hipStream_t st) {
   hipLaunchKernelGGL(attend_narrow_kernel, dim3(A.S, A.kv.n_kv, (A.M + 1) / 2), dim3(256), 0, st, A);
 }
 
-// combiner (reference: src/attention_kv4q.cu:325-332): M2 = max pm; w = pm > -1e29 ? 2^(pm-M2) : 0; y = sum w acc / sum w l.
-// grid (n_heads, M), block 128 (thread = channel)
-__global__ void __launch_bounds__(128) combine_kernel(CombineArgs A) {
-  const int head = blockIdx.x, tok = blockIdx.y, d = threadIdx.x;
-  float M2 = -1e30f;
-  for (int s = 0; s < A.S; ++s) M2 = fmaxf(M2, A.pm[((size_t)tok * A.S + s) * A.n_heads + head]);
-  float L = 0.f, o = 0.f;
-  for (int s = 0; s < A.S; ++s) {
-    const size_t p = ((size_t)tok * A.S + s) * A.n_heads + head;
-    const float pmv = A.pm[p];
-    const float w = pmv > -1e29f ? exp2f(pmv - M2) : 0.f;
-    L += w * A.pl[p]; o += w * A.pacc[p * kD + d];
+// combiner (reference: src/attention_kv4q.cu:325-332): M2 = max pm; w_s = pm_s > -1e29 ? 2^(pm_s - M2) * pl_s : 0;
+// y = sum w_s * (acc_s / l_s) / sum w_s.  grid (n_heads, M), block 256: 16 lanes x 8 channels cover a row, 16 split
+// lanes run in parallel and are summed through LDS.
+__global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
+  __shared__ float s_w[128];
+  __shared__ float s_o[16][kD + 4];
+  __shared__ float s_wsum[16];
+  const int head = blockIdx.x, tok = blockIdx.y, tid = threadIdx.x;
+  const size_t p0 = (size_t)tok * A.S * A.n_heads + head;      // split s lives at p0 + s * n_heads
+  // weights: every thread of the first two waves looks at one split
+  float pmv = -1e30f, plv = 0.f;
+  if (tid < A.S) { pmv = A.pm[p0 + (size_t)tid * A.n_heads]; plv = A.pl[p0 + (size_t)tid * A.n_heads]; }
+  float M2 = pmv;
+#pragma unroll
+  for (int o = 32; o; o >>= 1) M2 = fmaxf(M2, __shfl_xor(M2, o, 64));
+  if (tid < 128 && (tid & 63) == 0) s_wsum[tid >> 6] = M2;
+  __syncthreads();
+  M2 = fmaxf(s_wsum[0], s_wsum[1]);
+  if (tid < 128) s_w[tid] = (tid < A.S && pmv > -1e29f) ? exp2f(pmv - M2) * plv : 0.f;
+  __syncthreads();
+  const int sl = tid >> 4, c8 = (tid & 15) * 8;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float wsum = 0.f;
+  for (int s = sl; s < A.S; s += 16) {
+    const float w = s_w[s];
+    const uint4 u = *reinterpret_cast<const uint4*>(A.pacc16 + (p0 + (size_t)s * A.n_heads) * kD + c8);
+    const h8 v = __builtin_bit_cast(h8, u);
+#pragma unroll
+    for (int c = 0; c < 8; ++c) acc[c] += w * (float)v[c];
+    wsum += w;
   }
-  A.out16[((size_t)tok * A.n_heads + head) * kD + d] = __half_as_ushort(__float2half_rn(o / L));
+#pragma unroll
+  for (int c = 0; c < 8; ++c) s_o[sl][c8 + c] = acc[c];
+  if ((tid & 15) == 0) s_wsum[sl] = wsum;
+  __syncthreads();
+  if (tid < kD) {
+    float o = 0.f, L = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) { o += s_o[k][tid]; L += s_wsum[k]; }
+    A.out16[((size_t)tok * A.n_heads + head) * kD + tid] = __half_as_ushort(__float2half_rn(o / L));
+  }
 }
 void launch_combine(const CombineArgs& A, hipStream_t st) {
-  hipLaunchKernelGGL(combine_kernel, dim3(A.n_heads, A.M), dim3(128), 0, st, A);
+  hipLaunchKernelGGL(combine_kernel, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
 }
-
-void launch_attend_wide(const AttnArgs& A, hipStream_t st) { launch_attend_narrow(A, st); }
 
 }  // namespace yka

@@ -1,0 +1,276 @@
+// Split-KV attention for windows of 3..64 query tokens (verify windows, prefill slices).  gfx950.
+//
+// Same mathematics as the narrow kernel (reference: src/q35_atxpk4.cuh:71-499 for the window shape, row geometry
+// src/q35_atxpk.cu:391-411): every row t of the window runs an online softmax over the keys [0, len(t)) of its
+// split and leaves (m, l, acc) partials for the combiner.  What differs is who dequantizes:
+//   * a workgroup of 4 waves owns up to 128 query rows (token-major, 6 heads per token) and one split of the keys.
+//     Each 32-key tile is dequantized ONCE per workgroup into LDS - K as exact integer codes in fp16 (n-8, odd nibbles
+//     16(n-8)), V scaled and transposed (channel-major, the operand shape of the token-contracting MFMA) - and every
+//     wave reads its MFMA fragments from there;
+//   * a wave owns one tile of 32 rows (MFMA 32x32x16, the shape that sustains the full matrix rate on this chip) and
+//     stays under 256 registers, so two waves share a SIMD: one runs MFMAs while the other runs the softmax VALU work,
+//     and all MFMA results live in ordinary VGPRs (no accumulator-file copies);
+//   * the group scales of K are applied to the fp32 partial sum of each 32-channel group (two chained MFMAs per
+//     group), so K is never rounded; V carries one fp16 rounding;
+//   * the running maximum of a row is only raised when a score exceeds it by more than 2^8: accumulators stay in
+//     their registers untouched on almost every tile;
+//   * LDS is double buffered: tile n+1 is dequantized while tile n is consumed; one barrier per tile.
+// LDS image of one tile (19200 bytes):
+//   K  [32 keys][272 B]   chunk 4m+g of a key = channels 32m+8g..+7 in the order n0,n4,n1,n5,n2,n6,n3,n7; the 272-byte
+//                          pitch makes the lanes of a fragment read hit distinct banks
+//   V  [128 rows][80 B]   channel 8*dw+c lives in row 16*sigma(c)+dw, sigma(c) = 2*(c&3) + (c>>2): the 16 lanes that
+//                          dequantize one byte position write 16 consecutive rows, and an output lane ends up with runs
+//                          of 8 consecutive channels.  Inside a row token 16u+8a+4h+b sits at position 16u+8h+4a+b, so
+//                          the 8 tokens an MFMA lane needs are 16 contiguous bytes
+//   Ks [32 keys][4] fp16
+#include "yka_internal.h"
+#include <hip/hip_fp16.h>
+
+namespace yka {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+namespace {
+
+__device__ __forceinline__ h2 as_h2(uint32_t u) { return __builtin_bit_cast(h2, u); }
+__device__ __forceinline__ uint32_t as_u32(h2 h) { return __builtin_bit_cast(uint32_t, h); }
+
+constexpr uint32_t kMagic = 0x64006400u;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kKPitch = 272, kVPitch = 80;
+constexpr int kLdsK = 0, kLdsV = 32 * kKPitch, kLdsKs = kLdsV + 128 * kVPitch, kLdsBuf = kLdsKs + 256;   // 19200
+constexpr int NT = 256;                        // threads per workgroup
+constexpr float kRaise = 8.f;                  // log2 slack before a running maximum is raised
+
+struct Raw {                                   // one thread's share of a raw 32-key tile
+  uint32_t kw[2];
+  uint32_t vw[2];
+  uint32_t vs;
+  uint32_t ks;
+};
+
+__device__ __forceinline__ void load_raw(const uint8_t* pg, int tp, int tid, Raw& R) {
+  const uint32_t* kc = reinterpret_cast<const uint32_t*>(pg + kPageKc + (size_t)tp * 64);
+  R.kw[0] = kc[tid]; R.kw[1] = kc[tid + NT];
+  const int pair = tid >> 4, dw = tid & 15;
+  const uint32_t* vc = reinterpret_cast<const uint32_t*>(pg + kPageVc + (size_t)(tp + 2 * pair) * 64) + dw;
+  R.vw[0] = vc[0]; R.vw[1] = vc[16];
+  R.vs = *reinterpret_cast<const uint32_t*>(pg + kPageVs + ((size_t)(dw >> 2) * kPageTok + tp + 2 * pair) * 2);
+  if (tid < 64) R.ks = reinterpret_cast<const uint32_t*>(pg + kPageKs + (size_t)tp * 8)[tid];
+}
+
+__device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw& R) {
+  const h2 c1032 = {(_Float16)1032.f, (_Float16)1032.f}, c1152 = {(_Float16)1152.f, (_Float16)1152.f};
+#pragma unroll
+  for (int u = 0; u < 2; ++u) {
+    const int idx = tid + u * NT, key = idx >> 4, p = idx & 15;      // physical dword p = 4g+m of the key row
+    const uint32_t w = R.kw[u], t = w >> 8;
+    uint4 o;
+    o.x = as_u32(as_h2((w & 0x000f000fu) | kMagic) - c1032);
+    o.y = as_u32(as_h2((w & 0x00f000f0u) | kMagic) - c1152);
+    o.z = as_u32(as_h2((t & 0x000f000fu) | kMagic) - c1032);
+    o.w = as_u32(as_h2((t & 0x00f000f0u) | kMagic) - c1152);
+    *reinterpret_cast<uint4*>(buf + kLdsK + key * kKPitch + (4 * (p & 3) + (p >> 2)) * 16) = o;
+  }
+  {
+    const int pair = tid >> 4, dw = tid & 15;
+    const int t0 = 2 * pair;                                         // token 16u + 8a + 4h + b -> position 16u + 8h + 4a + b
+    const int posn = (t0 & 16) + 8 * ((t0 >> 2) & 1) + 4 * ((t0 >> 3) & 1) + (t0 & 3);
+    const h2 s2 = as_h2(R.vs), s2q = s2 * h2{(_Float16)0.0625f, (_Float16)0.0625f};
+    const uint32_t w0 = R.vw[0], w1 = R.vw[1];
+    uint8_t* vb = buf + kLdsV + dw * kVPitch + posn * 2;
+#pragma unroll
+    for (int bb = 0; bb < 4; ++bb) {
+      // byte bb of both tokens side by side (low half = token t0, high half = token t0+1)
+      const uint32_t x = __builtin_amdgcn_perm(w1, w0, 0x0c040c00u + bb * 0x00010001u);
+      const h2 lo = (as_h2((x & 0x000f000fu) | kMagic) - c1032) * s2;       // channel c = 2bb
+      const h2 hi = (as_h2((x & 0x00f000f0u) | kMagic) - c1152) * s2q;      // channel c = 2bb+1
+      const int c0 = 2 * bb, c1 = 2 * bb + 1;
+      *reinterpret_cast<uint32_t*>(vb + 16 * (2 * (c0 & 3) + (c0 >> 2)) * kVPitch) = as_u32(lo);
+      *reinterpret_cast<uint32_t*>(vb + 16 * (2 * (c1 & 3) + (c1 >> 2)) * kVPitch) = as_u32(hi);
+    }
+  }
+  if (tid < 64) reinterpret_cast<uint32_t*>(buf + kLdsKs)[tid] = R.ks;
+}
+
+}  // namespace
+
+// grid (S, n_kv, ceil(6M / rows_per_block)), block 256; wave w owns rows [32 RT w, 32 RT (w+1)) of the block
+template <int RT>
+__global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
+  __shared__ __align__(16) uint8_t lds[2][kLdsBuf];
+  const int split = blockIdx.x, kvh = blockIdx.y, rb = blockIdx.z;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 31, h = lane >> 5;
+  const int pos = *A.d_pos;
+  const int nrows = kG * A.M;
+
+  // rows of this wave: R = rb*128*RT + wave*32*RT + rt*32 + j  ->  token R/6 of the slice, head kvh*6 + R%6
+  const int RPB = A.rows_per_block;
+  const int row0 = rb * RPB + wave * 32 * RT;
+  int len[RT]; bool vrow[RT]; size_t pidx[RT];
+  h8 qf[RT][8];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    const int R = row0 + rt * 32 + j;
+    vrow[rt] = R < nrows && R < (rb + 1) * RPB;
+    const int tl = R / kG, head = kvh * kG + R % kG;
+    len[rt] = 0;
+    if (vrow[rt]) { const int tg = A.tok0 + tl; len[rt] = min(pos + (A.depth ? (int)A.depth[tg] : tg) + 1, A.kv.max_ctx); }
+    pidx[rt] = ((size_t)tl * A.S + split) * A.n_heads + head;
+    // B operand of S^T = K Q^T, k-step ks: lane (row j, half h) holds chunk 2ks+h = (group ks/2, sub-chunk 2(ks&1)+h)
+    const uint16_t* qrow = A.q16 + ((size_t)tl * A.n_heads + head) * kD;
+    const _Float16 sx = (_Float16)0.0625f;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      uint4 u = vrow[rt] ? *reinterpret_cast<const uint4*>(qrow + 32 * (ks >> 1) + 8 * (2 * (ks & 1) + h)) : make_uint4(0, 0, 0, 0);
+      const h8 c = __builtin_bit_cast(h8, u);
+      qf[rt][ks] = h8{c[0], c[4], c[1] * sx, c[5] * sx, c[2], c[6], c[3] * sx, c[7] * sx};
+    }
+  }
+  const int nrt = min(RT, max(0, (min(nrows, (rb + 1) * RPB) - row0 + 31) / 32));         // row tiles of this wave that hold rows (wave uniform)
+
+  // key range of the workgroup: its splits cut [0, maxlen) of the block's longest row into 32-key tiles
+  const int tok_lo = (rb * RPB) / kG, tok_hi = min(A.M, (rb * RPB + RPB + kG - 1) / kG);
+  int maxdep = 0, mindep = 0x7fffffff;
+  for (int t = tok_lo; t < tok_hi; ++t) { const int tg = A.tok0 + t; const int dp = A.depth ? (int)A.depth[tg] : tg; maxdep = max(maxdep, dp); mindep = min(mindep, dp); }
+  const int maxlen = min(pos + maxdep + 1, A.kv.max_ctx), minlen = min(pos + mindep + 1, A.kv.max_ctx);
+  const int ntiles = (maxlen + 31) >> 5, tps = (ntiles + A.S - 1) / A.S;
+  const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
+
+  const float sc_log2 = kLog2e / sqrtf((float)kD);
+  float m_run[RT], l_run[RT];                  // m_run in log2 units, shared by the two lanes of a row
+  f16v o[RT][4];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    m_run[rt] = -1e30f; l_run[rt] = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[rt][dt][r] = 0.f;
+  }
+
+  Raw raw;
+  if (tile0 < tile1) {
+    load_raw(kv_page(A.kv, kvh, tile0 << 5), (tile0 << 5) % kPageTok, tid, raw);
+    dequant_to_lds(lds[0], tid, raw);
+    if (tile0 + 1 < tile1) load_raw(kv_page(A.kv, kvh, (tile0 + 1) << 5), ((tile0 + 1) << 5) % kPageTok, tid, raw);
+  }
+  __syncthreads();
+  for (int T = tile0; T < tile1; ++T) {
+    const int cb = (T - tile0) & 1;
+    if (T + 1 < tile1) {
+      dequant_to_lds(lds[cb ^ 1], tid, raw);                          // tile T+1 (loaded one iteration ago)
+      if (T + 2 < tile1) load_raw(kv_page(A.kv, kvh, (T + 2) << 5), ((T + 2) << 5) % kPageTok, tid, raw);
+    }
+    const uint8_t* buf = lds[cb];
+    const int t0 = T << 5;
+    const bool need_mask = t0 + 32 > minlen;
+    if (nrt > 0) {
+      // group scales of the 16 keys whose scores this lane receives: keys 8a + 4h + b, 4 fp16 each
+      uint4 sc[4][2];
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const uint4* sp = reinterpret_cast<const uint4*>(buf + kLdsKs + (8 * a + 4 * h) * 8);
+        sc[a][0] = sp[0]; sc[a][1] = sp[1];
+      }
+      h8 pf[RT][2];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        if (rt < nrt) {
+          // ---- scores: per scale group two chained MFMAs (32 channels), then the fp32 sum times the group scale ----
+          float s[16];
+#pragma unroll
+          for (int m = 0; m < 4; ++m) {
+            const h8 k0 = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsK + j * kKPitch + (4 * m + h) * 16));
+            const h8 k1 = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsK + j * kKPitch + (4 * m + 2 + h) * 16));
+            f16v part;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) part[r] = 0.f;
+            part = __builtin_amdgcn_mfma_f32_32x32x16_f16(k0, qf[rt][2 * m], part, 0, 0, 0);
+            part = __builtin_amdgcn_mfma_f32_32x32x16_f16(k1, qf[rt][2 * m + 1], part, 0, 0, 0);
+            // part[r]: key 8(r/4) + 4h + r%4 of the tile against row j
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int a = r >> 2, b = r & 3;
+              const uint32_t w2 = (&sc[a][b >> 1].x)[2 * (b & 1) + (m >> 1)];   // halfwords 4b+m, 4b+m+1 pair
+              const _Float16 sh = as_h2(w2)[m & 1];
+              s[r] = m == 0 ? part[r] * (float)sh : __builtin_fmaf(part[r], (float)sh, s[r]);
+            }
+          }
+          // ---- online softmax with a lazily raised maximum ----
+          float tmax = -INFINITY;
+          if (need_mask) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int key = t0 + 8 * (r >> 2) + 4 * h + (r & 3);
+              s[r] = key < len[rt] ? s[r] * sc_log2 : -INFINITY;
+            }
+          } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[r] *= sc_log2;
+          }
+#pragma unroll
+          for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[r]);
+          if (__any(tmax > m_run[rt] + kRaise)) {
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+            const float m_new = fmaxf(m_run[rt], tmax);
+            const float alpha = __builtin_amdgcn_exp2f(m_run[rt] - m_new);
+            m_run[rt] = m_new; l_run[rt] *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) o[rt][dt][r] *= alpha;
+          }
+          float lsum = 0.f;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float p = __builtin_amdgcn_exp2f(s[r] - m_run[rt]);
+            lsum += p; pf[rt][r >> 3][r & 7] = (_Float16)p;
+          }
+          l_run[rt] += lsum;
+        }
+      }
+      // ---- O^T += V^T P^T : d-tile dt (32 rows of the V image), k-step u (16 tokens) ----
+#pragma unroll
+      for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          const h8 vf = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsV + (32 * dt + j) * kVPitch + (16 * u + 8 * h) * 2));
+#pragma unroll
+          for (int rt = 0; rt < RT; ++rt)
+            if (rt < nrt) o[rt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[rt][u], o[rt][dt], 0, 0, 0);
+        }
+    }
+    __syncthreads();
+  }
+  // ---- partials: normalised fp16.  o[dt][4a+b] of lane (row j, half h) is V-image row 32dt + 8a + 4h + b, i.e.
+  //      channel 64(a&1) + 32h + 8b + 4(a>>1) + dt: for each (a&1, b) the lane owns 8 consecutive channels ----
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    float l = l_run[rt];
+    l += __shfl_xor(l, 32, 64);
+    if (vrow[rt]) {
+      if (h == 0) { A.pm[pidx[rt]] = m_run[rt]; A.pl[pidx[rt]] = l; }
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      uint16_t* dst = A.pacc16 + pidx[rt] * kD + 32 * h;
+#pragma unroll
+      for (int a0 = 0; a0 < 2; ++a0)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+          h8 v;
+#pragma unroll
+          for (int c = 0; c < 8; ++c) v[c] = (_Float16)(o[rt][c & 3][4 * (2 * (c >> 2) + a0) + b] * inv);
+          *reinterpret_cast<uint4*>(dst + 64 * a0 + 8 * b) = __builtin_bit_cast(uint4, v);
+        }
+    }
+  }
+}
+
+void launch_attend_wide(const AttnArgs& A, hipStream_t st) {
+  const int rows = kG * A.M, rb = (rows + A.rows_per_block - 1) / A.rows_per_block;
+  hipLaunchKernelGGL(attend_wide_kernel<1>, dim3(A.S, A.kv.n_kv, rb), dim3(NT), 0, st, A);
+}
+
+}  // namespace yka

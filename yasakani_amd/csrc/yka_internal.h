@@ -35,16 +35,19 @@ __host__ __device__ inline size_t kv_page_bytes(int n_kv) { return (size_t)n_kv 
 struct AppendArgs { KvView kv; const uint16_t* k16; const uint16_t* v16; const int* d_pos; int M; };
 
 // partial results of the split-KV kernels (same roles as pm/pl/pacc of the reference, args.hpp:10):
-//   pm, pl [rows_tok][S][n_heads]; pacc [rows_tok][S][n_heads][128].  pm is in log2 units; empty split: pm=-1e30, pl=0.
+//   pm, pl [rows_tok][S][n_heads] fp32; pacc16 [rows_tok][S][n_heads][128] fp16 = acc / l (normalised, so that fp16
+//   costs nothing measurable: every split's row is a convex combination of V rows).  pm is in log2 units; empty
+//   split: pm = -1e30, pl = 0, pacc16 = 0.
 struct AttnArgs {
   KvView kv; const uint16_t* q16; const int* d_pos; const uint8_t* depth;
   int M;        // rows (tokens) of this slice
   int tok0;     // index of the slice's first row inside the pass (row t sees keys [0, *d_pos + depth(tok0+t) + 1))
   int n_heads;
   int S;        // splits
-  float* pm; float* pl; float* pacc;
+  int rows_per_block;  // wide kernel: query rows one workgroup owns (multiple of 32)
+  float* pm; float* pl; uint16_t* pacc16;
 };
-struct CombineArgs { const float* pm; const float* pl; const float* pacc; int S; int M; int n_heads; uint16_t* out16; };
+struct CombineArgs { const float* pm; const float* pl; const uint16_t* pacc16; int S; int M; int n_heads; uint16_t* out16; };
 
 // launchers (each checks nothing: the C layer validates shapes first)
 void launch_append(const AppendArgs&, hipStream_t);
