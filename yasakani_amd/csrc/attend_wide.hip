@@ -22,7 +22,9 @@
 //                          dequantize one byte position write 16 consecutive rows, and an output lane ends up with runs
 //                          of 8 consecutive channels.  Inside a row token 16u+8a+4h+b sits at position 16u+8h+4a+b, so
 //                          the 8 tokens an MFMA lane needs are 16 contiguous bytes
-//   Ks [32 keys][4] fp16
+// The K group scales are not staged: every lane needs the scales of 16 keys x 4 groups, the same for all 32 lanes of a
+// wave half, so they come straight from the page's scale plane (L1/L2 resident) one tile ahead, which keeps a third of
+// the fragment traffic off the LDS, the unit this kernel saturates.
 #include "yka_internal.h"
 #include <hip/hip_fp16.h>
 
@@ -40,7 +42,7 @@ __device__ __forceinline__ uint32_t as_u32(h2 h) { return __builtin_bit_cast(uin
 constexpr uint32_t kMagic = 0x64006400u;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kKPitch = 272, kVPitch = 80;
-constexpr int kLdsK = 0, kLdsV = 32 * kKPitch, kLdsKs = kLdsV + 128 * kVPitch, kLdsBuf = kLdsKs + 256;   // 19200
+constexpr int kLdsK = 0, kLdsV = 32 * kKPitch, kLdsBuf = kLdsV + 128 * kVPitch;   // 18944
 constexpr int NT = 256;                        // threads per workgroup
 constexpr float kRaise = 8.f;                  // log2 slack before a running maximum is raised
 
@@ -48,7 +50,6 @@ struct Raw {                                   // one thread's share of a raw 32
   uint32_t kw[2];
   uint32_t vw[2];
   uint32_t vs;
-  uint32_t ks;
 };
 
 __device__ __forceinline__ void load_raw(const uint8_t* pg, int tp, int tid, Raw& R) {
@@ -58,7 +59,6 @@ __device__ __forceinline__ void load_raw(const uint8_t* pg, int tp, int tid, Raw
   const uint32_t* vc = reinterpret_cast<const uint32_t*>(pg + kPageVc + (size_t)(tp + 2 * pair) * 64) + dw;
   R.vw[0] = vc[0]; R.vw[1] = vc[16];
   R.vs = *reinterpret_cast<const uint32_t*>(pg + kPageVs + ((size_t)(dw >> 2) * kPageTok + tp + 2 * pair) * 2);
-  if (tid < 64) R.ks = reinterpret_cast<const uint32_t*>(pg + kPageKs + (size_t)tp * 8)[tid];
 }
 
 __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw& R) {
@@ -92,7 +92,16 @@ __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw&
       *reinterpret_cast<uint32_t*>(vb + 16 * (2 * (c1 & 3) + (c1 >> 2)) * kVPitch) = as_u32(hi);
     }
   }
-  if (tid < 64) reinterpret_cast<uint32_t*>(buf + kLdsKs)[tid] = R.ks;
+}
+
+// group scales of the 16 keys whose scores a lane of half h receives: keys 8a + 4h + b of the tile, 4 fp16 each
+struct KScales { uint4 v[4][2]; };
+__device__ __forceinline__ void load_kscales(const uint8_t* pg, int tp, int h, KScales& K) {
+#pragma unroll
+  for (int a = 0; a < 4; ++a) {
+    const uint4* sp = reinterpret_cast<const uint4*>(pg + kPageKs + (size_t)(tp + 8 * a + 4 * h) * 8);
+    K.v[a][0] = sp[0]; K.v[a][1] = sp[1];
+  }
 }
 
 }  // namespace
@@ -152,8 +161,10 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
   }
 
   Raw raw;
+  KScales sc;
   if (tile0 < tile1) {
     load_raw(kv_page(A.kv, kvh, tile0 << 5), (tile0 << 5) % kPageTok, tid, raw);
+    load_kscales(kv_page(A.kv, kvh, tile0 << 5), (tile0 << 5) % kPageTok, h, sc);
     dequant_to_lds(lds[0], tid, raw);
     if (tile0 + 1 < tile1) load_raw(kv_page(A.kv, kvh, (tile0 + 1) << 5), ((tile0 + 1) << 5) % kPageTok, tid, raw);
   }
@@ -168,13 +179,6 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
     const int t0 = T << 5;
     const bool need_mask = t0 + 32 > minlen;
     if (nrt > 0) {
-      // group scales of the 16 keys whose scores this lane receives: keys 8a + 4h + b, 4 fp16 each
-      uint4 sc[4][2];
-#pragma unroll
-      for (int a = 0; a < 4; ++a) {
-        const uint4* sp = reinterpret_cast<const uint4*>(buf + kLdsKs + (8 * a + 4 * h) * 8);
-        sc[a][0] = sp[0]; sc[a][1] = sp[1];
-      }
       h8 pf[RT][2];
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
@@ -194,7 +198,7 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
               const int a = r >> 2, b = r & 3;
-              const uint32_t w2 = (&sc[a][b >> 1].x)[2 * (b & 1) + (m >> 1)];   // halfwords 4b+m, 4b+m+1 pair
+              const uint32_t w2 = (&sc.v[a][b >> 1].x)[2 * (b & 1) + (m >> 1)];   // halfwords 4b+m, 4b+m+1 pair
               const _Float16 sh = as_h2(w2)[m & 1];
               s[r] = m == 0 ? part[r] * (float)sh : __builtin_fmaf(part[r], (float)sh, s[r]);
             }
@@ -232,6 +236,8 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
           l_run[rt] += lsum;
         }
       }
+      // scales of the next tile: requested now, needed after the next barrier
+      if (T + 1 < tile1) load_kscales(kv_page(A.kv, kvh, (T + 1) << 5), ((T + 1) << 5) % kPageTok, h, sc);
       // ---- O^T += V^T P^T : d-tile dt (32 rows of the V image), k-step u (16 tokens) ----
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
