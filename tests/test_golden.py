@@ -1,0 +1,64 @@
+"""Committed fixtures (tests/golden/*.npz, written by tests/golden/make_golden.py from the pinned oracle).
+
+CPU part: the oracle still reproduces them bit for bit.  GPU part: the HIP path reproduces the codec fixture bit for
+bit and the attention fixtures within the attention bar, without running the oracle.
+"""
+import os
+
+import numpy as np
+import pytest
+
+from tests.tolerances import assert_attn_close
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+CASES = ("decode_ctx100", "window5_ctx70", "window6_depth")
+
+
+def _load(name):
+    return np.load(os.path.join(GOLD, name), allow_pickle=False)
+
+
+def test_oracle_reproduces_codec_fixture(oracle):
+    g = _load("codec_v1.npz")
+    codes, scales = oracle.quant_rows(g["x16"].view(np.float16))
+    assert (codes == g["codes"]).all() and (scales == g["scales"]).all()
+    assert (oracle.dequant_rows(codes, scales).view(np.uint32) == g["dequant_bits"]).all()
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_oracle_reproduces_attention_fixture(oracle, case):
+    g = _load("attention_v1.npz")
+    ctx = int(g[f"{case}.ctx"]); q = g[f"{case}.q"].view(np.float16); M = q.shape[0]
+    c = oracle.Cache(512)
+    n = ctx + M
+    c.kc[:, :n], c.ks[:, :n], c.vc[:, :n], c.vs[:, :n] = g[f"{case}.kc"], g[f"{case}.ks"], g[f"{case}.vc"], g[f"{case}.vs"]
+    dep = g[f"{case}.depth"]; dep = dep if dep.size else None
+    o16 = c.attend_f32(q, ctx, dep)
+    assert (o16.view(np.uint16) == g[f"{case}.out16"]).all()
+    # the appended rows of the fixture are what quantizing k_new / v_new gives
+    c2 = oracle.Cache(512)
+    c2.append(g[f"{case}.k_new"].view(np.float16), g[f"{case}.v_new"].view(np.float16), ctx)
+    assert (c2.kc[:, ctx:n] == g[f"{case}.kc"][:, ctx:n]).all() and (c2.vs[:, ctx:n] == g[f"{case}.vs"][:, ctx:n]).all()
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_codec_fixture(native):
+    g = _load("codec_v1.npz")
+    codes, scales, y = native.codec_probe(g["x16"].view(np.float16))
+    assert (codes == g["codes"]).all() and (scales == g["scales"]).all()
+    assert (y.view(np.uint32) == g["dequant_bits"]).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", CASES)
+def test_gpu_reproduces_attention_fixture(native, case):
+    g = _load("attention_v1.npz")
+    ctx = int(g[f"{case}.ctx"]); q = g[f"{case}.q"].view(np.float16); M = q.shape[0]
+    dep = g[f"{case}.depth"]; dep = dep if dep.size else None
+    with native.KvCache(max_ctx=512) as kv:
+        kv.import_rows(0, 0, g[f"{case}.kc"][:, :ctx], g[f"{case}.ks"][:, :ctx], g[f"{case}.vc"][:, :ctx], g[f"{case}.vs"][:, :ctx])
+        out = kv.layer_call(0, q, g[f"{case}.k_new"].view(np.float16), g[f"{case}.v_new"].view(np.float16), ctx, depth=dep)
+        got = kv.export_rows(0, ctx, M)
+    assert (got[0] == g[f"{case}.kc"][:, ctx:]).all() and (got[1] == g[f"{case}.ks"][:, ctx:]).all()
+    assert (got[2] == g[f"{case}.vc"][:, ctx:]).all() and (got[3] == g[f"{case}.vs"][:, ctx:]).all()
+    assert_attn_close(out, g[f"{case}.out32"], case)
