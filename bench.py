@@ -91,6 +91,39 @@ def timed_passes(torch, kv, layers, q, kn, vn, ctx, M, steps, warmup):
     return dt, out
 
 
+def big_configs(native):
+    """Secondary figures for the two large configurations: a 2048-row prefill chunk on 131072 cached tokens (cut into
+    64-row slices inside the library) and decode / verify-64 on 262144 tokens in shuffled 256-token pages."""
+    out = {}
+    # chunked prefill: 4 containers x 76.7 MB
+    ctx, M, L = 131072, 2048, 4
+    q, k, v = synth(31, ctx, M)
+    kv = native.KvCache(n_layers=L, max_ctx=ctx + M, max_rows=M)
+    fill_cache(kv, k, v, ctx, chunk=16384)
+    ms, _ = kv.bench(q, k[ctx:], v[ctx:], ctx, mode=0, use_graph=True, reps=5)
+    us = float(np.median(ms)) * 1e3 / L
+    keys = sum(ctx + t + 1 for t in range(M))
+    fl = 4.0 * NH * D * keys
+    out["prefill_2048_at_131072"] = {"us_per_layer": us, "tflops": fl / (us * 1e-6) / 1e12,
+                                     "mfma_peak_frac": fl / (us * 1e-6) / 1e12 / MFMA_F16_PEAK_TFLOPS}
+    kv.close()
+    # 262144 tokens, shuffled pages: 3 containers x 151 MB
+    ctx, L = 262144, 3
+    q, k, v = synth(32, ctx, 64)
+    kv = native.KvCache(n_layers=L, max_ctx=ctx + 256, max_rows=64, paged=True)
+    kv.set_page_table(np.random.default_rng(32).permutation((ctx + 256) // 256).astype(np.int32))
+    fill_cache(kv, k, v, ctx, chunk=16384)
+    for rows in (1, 64):
+        ms, _ = kv.bench(q[:rows], k[ctx:ctx + rows], v[ctx:ctx + rows], ctx, mode=0, use_graph=True, reps=10)
+        us = float(np.median(ms)) * 1e3 / L
+        by = algorithmic_bytes(ctx, rows)
+        out[f"paged_262144_rows_{rows}"] = {"us_per_layer": us, "value_GBs": by / (us * 1e-6) / 1e9,
+                                            "hbm_peak_frac": by / (us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                                            "tflops": algorithmic_flops(ctx, rows) / (us * 1e-6) / 1e12}
+    kv.close()
+    return out
+
+
 def cpu_baseline(kv, q, ctx, M, budget_s=20.0):
     """The CPU oracle (threaded port of the reference's token-streaming split-KV loop) on the same quantized cache.
     Bounded sample: whole layer calls are repeated until about `budget_s` seconds of CPU work are spent."""
@@ -183,6 +216,8 @@ def main():
         a, b = out.astype(np.float64), ref16.astype(np.float64)
         line["parity_vs_cpu"] = {"max_abs": float(np.abs(a - b).max()), "rel_l2": float(np.linalg.norm(a - b) / np.linalg.norm(b))}
     kv.close()
+    if not args.no_extra:
+        line["other_configs"] = big_configs(native)
     print(json.dumps(line))
 
 

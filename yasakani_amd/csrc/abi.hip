@@ -85,15 +85,19 @@ void do_append(yka_kv* kv, int layer, const uint16_t* k16, const uint16_t* v16, 
   launch_append(AppendArgs{kv->view(layer), k16, v16, d_pos, M}, st);
 }
 
-// mode 0: attention + combine; 2: attention kernel alone
+// mode 0: attention + combine; 2: attention kernel alone.  k16/v16 != nullptr asks for quantize-on-append as well:
+// rows of at most 2 tokens fuse it into the attention launch, wider passes launch the append kernel first.
 void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_pos, const uint8_t* depth, uint16_t* out16,
-               hipStream_t st, int mode = 0) {
+               hipStream_t st, int mode = 0, const uint16_t* k16 = nullptr, const uint16_t* v16 = nullptr) {
   const int NH = kv->cfg.n_heads;
+  const bool fuse_append = k16 && M <= 2;
+  if (k16 && !fuse_append) do_append(kv, layer, k16, v16, M, d_pos, st);
   for (int s0 = 0; s0 < M; s0 += kMaxSlice) {   // 64-row slices, as attn_block cuts wide passes (engine35.cpp:935-947)
     const int Ms = std::min(kMaxSlice, M - s0);
     const bool narrow = Ms <= 2 || kv->opt_force_narrow;
     const int S = narrow ? narrow_splits(kv, Ms) : wide_splits(kv, Ms);
-    AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * kD, d_pos, depth, Ms, s0, NH, S, wide_rows_per_block(Ms), kv->pm, kv->pl, kv->pacc16};
+    AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * kD, d_pos, depth, Ms, s0, NH, S, wide_rows_per_block(Ms), kv->pm, kv->pl, kv->pacc16,
+               fuse_append ? k16 : nullptr, fuse_append ? v16 : nullptr};
     if (narrow) launch_attend_narrow(A, st); else launch_attend_wide(A, st);
     if (mode != 2) launch_combine(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD}, st);
   }
@@ -224,8 +228,7 @@ int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16
   YKA_TRY
   on_device(kv); check_layer(kv, layer); check_rows(kv, M);
   if (!d_q16 || !d_k16 || !d_v16 || !d_pos || !d_out16) throw std::runtime_error("null pointer");
-  do_append(kv, layer, d_k16, d_v16, M, d_pos, (hipStream_t)hip_stream);
-  do_attend(kv, layer, d_q16, M, d_pos, d_depth, d_out16, (hipStream_t)hip_stream);
+  do_attend(kv, layer, d_q16, M, d_pos, d_depth, d_out16, (hipStream_t)hip_stream, 0, d_k16, d_v16);
   HIPCHK(hipGetLastError());
   YKA_CATCH_INT
 }
@@ -325,8 +328,8 @@ int yka_layer_call_host(yka_kv* kv, int layer, const uint16_t* q16, const uint16
   if (depth) HIPCHK(hipMemcpy(dd.p, depth, (size_t)M, hipMemcpyHostToDevice));
   HIPCHK(hipDeviceSynchronize());
   launch_set_int(kv->d_pos, pos, st);
-  if (k16) do_append(kv, layer, dk.as<uint16_t>(), dv.as<uint16_t>(), M, kv->d_pos, st);
-  do_attend(kv, layer, dq.as<uint16_t>(), M, kv->d_pos, depth ? dd.as<uint8_t>() : nullptr, dout.as<uint16_t>(), st);
+  do_attend(kv, layer, dq.as<uint16_t>(), M, kv->d_pos, depth ? dd.as<uint8_t>() : nullptr, dout.as<uint16_t>(), st, 0,
+            k16 ? dk.as<uint16_t>() : nullptr, k16 ? dv.as<uint16_t>() : nullptr);
   HIPCHK(hipGetLastError());
   HIPCHK(hipStreamSynchronize(st));
   HIPCHK(hipMemcpy(out16, dout.p, nq * 2, hipMemcpyDeviceToHost));
@@ -367,8 +370,7 @@ yka_pass* yka_pass_capture(yka_kv* kv, const int32_t* layers, int n, const uint1
     HIPCHK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
     capturing = true;
     for (int i = 0; i < n; ++i) {
-      if (mode == 0) do_append(kv, layers[i], d_k16, d_v16, M, d_pos, st);
-      do_attend(kv, layers[i], d_q16, M, d_pos, d_depth, d_out16, st, mode == 2 ? 2 : 0);
+      do_attend(kv, layers[i], d_q16, M, d_pos, d_depth, d_out16, st, mode == 2 ? 2 : 0, mode == 0 ? d_k16 : nullptr, mode == 0 ? d_v16 : nullptr);
     }
     capturing = false;
     HIPCHK(hipStreamEndCapture(st, &p->graph));
@@ -416,8 +418,8 @@ int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const u
     launch_set_int(kv->d_pos, pos, st);
     auto sweep = [&]() {
       for (int l = 0; l < kv->cfg.n_layers; ++l) {
-        if (mode == 0) do_append(kv, l, dk.as<uint16_t>(), dv.as<uint16_t>(), M, kv->d_pos, st);
-        do_attend(kv, l, dq.as<uint16_t>(), M, kv->d_pos, nullptr, dout.as<uint16_t>(), st, mode == 2 ? 2 : 0);
+        do_attend(kv, l, dq.as<uint16_t>(), M, kv->d_pos, nullptr, dout.as<uint16_t>(), st, mode == 2 ? 2 : 0,
+                  mode == 0 ? dk.as<uint16_t>() : nullptr, mode == 0 ? dv.as<uint16_t>() : nullptr);
       }
     };
     if (use_graph) {

@@ -16,9 +16,12 @@
 //     channels, most of the 1e-3 budget).  V is scaled in fp16 (one rounding, 2e-4);
 //   * scores S^T = K Q^T come out of the MFMA with one query row per lane column, which is already the B-operand
 //     layout of O^T += V^T P^T: probabilities never move between lanes;
-//   * running maxima are shared by the 4 lane groups of a row through two cross-lane exchanges per tile.
-#include "yka_internal.h"
-#include <hip/hip_fp16.h>
+//   * running maxima are shared by the 4 lane groups of a row through two cross-lane exchanges per tile;
+//   * quantize-on-append is fused into the decode launch (a launch costs about 2.5 us here, the same order as the
+//     whole KV stream): the workgroup whose tiles contain a row appended by this pass quantizes and stores that row
+//     before it loads the tile.  The split merge stays a second launch: the 8 XCDs keep separate L2s, so merging in
+//     the last workgroup needs a device-scope release (an L2 write-back) in every workgroup, measured 4x slower.
+#include "codec_device.h"
 
 namespace yka {
 
@@ -85,6 +88,27 @@ __global__ void __launch_bounds__(256) attend_narrow_kernel(AttnArgs A) {
   for (int o = 1; o < 16; o <<= 1) maxlen = max(maxlen, __shfl_xor(maxlen, o, 64));
   const int ntiles = (maxlen + 31) >> 5, tps = (ntiles + A.S - 1) / A.S;
   const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
+
+  // ---- fused quantize-on-append (decode, M <= 2, one row tile): a row of this pass is written by the one workgroup
+  //      whose tile range holds it - the only workgroup of this kv head that will read it in this launch.  Writer and
+  //      readers are waves of one workgroup, i.e. of one CU and one (write-through) L1, so workgroup-scope fences
+  //      around the barrier order the stores before the loads without any cache maintenance. ----
+  if (A.k16) {
+    bool mine = false;
+    for (int t = 0; t < A.M; ++t) {
+      const int r = pos + t;
+      if (r < 0 || r >= A.kv.max_ctx || (r >> 5) < tile0 || (r >> 5) >= tile1) continue;
+      mine = true;
+      const bool isv = threadIdx.x >= 128;
+      const uint16_t* src = (isv ? A.v16 : A.k16) + ((size_t)t * A.kv.n_kv + kvh) * kD;
+      quant_store_row(A.kv, kvh, r, isv, src, threadIdx.x & 127);
+    }
+    if (mine) {                      // uniform over the workgroup
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __syncthreads();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    }
+  }
 
   // Q fragments: B operand of S^T = K Q^T.  MFMA step m (= scale group m), lane (row i, lane group g), element e
   // <-> channel 32m + 8g + pi(e), pi = [0,4,1,5,2,6,3,7] (the order dq_dword_int produces); odd channels carry 1/16.

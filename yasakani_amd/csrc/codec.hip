@@ -1,31 +1,9 @@
 // Quantize-on-append and the codec probes.  Compiled with -ffp-contract=off: the codec is bit-exact by contract,
 // and the reference builds with --fmad=false (CMakeLists.txt:60-63).
-//
-// Arithmetic per 32-channel group (reference: src/kvq_fast.cuh:194-198, src/kvq_gpu.cuh:85-86):
-//   am = max|x|; s = fp16(am / 7); if (s == 0) s = 1; q = clamp(rint(x / s), -7, 7); stored nibble = q + 8.
-// The division is by the stored (fp16-rounded) scale, as the reference divides by the scale it stores.
-#include "yka_internal.h"
-#include <hip/hip_fp16.h>
+// The quantizer itself lives in codec_device.h (shared with the fused decode kernel).
+#include "codec_device.h"
 
 namespace yka {
-
-__device__ __forceinline__ float h2f_bits(uint16_t b) { return __half2float(__ushort_as_half(b)); }
-// physical byte of a K row that holds logical byte j (channels 2j, 2j+1)
-__device__ __forceinline__ int k_code_byte(int j) { return 4 * k_phys_dword(j >> 2) + (j & 3); }
-
-// one lane = one channel; lanes of a 32-lane half-wave form one scale group
-__device__ __forceinline__ void quant_lane(float x, int& code, uint16_t& s16) {
-  float am = fabsf(x);
-#pragma unroll
-  for (int o = 16; o; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, 32));
-  const float s32 = __fdiv_rn(am, 7.0f);
-  s16 = __half_as_ushort(__float2half_rn(s32));
-  if ((s16 & 0x7fffu) == 0) s16 = 0x3c00u;
-  const float sd = h2f_bits(s16);
-  float q = rintf(__fdiv_rn(x, sd));
-  q = fminf(fmaxf(q, -7.f), 7.f);
-  code = (int)q + 8;
-}
 
 // grid (M, n_kv * 2), block 128: blockIdx.y = kvh * 2 + (0: K, 1: V); thread = channel.
 // Rows land at *d_pos + tok (reference: q35_kernels.cu:1038,1064 write the pass's rows before attention reads them).
@@ -34,21 +12,7 @@ __global__ void __launch_bounds__(128) append_kernel(AppendArgs A) {
   const int pos = *A.d_pos + tok;
   if (pos < 0 || pos >= A.kv.max_ctx) return;
   const uint16_t* src = (isv ? A.v16 : A.k16) + ((size_t)tok * A.kv.n_kv + kvh) * kD;
-  const float x = h2f_bits(src[d]);
-  int code; uint16_t s16;
-  quant_lane(x, code, s16);
-  const int nb = __shfl_xor(code, 1, 64);
-  uint8_t* pg = kv_page(A.kv, kvh, pos);
-  const int tp = pos % kPageTok;
-  if ((d & 1) == 0) {
-    const uint8_t byte = (uint8_t)((code & 15) | ((nb & 15) << 4));
-    if (isv) pg[kPageVc + tp * 64 + (d >> 1)] = byte;
-    else pg[kPageKc + tp * 64 + k_code_byte(d >> 1)] = byte;
-  }
-  if ((d & 31) == 0) {
-    if (isv) reinterpret_cast<uint16_t*>(pg + kPageVs)[(d >> 5) * kPageTok + tp] = s16;
-    else reinterpret_cast<uint16_t*>(pg + kPageKs)[tp * kNG + (d >> 5)] = s16;
-  }
+  quant_store_row(A.kv, kvh, pos, isv != 0, src, d);
 }
 void launch_append(const AppendArgs& A, hipStream_t st) {
   hipLaunchKernelGGL(append_kernel, dim3(A.M, A.kv.n_kv * 2), dim3(128), 0, st, A);

@@ -46,6 +46,9 @@ struct AttnArgs {
   int S;        // splits
   int rows_per_block;  // wide kernel: query rows one workgroup owns (multiple of 32)
   float* pm; float* pl; uint16_t* pacc16;
+  // narrow kernel only.  k16/v16 != nullptr (M <= 2): the workgroup whose tiles hold a new row quantizes and stores it
+  // before reading it (fused quantize-on-append).
+  const uint16_t* k16; const uint16_t* v16;
 };
 struct CombineArgs { const float* pm; const float* pl; const uint16_t* pacc16; int S; int M; int n_heads; uint16_t* out16; };
 
