@@ -47,7 +47,7 @@ YKA_API const char* yka_last_error(void);
 /* replaces yskn_build_info (yskn_abi.h:84): "hip=<version>;arch=gfx950;..." */
 YKA_API const char* yka_build_info(void);
 /* replaces yskn_set_opt (yskn_abi.h:87) for the options of this path.
- * key 1: split count of the narrow kernel (decode, rows of at most 2 tokens); key 2: split count of the wide kernel;
+ * key 1: split count of the narrow kernel (decode, rows of at most 2 tokens; at most 256); key 2: split count of the wide kernel;
  * key 3: 1 forces the narrow kernel for every width (cross-check of the wide kernel), 0 = automatic. */
 YKA_API int yka_set_opt(yka_kv* kv, int key, int value);
 

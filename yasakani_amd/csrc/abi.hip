@@ -52,14 +52,14 @@ void on_device(const yka_kv* kv) {
   HIPCHK(hipSetDevice(kv->cfg.device));
 }
 
-constexpr int kMaxSplits = 128;
+constexpr int kMaxSplits = 256;
 constexpr size_t kWsPairs = 4096;  // (token, split) pairs the partial workspace holds: 4096 * 24 * (256 + 8) bytes = 26 MB
 
-// splits for the narrow kernel: enough workgroups (n_kv * S * ceil(M/2)) to cover 256 CUs about twice over
+// splits for the narrow kernel: enough workgroups (n_kv * S * ceil(M/2)) to put 4 waves on every SIMD of 256 CUs
 int narrow_splits(const yka_kv* kv, int M) {
   if (kv->opt_splits_narrow > 0) return std::min(kv->opt_splits_narrow, (int)(kWsPairs / (size_t)M));
   const int tiles = (M + 1) / 2;
-  int S = 512 / (kv->cfg.n_kv_heads * tiles);
+  int S = 1024 / (kv->cfg.n_kv_heads * tiles);
   S = std::max(2, std::min(kMaxSplits, S));
   return std::min(S, (int)(kWsPairs / (size_t)M));
 }
@@ -179,8 +179,8 @@ int yka_set_opt(yka_kv* kv, int key, int value) {
   YKA_TRY
   if (!kv) throw std::runtime_error("null handle");
   switch (key) {
-    case 1: if (value < 0 || value > kMaxSplits) throw std::runtime_error("splits must be in [0, 128]"); kv->opt_splits_narrow = value; break;
-    case 2: if (value < 0 || value > kMaxSplits) throw std::runtime_error("splits must be in [0, 128]"); kv->opt_splits_wide = value; break;
+    case 1: if (value < 0 || value > kMaxSplits) throw std::runtime_error("splits must be in [0, 256]"); kv->opt_splits_narrow = value; break;
+    case 2: if (value < 0 || value > kMaxSplits) throw std::runtime_error("splits must be in [0, 256]"); kv->opt_splits_wide = value; break;
     case 3: kv->opt_force_narrow = value != 0; break;
     default: throw std::runtime_error("unknown option key");
   }

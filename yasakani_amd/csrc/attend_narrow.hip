@@ -17,6 +17,8 @@
 //   * scores S^T = K Q^T come out of the MFMA with one query row per lane column, which is already the B-operand
 //     layout of O^T += V^T P^T: probabilities never move between lanes;
 //   * running maxima are shared by the 4 lane groups of a row through two cross-lane exchanges per tile;
+//   * the kernel stays at 128 registers so that 4 waves share a SIMD (16 per CU): with one 32-key tile in flight per
+//     wave that is the memory-level parallelism the HBM stream needs; raw tiles are not double buffered in registers;
 //   * quantize-on-append is fused into the decode launch (a launch costs about 2.5 us here, the same order as the
 //     whole KV stream): the workgroup whose tiles contain a row appended by this pass quantizes and stores that row
 //     before it loads the tile.  The split merge stays a second launch: the 8 XCDs keep separate L2s, so merging in
@@ -70,7 +72,7 @@ __device__ __forceinline__ void load_tile(const uint8_t* pg, int tp, int i, int 
 }
 
 // grid (S, n_kv, ceil(M/2)), block 256 (4 waves).  Workgroup = (split, kv head, row tile of 2 tokens x 6 heads).
-__global__ void __launch_bounds__(256) attend_narrow_kernel(AttnArgs A) {
+__global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
   __shared__ float s_m[4][16], s_l[4][16];
   __shared__ float s_acc[4][16][kD + 4];
   const int split = blockIdx.x, kvh = blockIdx.y, rt = blockIdx.z;
@@ -130,11 +132,9 @@ __global__ void __launch_bounds__(256) attend_narrow_kernel(AttnArgs A) {
 #pragma unroll
   for (int b = 0; b < 8; ++b) o[b] = f4{0.f, 0.f, 0.f, 0.f};
 
-  RawTile cur, nxt;
-  int T = tile0 + wave;
-  if (T < tile1) load_tile(kv_page(A.kv, kvh, T << 5), (T << 5) % kPageTok, i, g, cur);
-  for (; T < tile1; T += 4) {
-    if (T + 4 < tile1) load_tile(kv_page(A.kv, kvh, (T + 4) << 5), ((T + 4) << 5) % kPageTok, i, g, nxt);
+  RawTile cur;
+  for (int T = tile0 + wave; T < tile1; T += 4) {
+    load_tile(kv_page(A.kv, kvh, T << 5), (T << 5) % kPageTok, i, g, cur);
     const int t0 = T << 5;
     // ---- scores: two 16-key MFMA tiles; step m contracts scale group m, its fp32 sum is scaled afterwards ----
     float s[8];
@@ -198,7 +198,6 @@ __global__ void __launch_bounds__(256) attend_narrow_kernel(AttnArgs A) {
       const h8 vf = h8{va[b][0][0], va[b][0][1], va[b][1][0], va[b][1][1], va[b][2][0], va[b][2][1], va[b][3][0], va[b][3][1]};
       o[b] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[b], 0, 0, 0);
     }
-    cur = nxt;
   }
   // ---- merge the 4 waves of the workgroup, write one partial per (row, split) ----
   l_run += __shfl_xor(l_run, 16, 64);
@@ -230,9 +229,9 @@ void launch_attend_narrow(const AttnArgs& A, hipStream_t st) {
 
 // combiner (reference: src/attention_kv4q.cu:325-332): M2 = max pm; w_s = pm_s > -1e29 ? 2^(pm_s - M2) * pl_s : 0;
 // y = sum w_s * (acc_s / l_s) / sum w_s.  grid (n_heads, M), block 256: 16 lanes x 8 channels cover a row, 16 split
-// lanes run in parallel and are summed through LDS.
+// lanes run in parallel and are summed through LDS.  S <= 256.
 __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
-  __shared__ float s_w[128];
+  __shared__ float s_w[256];
   __shared__ float s_o[16][kD + 4];
   __shared__ float s_wsum[16];
   const int head = blockIdx.x, tok = blockIdx.y, tid = threadIdx.x;
@@ -243,21 +242,32 @@ __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
   float M2 = pmv;
 #pragma unroll
   for (int o = 32; o; o >>= 1) M2 = fmaxf(M2, __shfl_xor(M2, o, 64));
-  if (tid < 128 && (tid & 63) == 0) s_wsum[tid >> 6] = M2;
+  if ((tid & 63) == 0) s_wsum[tid >> 6] = M2;
   __syncthreads();
-  M2 = fmaxf(s_wsum[0], s_wsum[1]);
-  if (tid < 128) s_w[tid] = (tid < A.S && pmv > -1e29f) ? exp2f(pmv - M2) * plv : 0.f;
+  M2 = fmaxf(fmaxf(s_wsum[0], s_wsum[1]), fmaxf(s_wsum[2], s_wsum[3]));
+  s_w[tid] = (tid < A.S && pmv > -1e29f) ? exp2f(pmv - M2) * plv : 0.f;
   __syncthreads();
   const int sl = tid >> 4, c8 = (tid & 15) * 8;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float wsum = 0.f;
-  for (int s = sl; s < A.S; s += 16) {
-    const float w = s_w[s];
-    const uint4 u = *reinterpret_cast<const uint4*>(A.pacc16 + (p0 + (size_t)s * A.n_heads) * kD + c8);
-    const h8 v = __builtin_bit_cast(h8, u);
+  // 16 split lanes; each takes splits sl, sl+16, ...; loads are issued 4 at a time so that their latencies overlap
+  const uint16_t* src = A.pacc16 + p0 * kD + c8;
+  const size_t stride = (size_t)A.n_heads * kD;
+  for (int s0 = sl; s0 < A.S; s0 += 64) {
+    uint4 u[4]; float w[4];
 #pragma unroll
-    for (int c = 0; c < 8; ++c) acc[c] += w * (float)v[c];
-    wsum += w;
+    for (int k = 0; k < 4; ++k) {
+      const int sp = s0 + 16 * k;
+      w[k] = sp < A.S ? s_w[sp] : 0.f;
+      u[k] = sp < A.S ? *reinterpret_cast<const uint4*>(src + (size_t)sp * stride) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const h8 v = __builtin_bit_cast(h8, u[k]);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) acc[c] += w[k] * (float)v[c];
+      wsum += w[k];
+    }
   }
 #pragma unroll
   for (int c = 0; c < 8; ++c) s_o[sl][c8 + c] = acc[c];
