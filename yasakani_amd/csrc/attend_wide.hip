@@ -15,7 +15,7 @@
 //   * the running maximum of a row is only raised when a score exceeds it by more than 2^8: accumulators stay in
 //     their registers untouched on almost every tile;
 //   * LDS is double buffered: tile n+1 is dequantized while tile n is consumed; one barrier per tile.
-// LDS image of one tile (19200 bytes):
+// LDS image of one tile (18944 bytes):
 //   K  [32 keys][272 B]   chunk 4m+g of a key = channels 32m+8g..+7 in the order n0,n4,n1,n5,n2,n6,n3,n7; the 272-byte
 //                          pitch makes the lanes of a fragment read hit distinct banks
 //   V  [128 rows][80 B]   channel 8*dw+c lives in row 16*sigma(c)+dw, sigma(c) = 2*(c&3) + (c>>2): the 16 lanes that
@@ -23,8 +23,8 @@
 //                          of 8 consecutive channels.  Inside a row token 16u+8a+4h+b sits at position 16u+8h+4a+b, so
 //                          the 8 tokens an MFMA lane needs are 16 contiguous bytes
 // The K group scales are not staged: every lane needs the scales of 16 keys x 4 groups, the same for all 32 lanes of a
-// wave half, so they come straight from the page's scale plane (L1/L2 resident) one tile ahead, which keeps a third of
-// the fragment traffic off the LDS, the unit this kernel saturates.
+// wave half, so they come straight from the page's scale plane (L1/L2 resident) one tile ahead and stay in registers.
+// Partial results leave through the same LDS after the last tile so that every store writes whole 256-byte rows.
 #include "yka_internal.h"
 #include <hip/hip_fp16.h>
 
@@ -252,24 +252,39 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
     __syncthreads();
   }
   // ---- partials: normalised fp16.  o[dt][4a+b] of lane (row j, half h) is V-image row 32dt + 8a + 4h + b, i.e.
-  //      channel 64(a&1) + 32h + 8b + 4(a>>1) + dt: for each (a&1, b) the lane owns 8 consecutive channels ----
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    float l = l_run[rt];
+  //      channel 64(a&1) + 32h + 8b + 4(a>>1) + dt: for each (a&1, b) the lane owns 8 consecutive channels.
+  //      Rows go through LDS (the tile buffers are free after the last barrier) so that every store instruction
+  //      writes whole 256-byte rows: 16 lanes per row instead of 64 scattered 16-byte pieces. ----
+  static_assert(RT == 1, "the staging below holds one 32-row tile per wave");
+  constexpr int kOPitch = 2 * kD + 16;                       // bytes per staged row
+  uint8_t* stage = &lds[0][0] + wave * 32 * kOPitch;         // 4 waves x 8704 bytes
+  {
+    float l = l_run[0];
     l += __shfl_xor(l, 32, 64);
-    if (vrow[rt]) {
-      if (h == 0) { A.pm[pidx[rt]] = m_run[rt]; A.pl[pidx[rt]] = l; }
-      const float inv = l > 0.f ? 1.f / l : 0.f;
-      uint16_t* dst = A.pacc16 + pidx[rt] * kD + 32 * h;
+    if (vrow[0] && h == 0) { A.pm[pidx[0]] = m_run[0]; A.pl[pidx[0]] = l; }
+    const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
-      for (int a0 = 0; a0 < 2; ++a0)
+    for (int a0 = 0; a0 < 2; ++a0)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
-          h8 v;
+      for (int b = 0; b < 4; ++b) {
+        h8 v;
 #pragma unroll
-          for (int c = 0; c < 8; ++c) v[c] = (_Float16)(o[rt][c & 3][4 * (2 * (c >> 2) + a0) + b] * inv);
-          *reinterpret_cast<uint4*>(dst + 64 * a0 + 8 * b) = __builtin_bit_cast(uint4, v);
-        }
+        for (int c = 0; c < 8; ++c) v[c] = (_Float16)(o[0][c & 3][4 * (2 * (c >> 2) + a0) + b] * inv);
+        *reinterpret_cast<uint4*>(stage + j * kOPitch + (64 * a0 + 32 * h + 8 * b) * 2) = __builtin_bit_cast(uint4, v);
+      }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");     // the wave reads back what its own lanes wrote
+  {
+    const int chunk = lane & 15;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      const int jr = 4 * k + (lane >> 4);
+      const int R = row0 + jr;
+      if (R < nrows && R < (rb + 1) * RPB) {
+        const size_t p = ((size_t)(R / kG) * A.S + split) * A.n_heads + kvh * kG + R % kG;
+        const uint4 v = *reinterpret_cast<const uint4*>(stage + jr * kOPitch + chunk * 16);
+        *reinterpret_cast<uint4*>(A.pacc16 + p * kD + chunk * 8) = v;
+      }
     }
   }
 }
