@@ -26,6 +26,10 @@ NH, KVH, D = 24, 4, 128
 TOKEN_BYTES = KVH * 2 * (D // 2 + 2 * (D // 32))      # 576 B per cached token per layer (codes + fp16 group scales)
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
+# HBM bytes per launch of the dominant kernel from two `rocprofv3 --pmc` runs (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00,
+# factors from a 256 MiB copy in the same runs; see profiles/attend_*_ctx32768.md).  Keyed by (rows, ctx, containers
+# irrelevant); any other workload reports null.
+MEASURED_TRAFFIC_BYTES = {(64, 32768): 39.8e6, (1, 32768): 20.9e6}
 
 
 def algorithmic_bytes(ctx, M):
@@ -155,6 +159,8 @@ def main():
     ap.add_argument("--rows", type=int, default=64, help="query rows of the window (64 = headline; 1 = decode)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary decode / verify-16 / verify-32 lines")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three device-to-device copies of 256 MiB (a kernel of known traffic, for scaling FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU (one process, one device); --gpus above 1 is not supported")
@@ -185,7 +191,7 @@ def main():
         else:
             roof = {"bound": "hbm", "achieved": by / (k_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s"}
         roof["frac"] = roof["achieved"] / roof["peak"]
-        roof["traffic"] = None
+        roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((rows, ctx))
         roof["kernel_us"] = k_us
         roof["hbm_frac"] = by / (k_us * 1e-6) / 1e9 / HBM_PEAK_GBS
         return us, by / (us * 1e-6) / 1e9, roof, out
@@ -216,6 +222,13 @@ def main():
         a, b = out.astype(np.float64), ref16.astype(np.float64)
         line["parity_vs_cpu"] = {"max_abs": float(np.abs(a - b).max()), "rel_l2": float(np.linalg.norm(a - b) / np.linalg.norm(b))}
     kv.close()
+    if args.calibrate_copy:
+        src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda:0")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        line["calibration_copy_bytes"] = 256 << 20
     if not args.no_extra:
         line["other_configs"] = big_configs(native)
     print(json.dumps(line))
