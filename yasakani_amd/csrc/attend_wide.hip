@@ -52,26 +52,38 @@ struct Raw {                                   // one thread's share of a raw 32
   uint32_t vs;
 };
 
-__device__ __forceinline__ void load_raw(const uint8_t* pg, int tp, int tid, Raw& R) {
-  const uint32_t* kc = reinterpret_cast<const uint32_t*>(pg + kPageKc + (size_t)tp * 64);
-  R.kw[0] = kc[tid]; R.kw[1] = kc[tid + NT];
-  const int pair = tid >> 4, dw = tid & 15;
-  const uint32_t* vc = reinterpret_cast<const uint32_t*>(pg + kPageVc + (size_t)(tp + 2 * pair) * 64) + dw;
-  R.vw[0] = vc[0]; R.vw[1] = vc[16];
-  R.vs = *reinterpret_cast<const uint32_t*>(pg + kPageVs + ((size_t)(dw >> 2) * kPageTok + tp + 2 * pair) * 2);
+// Byte offsets of one thread inside a page, fixed for the whole kernel; the page pointer and the tile's first token
+// are wave uniform, so every load is "scalar base + 32-bit lane offset".
+struct LaneOffs { uint32_t k, v, vs, ks; };
+__device__ __forceinline__ LaneOffs lane_offs(int tid, int h) {
+  const uint32_t pair = tid >> 4, dw = tid & 15;
+  return LaneOffs{(uint32_t)tid * 4u, kPageVc + pair * 128u + dw * 4u, kPageVs + (dw >> 2) * (kPageTok * 2u) + pair * 4u,
+                  kPageKs + (uint32_t)h * 32u};
+}
+__device__ __forceinline__ void load_raw(const uint8_t* pg, int tp, const LaneOffs& L, Raw& R) {
+  const uint8_t* kt = pg + (uint32_t)tp * 64u;            // K and V code rows of the tile start here (+ plane offset)
+  R.kw[0] = *reinterpret_cast<const uint32_t*>(kt + L.k);
+  R.kw[1] = *reinterpret_cast<const uint32_t*>(kt + L.k + NT * 4);
+  R.vw[0] = *reinterpret_cast<const uint32_t*>(kt + L.v);
+  R.vw[1] = *reinterpret_cast<const uint32_t*>(kt + L.v + 64);
+  R.vs = *reinterpret_cast<const uint32_t*>(pg + (uint32_t)tp * 2u + L.vs);
 }
 
-__device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw& R) {
+// (w & mask) | magic as one bit-field insert: `magic` (0x64006400, no bit inside either nibble mask) is kept opaque to
+// the optimizer so that the select form survives to instruction selection
+__device__ __forceinline__ uint32_t nib(uint32_t w, uint32_t mask, uint32_t magic) { return (w & mask) | (magic & ~mask); }
+
+__device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw& R, uint32_t magic) {
   const h2 c1032 = {(_Float16)1032.f, (_Float16)1032.f}, c1152 = {(_Float16)1152.f, (_Float16)1152.f};
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int idx = tid + u * NT, key = idx >> 4, p = idx & 15;      // physical dword p = 4g+m of the key row
     const uint32_t w = R.kw[u], t = w >> 8;
     uint4 o;
-    o.x = as_u32(as_h2((w & 0x000f000fu) | kMagic) - c1032);
-    o.y = as_u32(as_h2((w & 0x00f000f0u) | kMagic) - c1152);
-    o.z = as_u32(as_h2((t & 0x000f000fu) | kMagic) - c1032);
-    o.w = as_u32(as_h2((t & 0x00f000f0u) | kMagic) - c1152);
+    o.x = as_u32(as_h2(nib(w, 0x000f000fu, magic)) - c1032);
+    o.y = as_u32(as_h2(nib(w, 0x00f000f0u, magic)) - c1152);
+    o.z = as_u32(as_h2(nib(t, 0x000f000fu, magic)) - c1032);
+    o.w = as_u32(as_h2(nib(t, 0x00f000f0u, magic)) - c1152);
     *reinterpret_cast<uint4*>(buf + kLdsK + key * kKPitch + (4 * (p & 3) + (p >> 2)) * 16) = o;
   }
   {
@@ -85,8 +97,8 @@ __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw&
     for (int bb = 0; bb < 4; ++bb) {
       // byte bb of both tokens side by side (low half = token t0, high half = token t0+1)
       const uint32_t x = __builtin_amdgcn_perm(w1, w0, 0x0c040c00u + bb * 0x00010001u);
-      const h2 lo = (as_h2((x & 0x000f000fu) | kMagic) - c1032) * s2;       // channel c = 2bb
-      const h2 hi = (as_h2((x & 0x00f000f0u) | kMagic) - c1152) * s2q;      // channel c = 2bb+1
+      const h2 lo = (as_h2(nib(x, 0x000f000fu, magic)) - c1032) * s2;       // channel c = 2bb
+      const h2 hi = (as_h2(nib(x, 0x00f000f0u, magic)) - c1152) * s2q;      // channel c = 2bb+1
       const int c0 = 2 * bb, c1 = 2 * bb + 1;
       *reinterpret_cast<uint32_t*>(vb + 16 * (2 * (c0 & 3) + (c0 >> 2)) * kVPitch) = as_u32(lo);
       *reinterpret_cast<uint32_t*>(vb + 16 * (2 * (c1 & 3) + (c1 >> 2)) * kVPitch) = as_u32(hi);
@@ -96,11 +108,12 @@ __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw&
 
 // group scales of the 16 keys whose scores a lane of half h receives: keys 8a + 4h + b of the tile, 4 fp16 each
 struct KScales { uint4 v[4][2]; };
-__device__ __forceinline__ void load_kscales(const uint8_t* pg, int tp, int h, KScales& K) {
+__device__ __forceinline__ void load_kscales(const uint8_t* pg, int tp, const LaneOffs& L, KScales& K) {
+  const uint8_t* st = pg + (uint32_t)tp * 8u;
 #pragma unroll
   for (int a = 0; a < 4; ++a) {
-    const uint4* sp = reinterpret_cast<const uint4*>(pg + kPageKs + (size_t)(tp + 8 * a + 4 * h) * 8);
-    K.v[a][0] = sp[0]; K.v[a][1] = sp[1];
+    K.v[a][0] = *reinterpret_cast<const uint4*>(st + L.ks + 64 * a);
+    K.v[a][1] = *reinterpret_cast<const uint4*>(st + L.ks + 64 * a + 16);
   }
 }
 
@@ -162,33 +175,37 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
 
   Raw raw;
   KScales sc;
+  const LaneOffs offs = lane_offs(tid, h);
+  uint32_t magic = kMagic;
+  asm volatile("" : "+v"(magic));
   if (tile0 < tile1) {
-    load_raw(kv_page(A.kv, kvh, tile0 << 5), (tile0 << 5) % kPageTok, tid, raw);
-    load_kscales(kv_page(A.kv, kvh, tile0 << 5), (tile0 << 5) % kPageTok, h, sc);
-    dequant_to_lds(lds[0], tid, raw);
-    if (tile0 + 1 < tile1) load_raw(kv_page(A.kv, kvh, (tile0 + 1) << 5), ((tile0 + 1) << 5) % kPageTok, tid, raw);
+    load_raw(kv_page(A.kv, kvh, tile0 << 5), (tile0 << 5) % kPageTok, offs, raw);
+    load_kscales(kv_page(A.kv, kvh, tile0 << 5), (tile0 << 5) % kPageTok, offs, sc);
+    dequant_to_lds(lds[0], tid, raw, magic);
+    if (tile0 + 1 < tile1) load_raw(kv_page(A.kv, kvh, (tile0 + 1) << 5), ((tile0 + 1) << 5) % kPageTok, offs, raw);
   }
   __syncthreads();
   for (int T = tile0; T < tile1; ++T) {
     const int cb = (T - tile0) & 1;
     if (T + 1 < tile1) {
-      dequant_to_lds(lds[cb ^ 1], tid, raw);                          // tile T+1 (loaded one iteration ago)
-      if (T + 2 < tile1) load_raw(kv_page(A.kv, kvh, (T + 2) << 5), ((T + 2) << 5) % kPageTok, tid, raw);
+      dequant_to_lds(lds[cb ^ 1], tid, raw, magic);                   // tile T+1 (loaded one iteration ago)
+      if (T + 2 < tile1) load_raw(kv_page(A.kv, kvh, (T + 2) << 5), ((T + 2) << 5) % kPageTok, offs, raw);
     }
     const uint8_t* buf = lds[cb];
     const int t0 = T << 5;
     const bool need_mask = t0 + 32 > minlen;
     if (nrt > 0) {
       h8 pf[RT][2];
+      // ---- scores: per scale group two chained MFMAs (32 channels), then the fp32 sum times the group scale; one
+      //      K fragment read feeds every row tile of the wave ----
+      float s[RT][16];
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        if (rt < nrt) {
-          // ---- scores: per scale group two chained MFMAs (32 channels), then the fp32 sum times the group scale ----
-          float s[16];
+      for (int m = 0; m < 4; ++m) {
+        const h8 k0 = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsK + j * kKPitch + (4 * m + h) * 16));
+        const h8 k1 = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsK + j * kKPitch + (4 * m + 2 + h) * 16));
 #pragma unroll
-          for (int m = 0; m < 4; ++m) {
-            const h8 k0 = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsK + j * kKPitch + (4 * m + h) * 16));
-            const h8 k1 = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsK + j * kKPitch + (4 * m + 2 + h) * 16));
+        for (int rt = 0; rt < RT; ++rt) {
+          {                                    // row tiles past the wave's last row run on zero queries; nothing of them is stored
             f16v part;
 #pragma unroll
             for (int r = 0; r < 16; ++r) part[r] = 0.f;
@@ -200,23 +217,27 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
               const int a = r >> 2, b = r & 3;
               const uint32_t w2 = (&sc.v[a][b >> 1].x)[2 * (b & 1) + (m >> 1)];   // halfwords 4b+m, 4b+m+1 pair
               const _Float16 sh = as_h2(w2)[m & 1];
-              s[r] = m == 0 ? part[r] * (float)sh : __builtin_fmaf(part[r], (float)sh, s[r]);
+              s[rt][r] = __builtin_fmaf(part[r], (float)sh, m == 0 ? 0.f : s[rt][r]);
             }
           }
-          // ---- online softmax with a lazily raised maximum ----
+        }
+      }
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) {
+        {
+          // ---- online softmax with a lazily raised maximum.  s stays in raw units; the factor log2(e)/sqrt(d) is
+          //      folded into the exponent's fused multiply-add: p = 2^(s * sc_log2 - m_run) ----
           float tmax = -INFINITY;
           if (need_mask) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
               const int key = t0 + 8 * (r >> 2) + 4 * h + (r & 3);
-              s[r] = key < len[rt] ? s[r] * sc_log2 : -INFINITY;
+              s[rt][r] = key < len[rt] ? s[rt][r] : -INFINITY;
             }
-          } else {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) s[r] *= sc_log2;
           }
 #pragma unroll
-          for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[r]);
+          for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[rt][r]);
+          tmax *= sc_log2;
           if (__any(tmax > m_run[rt] + kRaise)) {
             tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
             const float m_new = fmaxf(m_run[rt], tmax);
@@ -230,14 +251,14 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
           float lsum = 0.f;
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const float p = __builtin_amdgcn_exp2f(s[r] - m_run[rt]);
+            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rt][r], sc_log2, -m_run[rt]));
             lsum += p; pf[rt][r >> 3][r & 7] = (_Float16)p;
           }
           l_run[rt] += lsum;
         }
       }
       // scales of the next tile: requested now, needed after the next barrier
-      if (T + 1 < tile1) load_kscales(kv_page(A.kv, kvh, (T + 1) << 5), ((T + 1) << 5) % kPageTok, h, sc);
+      if (T + 1 < tile1) load_kscales(kv_page(A.kv, kvh, (T + 1) << 5), ((T + 1) << 5) % kPageTok, offs, sc);
       // ---- O^T += V^T P^T : d-tile dt (32 rows of the V image), k-step u (16 tokens) ----
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
@@ -246,7 +267,7 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
           const h8 vf = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsV + (32 * dt + j) * kVPitch + (16 * u + 8 * h) * 2));
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt)
-            if (rt < nrt) o[rt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[rt][u], o[rt][dt], 0, 0, 0);
+            o[rt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[rt][u], o[rt][dt], 0, 0, 0);
         }
     }
     __syncthreads();
@@ -255,13 +276,14 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
   //      channel 64(a&1) + 32h + 8b + 4(a>>1) + dt: for each (a&1, b) the lane owns 8 consecutive channels.
   //      Rows go through LDS (the tile buffers are free after the last barrier) so that every store instruction
   //      writes whole 256-byte rows: 16 lanes per row instead of 64 scattered 16-byte pieces. ----
-  static_assert(RT == 1, "the staging below holds one 32-row tile per wave");
   constexpr int kOPitch = 2 * kD + 16;                       // bytes per staged row
-  uint8_t* stage = &lds[0][0] + wave * 32 * kOPitch;         // 4 waves x 8704 bytes
-  {
-    float l = l_run[0];
+  uint8_t* stage = &lds[0][0] + wave * 32 * kOPitch;         // 4 waves x 8704 bytes, reused for every row tile
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt) {
+    if (rt >= nrt) break;
+    float l = l_run[rt];
     l += __shfl_xor(l, 32, 64);
-    if (vrow[0] && h == 0) { A.pm[pidx[0]] = m_run[0]; A.pl[pidx[0]] = l; }
+    if (vrow[rt] && h == 0) { A.pm[pidx[rt]] = m_run[rt]; A.pl[pidx[rt]] = l; }
     const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
     for (int a0 = 0; a0 < 2; ++a0)
@@ -269,23 +291,22 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
       for (int b = 0; b < 4; ++b) {
         h8 v;
 #pragma unroll
-        for (int c = 0; c < 8; ++c) v[c] = (_Float16)(o[0][c & 3][4 * (2 * (c >> 2) + a0) + b] * inv);
+        for (int c = 0; c < 8; ++c) v[c] = (_Float16)(o[rt][c & 3][4 * (2 * (c >> 2) + a0) + b] * inv);
         *reinterpret_cast<uint4*>(stage + j * kOPitch + (64 * a0 + 32 * h + 8 * b) * 2) = __builtin_bit_cast(uint4, v);
       }
-  }
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");     // the wave reads back what its own lanes wrote
-  {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the wave reads back what its own lanes wrote
     const int chunk = lane & 15;
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
       const int jr = 4 * k + (lane >> 4);
-      const int R = row0 + jr;
+      const int R = row0 + rt * 32 + jr;
       if (R < nrows && R < (rb + 1) * RPB) {
         const size_t p = ((size_t)(R / kG) * A.S + split) * A.n_heads + kvh * kG + R % kG;
         const uint4 v = *reinterpret_cast<const uint4*>(stage + jr * kOPitch + chunk * 16);
         *reinterpret_cast<uint4*>(A.pacc16 + p * kD + chunk * 8) = v;
       }
     }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // reads done before the next row tile overwrites the stage
   }
 }
 
