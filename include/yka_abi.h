@@ -83,6 +83,14 @@ YKA_API int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, cons
  * codes [rows][64], scales [rows][4] fp16, y [rows][128] fp32 dequantized. */
 YKA_API int yka_codec_probe(const uint16_t* x16, int rows, uint8_t* codes, uint16_t* scales, float* y);
 
+/* Round trip through the reference's own 256-channel row format, replaces yskn_kvx_probe for it (kvx_probe.cu:7-36):
+ * x [rows][256] fp32 -> [signed Walsh-Hadamard rotation, kvx_codec.cuh:28-49, if rot] -> encode -> decode ->
+ * [inverse rotation] -> y [rows][256].  mode 0: int8 rows, q8 [rows][256], scale = max|x|/127 (kvx_codec.cuh:50-69);
+ * mode 1: flat int4, words [rows][32] with field e in bits [4e, 4e+4) of an MSB-first stream, scale = max|x|/7
+ * (kvq_fast.cuh:194-198,226-233; decode kvq_attn.cuh:33-37,53-54).  scales [rows] fp32.  The array of the other mode
+ * may be NULL.  Results are bit-identical to the reference's arithmetic. */
+YKA_API int yka_kvx256_probe(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, float* y);
+
 /* Canonical image of rows [pos0, pos0+n) of one layer, independent of the physical layout:
  * kc/vc [n_kv_heads][n][64], ks/vs [n_kv_heads][n][4].  export = device -> host, import = host -> device.
  * (The reference reads its containers back only inside its hooks, e.g. kvx_probe.cu:369.) Synchronous. */

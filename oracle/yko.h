@@ -21,6 +21,13 @@
  *   yko_attend_f64           pinned: same closed forms + numpy
  *   yko_combine              pinned: algebraic identity vs unsplit evaluation,
  *                            empty-split sentinel
+ *   yko_kvx_sign             pinned: independent arbitrary-precision evaluation of the integer hash
+ *   yko_kvx_rotate256        pinned: Sylvester Hadamard matrix (scipy) times the sign vector, in fp64;
+ *                            involution; norm preservation
+ *   yko_flat4_encode256 /    pinned: closed-form properties (zero row, max element -> +-7, ties to even),
+ *   yko_flat4_decode256      independent numpy restatement; packing against numpy.unpackbits on the
+ *                            big-endian byte image of the words
+ *   yko_int8_encode256       pinned: closed-form properties, independent numpy restatement
  *
  * The reference holds no golden vectors or known-answer tests for this path, so
  * none are replayed here; the checks above are what the mathematics fixes.
@@ -50,6 +57,16 @@ void yko_quant_rows(const uint16_t* x16, int rows, int dim, uint8_t* codes, uint
 void yko_dequant_rows(const uint8_t* codes, const uint16_t* scales, int rows, int dim, float* y);
 void yko_pack_nibbles(const uint8_t* fields, int n, uint8_t* bytes); /* n even; fields 0..15 */
 void yko_unpack_nibbles(const uint8_t* bytes, int n, uint8_t* fields);
+
+/* ---- the reference's own 256-channel row codec (yko_row256.c) ---- */
+float yko_kvx_sign(int d);                                              /* src/kvx_codec.cuh:28-32 */
+void yko_kvx_rotate256(const float* x, float* y, int inverse);          /* src/kvx_codec.cuh:35-49 */
+/* flat int4, one fp32 scale per row, MSB-first 4-bit fields in 32 words (src/kvq_fast.cuh:194-198,226-233) */
+void yko_flat4_encode256(const float* r, uint32_t* words32, float* scale, float* xq);
+void yko_flat4_decode256(const uint32_t* words32, float scale, float* y);   /* src/kvq_attn.cuh:33-37,53-54 */
+void yko_int8_encode256(const float* x, int8_t* q, float* scale);        /* src/kvx_codec.cuh:50-69 */
+/* round trip of the reference's codec probe (src/kvx_probe.cu:7-20); mode 0 int8 rows, mode 1 flat int4 */
+void yko_kvx_probe256(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, float* y);
 
 /* ---- canonical cache image used by the oracle and by the export/import hooks of the product ----
  * One layer: kc/vc [kvh][max_ctx][dim/2] bytes, ks/vs [kvh][max_ctx][dim/32] fp16 bit patterns. */

@@ -53,6 +53,12 @@ def lib():
         L.yko_splitmix64.restype = C.c_uint64; L.yko_splitmix64.argtypes = [C.c_uint64]
         L.yko_outlier_channels.argtypes = [C.c_uint64, C.c_int, vp]
         L.yko_fill_normal_f16.argtypes = [C.c_uint64, C.c_uint64, C.c_uint64, C.c_int, vp, C.c_float, vp]
+        L.yko_kvx_sign.restype = C.c_float; L.yko_kvx_sign.argtypes = [C.c_int]
+        L.yko_kvx_rotate256.argtypes = [vp, vp, C.c_int]
+        L.yko_flat4_encode256.argtypes = [vp, vp, vp, vp]
+        L.yko_flat4_decode256.argtypes = [vp, C.c_float, vp]
+        L.yko_int8_encode256.argtypes = [vp, vp, vp]
+        L.yko_kvx_probe256.argtypes = [vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]
         _lib = L
     return _lib
 
@@ -185,3 +191,52 @@ def make_inputs(seed, ctx, M, n_heads=24, n_kv_heads=4, dim=D):
     k = fill_normal_f16(seed + 2, (ctx + M) * n_kv_heads, dim, ch, 8.0).reshape(ctx + M, n_kv_heads, dim)
     v = fill_normal_f16(seed + 3, (ctx + M) * n_kv_heads, dim).reshape(ctx + M, n_kv_heads, dim)
     return q, k[:ctx], v[:ctx], k[ctx:], v[ctx:], ch
+
+
+# ---- the reference's own 256-channel row codec ----
+
+def kvx_signs():
+    return np.array([lib().yko_kvx_sign(d) for d in range(256)], dtype=np.float32)
+
+
+def kvx_rotate256(x, inverse=False):
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, 256)
+    y = np.empty_like(x)
+    for r in range(x.shape[0]):
+        lib().yko_kvx_rotate256(_p(x[r]), _p(y[r]), 1 if inverse else 0)
+    return y
+
+
+def flat4_encode256(r):
+    r = np.ascontiguousarray(r, dtype=np.float32).reshape(-1, 256)
+    n = r.shape[0]
+    words = np.empty((n, 32), np.uint32); scale = np.empty(n, np.float32); xq = np.empty_like(r)
+    for i in range(n):
+        lib().yko_flat4_encode256(_p(r[i]), _p(words[i]), _p(scale[i:i + 1]), _p(xq[i]))
+    return words, scale, xq
+
+
+def flat4_decode256(words, scale):
+    words = np.ascontiguousarray(words, dtype=np.uint32).reshape(-1, 32)
+    y = np.empty((words.shape[0], 256), np.float32)
+    for i in range(words.shape[0]):
+        lib().yko_flat4_decode256(_p(words[i]), float(scale[i]), _p(y[i]))
+    return y
+
+
+def int8_encode256(x):
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, 256)
+    q = np.empty(x.shape, np.int8); scale = np.empty(x.shape[0], np.float32)
+    for i in range(x.shape[0]):
+        lib().yko_int8_encode256(_p(x[i]), _p(q[i]), _p(scale[i:i + 1]))
+    return q, scale
+
+
+def kvx_probe256(x, mode, rot):
+    """round trip [rotate] -> encode -> decode -> [inverse rotate]; returns (q8 or None, words or None, scales, y)"""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, 256)
+    n = x.shape[0]
+    q8 = np.zeros((n, 256), np.int8); words = np.zeros((n, 32), np.uint32)
+    scales = np.empty(n, np.float32); y = np.empty_like(x)
+    lib().yko_kvx_probe256(_p(x), n, int(mode), int(rot), _p(q8), _p(words), _p(scales), _p(y))
+    return (q8 if mode == 0 else None), (words if mode == 1 else None), scales, y

@@ -93,3 +93,30 @@ def test_overwrite_rejected_rows(native, oracle):
         kv.layer_call(0, q, k2, v2, 53); oc.append(k2, v2, 53)
         got = kv.export_rows(0, 0, 256)
         assert (got[0] == oc.kc).all() and (got[1] == oc.ks).all() and (got[2] == oc.vc).all() and (got[3] == oc.vs).all()
+
+
+# ---- the reference's own 256-channel row format (rotation, flat int4 MSB-first, int8 rows) ----
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("rot", [0, 1])
+def test_row256_probe_bit_exact(native, oracle, mode, rot):
+    yko = oracle
+    rng = np.random.default_rng(100 + 2 * mode + rot)
+    x = (rng.standard_normal((257, 256)) * rng.uniform(1e-3, 30, size=(257, 1))).astype(np.float32)
+    x[7] = 0.0                                           # zero row: scale 1 (int4) / 0 (int8), all codes zero
+    x[8, :] = 0.0; x[8, 3] = -5.0                        # a single non-zero element encodes to the extreme code
+    x[9] = np.round(x[9])                                # integers: exact butterflies
+    q8, words, scales, y = native.kvx256_probe(x, mode, rot)
+    rq8, rwords, rscales, ry = yko.kvx_probe256(x, mode, rot)
+    assert np.array_equal(scales.view(np.uint32), rscales.view(np.uint32))
+    if mode == 0:
+        assert np.array_equal(q8, rq8)
+    else:
+        assert np.array_equal(words, rwords)
+    assert np.array_equal(y.view(np.uint32), ry.view(np.uint32))
+
+
+def test_row256_probe_rejects_bad_arguments(native):
+    x = np.zeros((2, 256), np.float32)
+    with pytest.raises(native.YkaError):
+        native.kvx256_probe(x, 2, 0)

@@ -248,6 +248,25 @@ int yka_codec_probe(const uint16_t* x16, int rows, uint8_t* codes, uint16_t* sca
   YKA_CATCH_INT
 }
 
+int yka_kvx256_probe(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, float* y) {
+  YKA_TRY
+  if (!x || !scales || !y || rows < 1 || (mode != 0 && mode != 1)) throw std::runtime_error("bad argument");
+  if ((mode == 0 && !q8) || (mode == 1 && !words)) throw std::runtime_error("the output array of the selected mode is null");
+  const size_t n = (size_t)rows * 256;
+  DevBuf dx(n * 4), dq(mode == 0 ? n : 4), dw(mode == 1 ? (size_t)rows * 128 : 4), ds((size_t)rows * 4), dy(n * 4);
+  HIPCHK(hipMemcpy(dx.p, x, n * 4, hipMemcpyHostToDevice));
+  launch_row256_encode(dx.as<float>(), rows, mode, rot != 0, dq.as<int8_t>(), dw.as<uint32_t>(), ds.as<float>(), nullptr);
+  HIPCHK(hipGetLastError());
+  launch_row256_decode(rows, mode, rot != 0, dq.as<int8_t>(), dw.as<uint32_t>(), ds.as<float>(), dy.as<float>(), nullptr);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipDeviceSynchronize());
+  if (mode == 0) HIPCHK(hipMemcpy(q8, dq.p, n, hipMemcpyDeviceToHost));
+  else HIPCHK(hipMemcpy(words, dw.p, (size_t)rows * 128, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(scales, ds.p, (size_t)rows * 4, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(y, dy.p, n * 4, hipMemcpyDeviceToHost));
+  YKA_CATCH_INT
+}
+
 static void check_range(const yka_kv* kv, int pos0, int n) {
   if (pos0 < 0 || n < 1 || (long long)pos0 + n > kv->cfg.max_ctx) throw std::runtime_error("row range outside the container");
 }

@@ -1,0 +1,106 @@
+// The reference's own 256-channel row codec on gfx950: signed Walsh-Hadamard rotation, flat int4 with one fp32 scale
+// per row and MSB-first packing, int8 rows.  Compiled with -ffp-contract=off: every value is produced by the same
+// sequence of single IEEE fp32 operations as in the reference, so results are bit-identical to it.
+//   rotation   src/kvx_codec.cuh:28-49        flat int4  src/kvq_fast.cuh:194-198, packing :226-233
+//   int8 rows  src/kvx_codec.cuh:50-69        decode     src/kvq_attn.cuh:33-37,53-54
+// One workgroup of 256 threads (4 waves) per row, thread d owns channel d.
+#include "yka_internal.h"
+
+namespace yka {
+namespace {
+
+__device__ __forceinline__ float kvx_sign(int d) {
+  uint32_t x = (uint32_t)d + 1u;
+  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+  return (x & 1u) ? -1.f : 1.f;
+}
+
+// The butterfly stages are element-wise, so where the partner lives does not change a bit of the result: partners at
+// distance 1..32 are in the same wave (cross-lane exchange), 64 and 128 go through LDS.
+__device__ __forceinline__ float rotate256(float x, float* buf, bool inverse) {
+  const int d = threadIdx.x;
+  float a = inverse ? x : __fmul_rn(x, kvx_sign(d));
+#pragma unroll
+  for (int h = 1; h < 64; h *= 2) {
+    const float b = __shfl_xor(a, h, 64);
+    a = (d & h) ? __fsub_rn(b, a) : __fadd_rn(a, b);
+  }
+#pragma unroll
+  for (int h = 64; h < 256; h *= 2) {
+    __syncthreads();
+    buf[d] = a;
+    __syncthreads();
+    const float b = buf[d ^ h];
+    a = (d & h) ? __fsub_rn(b, a) : __fadd_rn(a, b);
+  }
+  float y = __fmul_rn(a, 0.0625f);
+  if (inverse) y = __fmul_rn(y, kvx_sign(d));
+  return y;
+}
+
+__device__ __forceinline__ float row_absmax(float v, float* red) {
+  float m = fabsf(v);
+#pragma unroll
+  for (int o = 32; o; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  return fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+}
+
+__global__ void __launch_bounds__(256) row256_encode_kernel(const float* x, int mode, int rot, int8_t* q8, uint32_t* words, float* scales) {
+  __shared__ float buf[256];
+  __shared__ float red[4];
+  __shared__ uint8_t fld[256];
+  const int row = blockIdx.x, d = threadIdx.x;
+  float v = x[(size_t)row * 256 + d];
+  if (rot) v = rotate256(v, buf, false);
+  const float am = row_absmax(v, red);
+  if (mode == 0) {
+    const float sc = __fdiv_rn(am, 127.f);
+    int q = sc > 0.f ? __float2int_rn(__fdiv_rn(v, sc)) : 0;
+    q = max(-127, min(127, q));
+    q8[(size_t)row * 256 + d] = (int8_t)q;
+    if (d == 0) scales[row] = sc;
+  } else {
+    float s7 = __fdiv_rn(am, 7.f);
+    if (s7 == 0.f) s7 = 1.f;
+    float q = rintf(__fdiv_rn(v, s7));
+    q = fminf(fmaxf(q, -7.f), 7.f);
+    fld[d] = (uint8_t)((int)q + 8);
+    __syncthreads();
+    if (d < 32) {                               // word d = fields 8d .. 8d+7, the first in the top nibble
+      uint32_t w = 0u;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) w |= (uint32_t)fld[8 * d + i] << (28 - 4 * i);
+      words[(size_t)row * 32 + d] = w;
+    }
+    if (d == 0) scales[row] = s7;
+  }
+}
+
+__global__ void __launch_bounds__(256) row256_decode_kernel(int mode, int rot, const int8_t* q8, const uint32_t* words, const float* scales, float* y) {
+  __shared__ float buf[256];
+  const int row = blockIdx.x, d = threadIdx.x;
+  const float s = scales[row];
+  float v;
+  if (mode == 0) v = __fmul_rn((float)q8[(size_t)row * 256 + d], s);
+  else {
+    const uint32_t w = words[(size_t)row * 32 + (d >> 3)];
+    const int nib = (int)((w >> (28 - 4 * (d & 7))) & 15u);
+    v = __fmul_rn((float)(nib - 8), s);
+  }
+  if (rot) v = rotate256(v, buf, true);
+  y[(size_t)row * 256 + d] = v;
+}
+
+}  // namespace
+
+void launch_row256_encode(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, hipStream_t st) {
+  hipLaunchKernelGGL(row256_encode_kernel, dim3(rows), dim3(256), 0, st, x, mode, rot, q8, words, scales);
+}
+void launch_row256_decode(int rows, int mode, int rot, const int8_t* q8, const uint32_t* words, const float* scales, float* y, hipStream_t st) {
+  hipLaunchKernelGGL(row256_decode_kernel, dim3(rows), dim3(256), 0, st, mode, rot, q8, words, scales, y);
+}
+
+}  // namespace yka

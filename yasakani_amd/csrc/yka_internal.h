@@ -63,6 +63,9 @@ void launch_import_rows(const KvView&, int pos0, int n, const uint8_t* kc, const
 void launch_dequant_rows(const KvView&, int pos0, int n, float* k, float* v, hipStream_t);
 void launch_codec_probe(const uint16_t* x16, int rows, uint8_t* codes, uint16_t* scales, float* y, hipStream_t);
 void launch_set_int(int* p, int v, hipStream_t);
+// the reference's own 256-channel row format (row256.hip): mode 0 = int8 rows, 1 = flat int4 (32 MSB-first words per row)
+void launch_row256_encode(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, hipStream_t);
+void launch_row256_decode(int rows, int mode, int rot, const int8_t* q8, const uint32_t* words, const float* scales, float* y, hipStream_t);
 
 // start of the (page, kv head) block that holds token t
 __device__ __forceinline__ uint8_t* kv_page(const KvView& kv, int kvh, int t) {

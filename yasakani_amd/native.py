@@ -44,6 +44,7 @@ def _load():
         "yka_attend": (i32, [vp, i32, vp, i32, vp, vp, vp, vp]),
         "yka_append_attend": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
         "yka_codec_probe": (i32, [vp, i32, vp, vp, vp]),
+        "yka_kvx256_probe": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_kv_export_rows": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_kv_import_rows": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_kv_dequant_rows": (i32, [vp, i32, i32, i32, vp, vp]),
@@ -62,7 +63,7 @@ def _load():
 
 
 EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "yka_set_opt", "yka_kv_set_page_table",
-           "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kv_export_rows",
+           "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kvx256_probe", "yka_kv_export_rows",
            "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
            "yka_append_host", "yka_pass_capture", "yka_pass_launch", "yka_pass_destroy", "yka_attn_bench")
 
@@ -108,6 +109,21 @@ def codec_probe(x16):
     y = np.empty((rows, D), np.float32)
     _chk(lib().yka_codec_probe(_ptr(x), rows, _ptr(codes), _ptr(scales), _ptr(y)))
     return codes, scales, y
+
+
+def kvx256_probe(x, mode, rot):
+    """Round trip through the reference's 256-channel row format (kvx_probe.cu:7-36).  x [rows,256] f32;
+    mode 0 = int8 rows, 1 = flat int4 (MSB-first words); rot = signed Walsh-Hadamard rotation before and after.
+    Returns (q8 [rows,256] i8 or None, words [rows,32] u32 or None, scales [rows] f32, y [rows,256] f32)."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, 256)
+    rows = x.shape[0]
+    q8 = np.empty((rows, 256), np.int8) if mode == 0 else None
+    words = np.empty((rows, 32), np.uint32) if mode == 1 else None
+    scales = np.empty(rows, np.float32)
+    y = np.empty((rows, 256), np.float32)
+    _chk(lib().yka_kvx256_probe(_ptr(x), rows, int(mode), int(rot), _ptr(q8) if q8 is not None else None,
+                                _ptr(words) if words is not None else None, _ptr(scales), _ptr(y)))
+    return q8, words, scales, y
 
 
 class KvCache:
