@@ -128,6 +128,41 @@ def big_configs(native):
     return out
 
 
+def append_vs_post(torch, native, kv, ctx, rows_list=(1, 64), calls=400):
+    """Eager launches on torch's stream: plain quantize-on-append of fp16 rows against the fused norm + rotary + rotation +
+    quantize step fed with the projection's fp32 rows (one launch each; us per call, launch cost included)."""
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(7)
+    out = {}
+    stream = torch.cuda.current_stream().cuda_stream
+    for M in rows_list:
+        xq = torch.randn(M, NH, D, generator=g).to(dev); xk = torch.randn(M, KVH, D, generator=g).to(dev)
+        xv = torch.randn(M, KVH, D, generator=g).to(dev)
+        k16 = xk.half(); v16 = xv.half()
+        w = (torch.randn(D, generator=g) * 0.1).half().to(dev)
+        rd = 32
+        f = torch.arange(ctx + M, dtype=torch.float64)[:, None] * (10000.0 ** (-2.0 * torch.arange(rd // 2, dtype=torch.float64) / rd))[None, :]
+        rope = torch.stack([torch.cos(f), torch.sin(f)], dim=-1).float().contiguous().to(dev)
+        q16 = torch.empty(M, NH, D, dtype=torch.float16, device=dev)
+        dpos = torch.tensor([ctx], dtype=torch.int32, device=dev)
+        P = native.PostParams(w.data_ptr(), w.data_ptr(), 1e-6, rope.data_ptr(), rd, ctx + M, 1)
+        res = {}
+        for name, fn in (("append", lambda l: kv.append(l, k16.data_ptr(), v16.data_ptr(), M, dpos.data_ptr(), stream)),
+                         ("post", lambda l: kv.attn_post(l, xq.data_ptr(), xk.data_ptr(), xv.data_ptr(), M, dpos.data_ptr(), P, q16.data_ptr(), stream))):
+            for i in range(20):
+                fn(i % kv.cfg.n_layers)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for i in range(calls):
+                fn(i % kv.cfg.n_layers)
+            e1.record(); torch.cuda.synchronize()
+            res[name + "_us"] = e0.elapsed_time(e1) * 1e3 / calls
+        res["post_bytes"] = M * (NH + 2 * KVH) * D * 4 + M * NH * D * 2 + M * TOKEN_BYTES
+        out[f"rows_{M}"] = res
+    return out
+
+
 def cpu_baseline(kv, q, ctx, M, budget_s=20.0):
     """The CPU oracle (threaded port of the reference's token-streaming split-KV loop) on the same quantized cache.
     Bounded sample: whole layer calls are repeated until about `budget_s` seconds of CPU work are spent."""
@@ -221,6 +256,8 @@ def main():
         line["cpu_baseline"] = base
         a, b = out.astype(np.float64), ref16.astype(np.float64)
         line["parity_vs_cpu"] = {"max_abs": float(np.abs(a - b).max()), "rel_l2": float(np.linalg.norm(a - b) / np.linalg.norm(b))}
+    if not args.no_extra:                       # last: it overwrites the rows the parity check above reads
+        line["append_vs_post"] = append_vs_post(torch, native, kv, ctx)
     kv.close()
     if args.calibrate_copy:
         src = torch.ones(256 << 20, dtype=torch.uint8, device="cuda:0")

@@ -48,7 +48,9 @@ YKA_API const char* yka_last_error(void);
 YKA_API const char* yka_build_info(void);
 /* replaces yskn_set_opt (yskn_abi.h:87) for the options of this path.
  * key 1: split count of the narrow kernel (decode, rows of at most 2 tokens; at most 256); key 2: split count of the wide kernel;
- * key 3: 1 forces the narrow kernel for every width (cross-check of the wide kernel), 0 = automatic. */
+ * key 3: 1 forces the narrow kernel for every width (cross-check of the wide kernel), 0 = automatic;
+ * key 4: 1 = attention outputs get the inverse signed Hadamard rotation before they are rounded to fp16 (for caches
+ *        filled by yka_attn_post with rotate = 1; the reference un-rotates in its output step, q35_kernels.cu:1421). */
 YKA_API int yka_set_opt(yka_kv* kv, int key, int value);
 
 /* Paged mode: logical page p of `layer` (-1 = every layer) lives in physical page h_table[p]; n_pages = max_ctx/256
@@ -77,7 +79,33 @@ YKA_API int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, cons
                               const uint16_t* d_v16, int M, const int* d_pos, const uint8_t* d_depth,
                               uint16_t* d_out16, void* hip_stream);
 
+/* The step between the QKV projection and the cache, fused with quantize-on-append; replaces launch_q35_attn_post
+ * (q35.hpp:97-105, q35_kernels.cu:1013-1065) + launch_tb_requant (q35_kernels.cu:1084-1092) for 128-channel heads:
+ * per head, Q and K rows are RMS-normalised (x / sqrt(mean x^2 + eps) * (1 + w)), get the rotary embedding on their
+ * first rope_dims channels (pairing d <-> d + rope_dims/2, table row = position) and, if rotate, the signed
+ * Walsh-Hadamard rotation (kvx_codec.cuh:28-49 for 128 channels; K and V x 1/8, Q x 1/16); V rows are only rotated.
+ * Q rows are written to d_q16 [M][n_heads][128] fp16; K and V rows are rounded to fp16 and quantized into rows
+ * *d_pos .. *d_pos+M-1 of `layer` exactly as yka_append would store them.  d_xq [M][n_heads][128], d_xk, d_xv
+ * [M][n_kv_heads][128] are the projection's fp32 outputs (the reference's split-K recombination and per-column factors,
+ * q35_kernels.cu:1027-1032, happen before this call).  Allocates nothing, synchronises nothing. */
+typedef struct yka_post_params {
+  const uint16_t* d_qn_w16;  /* [128] fp16 norm weights of Q heads, applied as (1 + w) (q35_kernels.cu:1057) */
+  const uint16_t* d_kn_w16;  /* [128] the same for K heads */
+  float eps;
+  const float* d_rope;       /* [rope_rows][rope_dims/2][2] fp32 (cos, sin) by position (q35_kernels.cu:1101-1107) */
+  int32_t rope_dims;         /* even, 0..128; 0 = no rotary step (the reference rotates 64 of 256 channels, q35.hpp:13) */
+  int32_t rope_rows;         /* rows whose position is not below rope_rows are dropped */
+  int32_t rotate;            /* 0 / 1 */
+} yka_post_params;
+YKA_API int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float* d_xk, const float* d_xv, int M,
+                          const int* d_pos, const yka_post_params* params, uint16_t* d_q16, void* hip_stream);
+
 /* ---- hooks with host pointers (model: src/kvx_probe.cu) ---- */
+
+/* Host-pointer form of yka_attn_post: uploads everything, sets the device position to `pos`, runs, downloads q16. */
+YKA_API int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, const float* xv, int M, int pos,
+                               const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope,
+                               int rope_dims, int rope_rows, int rotate, uint16_t* q16);
 
 /* Codec round trip on the GPU, replaces yskn_kvx_probe (kvx_probe.cu:22-36): x16 [rows][128] fp16 ->
  * codes [rows][64], scales [rows][4] fp16, y [rows][128] fp32 dequantized. */

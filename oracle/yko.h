@@ -28,6 +28,10 @@
  *   yko_flat4_decode256      independent numpy restatement; packing against numpy.unpackbits on the
  *                            big-endian byte image of the words
  *   yko_int8_encode256       pinned: closed-form properties, independent numpy restatement
+ *   yko_rotate128            pinned: scipy Sylvester matrix (exact on integer rows), forward x inverse = identity,
+ *                            q.k invariance
+ *   yko_attn_post            pinned: numpy fp64 RMS normalisation and complex-multiplication rotary form within the
+ *                            fp16 roundings, position 0 = no rotary change, pair-norm preservation, V rows pass through
  *
  * The reference holds no golden vectors or known-answer tests for this path, so
  * none are replayed here; the checks above are what the mathematics fixes.
@@ -67,6 +71,15 @@ void yko_flat4_decode256(const uint32_t* words32, float scale, float* y);   /* s
 void yko_int8_encode256(const float* x, int8_t* q, float* scale);        /* src/kvx_codec.cuh:50-69 */
 /* round trip of the reference's codec probe (src/kvx_probe.cu:7-20); mode 0 int8 rows, mode 1 flat int4 */
 void yko_kvx_probe256(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, float* y);
+
+/* ---- between the QKV projection and the cache (yko_post.c; src/q35_kernels.cu:1013-1065 for 128-channel heads) ---- */
+void yko_rotate128(const float* x, float* y, int inverse, float factor);
+void yko_post_qk_row(const float* y, const uint16_t* w16, float eps, const float* cs, int rd, int rot, float rot_factor, uint16_t* out16);
+void yko_post_v_row(const float* y, int rot, uint16_t* out16);
+void yko_attn_post(const float* xq, const float* xk, const float* xv, int M, int n_heads, int n_kv,
+                   const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope, int rd, int pos,
+                   int rot, uint16_t* q16, uint16_t* k16, uint16_t* v16);
+void yko_unrotate_out(const float* y32, int rows, uint16_t* out16);
 
 /* ---- canonical cache image used by the oracle and by the export/import hooks of the product ----
  * One layer: kc/vc [kvh][max_ctx][dim/2] bytes, ks/vs [kvh][max_ctx][dim/32] fp16 bit patterns. */

@@ -59,6 +59,9 @@ def lib():
         L.yko_flat4_decode256.argtypes = [vp, C.c_float, vp]
         L.yko_int8_encode256.argtypes = [vp, vp, vp]
         L.yko_kvx_probe256.argtypes = [vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]
+        L.yko_rotate128.argtypes = [vp, vp, C.c_int, C.c_float]
+        L.yko_attn_post.argtypes = [vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, C.c_float, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp]
+        L.yko_unrotate_out.argtypes = [vp, C.c_int, vp]
         _lib = L
     return _lib
 
@@ -240,3 +243,45 @@ def kvx_probe256(x, mode, rot):
     scales = np.empty(n, np.float32); y = np.empty_like(x)
     lib().yko_kvx_probe256(_p(x), n, int(mode), int(rot), _p(q8), _p(words), _p(scales), _p(y))
     return (q8 if mode == 0 else None), (words if mode == 1 else None), scales, y
+
+
+# ---- between the QKV projection and the cache ----
+
+def rotate128(x, inverse=False, factor=0.125):
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, 128)
+    y = np.empty_like(x)
+    for r in range(x.shape[0]):
+        lib().yko_rotate128(_p(x[r]), _p(y[r]), 1 if inverse else 0, float(factor))
+    return y
+
+
+def rope_table(n_pos, rd, base=10000.0):
+    """(cos, sin) [n_pos][rd/2][2] fp32, frequencies base^(-2i/rd), values rounded to fp16 precision
+    (the reference rounds its table to its 16-bit activation type, q35_kernels.cu:1101-1107)."""
+    i = np.arange(rd // 2, dtype=np.float64)
+    f = np.arange(n_pos, dtype=np.float64)[:, None] * base ** (-2.0 * i / rd)[None, :]
+    t = np.stack([np.cos(f), np.sin(f)], axis=-1)
+    return np.ascontiguousarray(t.astype(np.float16).astype(np.float32))
+
+
+def attn_post(xq, xk, xv, qn_w16, kn_w16, eps, rope, rd, pos, rot):
+    """fp32 projection rows -> (q16, k16, v16) fp16 bit patterns; xq [M,H,128], xk/xv [M,KVH,128]"""
+    xq = np.ascontiguousarray(xq, np.float32); xk = np.ascontiguousarray(xk, np.float32); xv = np.ascontiguousarray(xv, np.float32)
+    M, H, _ = xq.shape; KVH = xk.shape[1]
+    q16 = np.empty((M, H, 128), np.uint16); k16 = np.empty((M, KVH, 128), np.uint16); v16 = np.empty((M, KVH, 128), np.uint16)
+    qw = _as_u16(qn_w16); kw = _as_u16(kn_w16)
+    if rd > 0:
+        rope = np.ascontiguousarray(rope, np.float32)
+        assert rope.shape[0] >= pos + M and rope.shape[1] == rd // 2
+    else:
+        rope = np.zeros(1, np.float32)             # never read when there is no rotary step
+    lib().yko_attn_post(_p(xq), _p(xk), _p(xv), M, H, KVH, _p(qw), _p(kw), float(eps), _p(rope), int(rd), int(pos), int(rot),
+                        _p(q16), _p(k16), _p(v16))
+    return q16, k16, v16
+
+
+def unrotate_out(y32):
+    y32 = np.ascontiguousarray(y32, np.float32)
+    out = np.empty(y32.shape, np.uint16)
+    lib().yko_unrotate_out(_p(y32), int(y32.size // 128), _p(out))
+    return out

@@ -1,0 +1,105 @@
+/* CPU oracle, part 4: the step between the QKV projection and the cache - per-head RMS normalisation, partial rotary
+ * embedding, optional signed Walsh-Hadamard rotation - for 128-channel heads.  TEST INFRASTRUCTURE ONLY.
+ *
+ * Follows q35_attn_post_kernel (src/q35_kernels.cu:1013-1065) with the roundings the reference makes to its 16-bit
+ * activation type (bf16 there, fp16 here, the type of this path's Q / K / V rows):
+ *   y            the projection's fp32 output for one head (128 values); the reference's split-K recombination and
+ *                its per-column factors happen before this point and are not restated
+ *   V rows       no normalisation, no rotary step (:1037-1047): [rotation] -> fp16
+ *   Q and K      ss = sum y^2 (:1050-1056); r = 1 / sqrt(ss / 128 + eps); xn = f16(y * r * (1 + w[d])) (:1057);
+ *                rotary on the first rd channels with the rotate-half pairing d <-> d + rd/2 (:1060-1063):
+ *                  d <  rd/2: f16( f16(xn[d] * cos) + f16(-xn[d + rd/2] * sin) )
+ *                  d >= rd/2: f16( f16(xn[d] * cos) + f16( xn[d - rd/2] * sin) )   with (cos, sin) of channel d - rd/2
+ *                then [rotation] -> fp16
+ * Sum order of ss (fixed so that every implementation can match it bit for bit): inside each half of 64 channels the
+ * butterfly a[i] += a[i ^ o], o = 32, 16, 8, 4, 2, 1; then half 0 + half 1.
+ * Rotation for 128 channels: signs from the same integer hash as the 256-channel form (src/kvx_codec.cuh:28-32),
+ * 7 butterfly stages as src/kvx_codec.cuh:40-45, then a power-of-two factor: 1/8 for K and V rows, 1/16 for Q rows and
+ * for the inverse applied to attention outputs.  (1/8)(1/16) 128 = 1, so q.k is unchanged by rotating both, and the
+ * inverse undoes the V rotation exactly up to fp32 rounding; all factors are exact in floating point.
+ */
+#include "yko.h"
+#include <math.h>
+#include <string.h>
+
+void yko_rotate128(const float* x, float* y, int inverse, float factor) {
+  float a[128], b[128];
+  for (int d = 0; d < 128; ++d) a[d] = inverse ? x[d] : x[d] * yko_kvx_sign(d);
+  for (int h = 1; h < 128; h *= 2) {
+    for (int d = 0; d < 128; ++d) {
+      const float self = a[d], other = a[d ^ h];
+      b[d] = (d & h) ? other - self : self + other;
+    }
+    memcpy(a, b, sizeof a);
+  }
+  for (int d = 0; d < 128; ++d) {
+    float v = a[d] * factor;
+    if (inverse) v = v * yko_kvx_sign(d);
+    y[d] = v;
+  }
+}
+
+static float f16r(float x) { return yko_h2f(yko_f2h(x)); }
+
+static float sumsq128(const float* y) {
+  float half[2];
+  for (int w = 0; w < 2; ++w) {
+    float a[64], b[64];
+    for (int i = 0; i < 64; ++i) a[i] = y[64 * w + i] * y[64 * w + i];
+    for (int o = 32; o; o >>= 1) {
+      for (int i = 0; i < 64; ++i) b[i] = a[i] + a[i ^ o];
+      memcpy(a, b, sizeof a);
+    }
+    half[w] = a[0];
+  }
+  return half[0] + half[1];
+}
+
+/* one Q or K head row: y[128] -> out16[128] */
+void yko_post_qk_row(const float* y, const uint16_t* w16, float eps, const float* cs /* [rd/2][2] of this position */,
+                     int rd, int rot, float rot_factor, uint16_t* out16) {
+  const float tot = sumsq128(y);
+  const float r = 1.f / sqrtf(tot / 128.f + eps);
+  float xn[128], o[128];
+  for (int d = 0; d < 128; ++d) xn[d] = f16r((y[d] * r) * (1.f + yko_h2f(w16[d])));
+  const int hr = rd / 2;
+  for (int d = 0; d < 128; ++d) {
+    if (d < hr) o[d] = f16r(f16r(xn[d] * cs[2 * d]) + f16r(-xn[d + hr] * cs[2 * d + 1]));
+    else if (d < rd) o[d] = f16r(f16r(xn[d] * cs[2 * (d - hr)]) + f16r(xn[d - hr] * cs[2 * (d - hr) + 1]));
+    else o[d] = xn[d];
+  }
+  if (rot) { float t[128]; yko_rotate128(o, t, 0, rot_factor); memcpy(o, t, sizeof o); }
+  for (int d = 0; d < 128; ++d) out16[d] = yko_f2h(o[d]);
+}
+
+void yko_post_v_row(const float* y, int rot, uint16_t* out16) {
+  float o[128];
+  if (rot) yko_rotate128(y, o, 0, 0.125f); else memcpy(o, y, sizeof o);
+  for (int d = 0; d < 128; ++d) out16[d] = yko_f2h(o[d]);
+}
+
+/* xq [M][n_heads][128], xk, xv [M][n_kv][128] fp32; rope [rows][rd/2][2] = (cos, sin) of position row; row t of the
+ * pass sits at position pos + t.  Outputs fp16 rows of the same shapes; k16 / v16 are what quantize-on-append then
+ * stores (yko_append). */
+void yko_attn_post(const float* xq, const float* xk, const float* xv, int M, int n_heads, int n_kv,
+                   const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope, int rd, int pos,
+                   int rot, uint16_t* q16, uint16_t* k16, uint16_t* v16) {
+  for (int t = 0; t < M; ++t) {
+    const float* cs = rope + (size_t)(pos + t) * rd;   /* rd/2 pairs of 2 floats */
+    for (int h = 0; h < n_heads; ++h)
+      yko_post_qk_row(xq + ((size_t)t * n_heads + h) * 128, qn_w16, eps, cs, rd, rot, 0.0625f, q16 + ((size_t)t * n_heads + h) * 128);
+    for (int h = 0; h < n_kv; ++h) {
+      yko_post_qk_row(xk + ((size_t)t * n_kv + h) * 128, kn_w16, eps, cs, rd, rot, 0.125f, k16 + ((size_t)t * n_kv + h) * 128);
+      yko_post_v_row(xv + ((size_t)t * n_kv + h) * 128, rot, v16 + ((size_t)t * n_kv + h) * 128);
+    }
+  }
+}
+
+/* inverse rotation of attention outputs: y32 [rows][128] fp32 (pre-rounding) -> out16 */
+void yko_unrotate_out(const float* y32, int rows, uint16_t* out16) {
+  for (int r = 0; r < rows; ++r) {
+    float o[128];
+    yko_rotate128(y32 + (size_t)r * 128, o, 1, 0.0625f);
+    for (int d = 0; d < 128; ++d) out16[(size_t)r * 128 + d] = yko_f2h(o[d]);
+  }
+}

@@ -1,0 +1,117 @@
+"""Pins the oracle's restatement of the step between the QKV projection and the cache (RMS normalisation, partial
+rotary embedding, 128-point signed Hadamard rotation) against numpy fp64 forms and structural properties.  CPU only."""
+import numpy as np
+from scipy.linalg import hadamard
+
+from oracle import yko
+
+
+def _h(x):
+    return np.asarray(x, np.uint16).view(np.float16).astype(np.float64)
+
+
+def test_rotate128_is_signed_sylvester_matrix_exact_on_integers():
+    rng = np.random.default_rng(1)
+    x = rng.integers(-8, 9, size=(8, 128)).astype(np.float32)
+    H = hadamard(128).astype(np.float64)
+    s = yko.kvx_signs()[:128].astype(np.float64)
+    for factor in (0.125, 0.0625):
+        fwd = (H @ (x * s).T).T * factor
+        assert np.array_equal(yko.rotate128(x, False, factor), fwd.astype(np.float32))
+        inv = (H @ x.astype(np.float64).T).T * factor * s
+        assert np.array_equal(yko.rotate128(x, True, factor), inv.astype(np.float32))
+
+
+def test_rotation_factors_compose_to_identity_and_keep_dot_products():
+    rng = np.random.default_rng(2)
+    q = rng.standard_normal((16, 128)).astype(np.float32)
+    k = rng.standard_normal((16, 128)).astype(np.float32)
+    rq, rk = yko.rotate128(q, False, 0.0625), yko.rotate128(k, False, 0.125)
+    assert np.allclose((rq.astype(np.float64) * rk).sum(1), (q.astype(np.float64) * k).sum(1), rtol=0, atol=2e-5)
+    back = yko.rotate128(yko.rotate128(k, False, 0.125), True, 0.0625)   # V forward, output inverse
+    assert np.abs(back - k).max() < 2e-6
+
+
+def _post_numpy(y, w16, eps, cs, rd):
+    """fp64 RMS normalisation + rotary as complex multiplication, no intermediate rounding"""
+    y = y.astype(np.float64)
+    r = 1.0 / np.sqrt((y * y).mean() + eps)
+    xn = y * r * (1.0 + _h(w16))
+    hr = rd // 2
+    z = (xn[:hr] + 1j * xn[hr:rd]) * (cs[:, 0] + 1j * cs[:, 1])
+    out = xn.copy(); out[:hr] = z.real; out[hr:rd] = z.imag
+    return out
+
+
+def test_post_rows_match_fp64_forms():
+    rng = np.random.default_rng(3)
+    M, H, KVH, rd, pos = 5, 24, 4, 32, 37
+    xq = (rng.standard_normal((M, H, 128)) * 3).astype(np.float32)
+    xk = (rng.standard_normal((M, KVH, 128)) * 0.5).astype(np.float32)
+    xv = rng.standard_normal((M, KVH, 128)).astype(np.float32)
+    qw = (rng.standard_normal(128) * 0.1).astype(np.float16).view(np.uint16)
+    kw = (rng.standard_normal(128) * 0.1).astype(np.float16).view(np.uint16)
+    rope = yko.rope_table(64, rd)
+    q16, k16, v16 = yko.attn_post(xq, xk, xv, qw, kw, 1e-6, rope, rd, pos, rot=0)
+    for t in range(M):
+        cs = rope[pos + t].astype(np.float64)
+        for h in range(H):
+            ref = _post_numpy(xq[t, h], qw, 1e-6, cs, rd)
+            # three fp16 roundings on the rotary channels, one elsewhere
+            assert np.abs(_h(q16[t, h]) - ref).max() <= 2.5e-3 * max(1.0, np.abs(ref).max())
+        for h in range(KVH):
+            ref = _post_numpy(xk[t, h], kw, 1e-6, cs, rd)
+            assert np.abs(_h(k16[t, h]) - ref).max() <= 2.5e-3 * max(1.0, np.abs(ref).max())
+    # V rows: plain rounding to fp16
+    assert np.array_equal(v16, xv.astype(np.float16).view(np.uint16))
+    # channels past rd carry no rotary change: one rounding only
+    ref = _post_numpy(xq[0, 0], qw, 1e-6, rope[pos].astype(np.float64), rd)
+    assert np.array_equal(q16[0, 0, rd:], ref[rd:].astype(np.float16).view(np.uint16))
+
+
+def test_post_structure():
+    rng = np.random.default_rng(4)
+    rd = 32
+    x = rng.standard_normal((1, 1, 128)).astype(np.float32)
+    zero_w = np.zeros(128, np.uint16)
+    rope = yko.rope_table(16, rd)
+    # position 0: cos = 1, sin = 0 -> the rotary step changes nothing; unit RMS after normalisation
+    q16, _, _ = yko.attn_post(x, x[:, :1], x[:, :1], zero_w, zero_w, 0.0, rope, rd, 0, 0)
+    assert abs(np.sqrt((_h(q16) ** 2).mean()) - 1.0) < 1e-3
+    qb, _, _ = yko.attn_post(x, x[:, :1], x[:, :1], zero_w, zero_w, 0.0, rope, rd, 7, 0)
+    a, b = _h(q16)[0, 0], _h(qb)[0, 0]
+    hr = rd // 2
+    assert np.allclose(a[:hr] ** 2 + a[hr:rd] ** 2, b[:hr] ** 2 + b[hr:rd] ** 2, atol=2e-2)   # each pair only turns
+    assert np.array_equal(a[rd:], b[rd:])
+    assert not np.array_equal(a[:rd], b[:rd])
+    # scale invariance of the normalisation (power-of-two factor: exact)
+    qc, _, _ = yko.attn_post(x * 4, x[:, :1], x[:, :1], zero_w, zero_w, 0.0, rope, rd, 7, 0)
+    assert np.array_equal(qb, qc)
+
+
+def test_post_with_rotation_equals_rotation_of_post():
+    rng = np.random.default_rng(5)
+    M, H, KVH, rd = 3, 24, 4, 32
+    xq = rng.standard_normal((M, H, 128)).astype(np.float32)
+    xk = rng.standard_normal((M, KVH, 128)).astype(np.float32)
+    xv = rng.standard_normal((M, KVH, 128)).astype(np.float32)
+    w = (rng.standard_normal(128) * 0.1).astype(np.float16).view(np.uint16)
+    rope = yko.rope_table(16, rd)
+    q0, k0, v0 = yko.attn_post(xq, xk, xv, w, w, 1e-6, rope, rd, 2, 0)
+    q1, k1, v1 = yko.attn_post(xq, xk, xv, w, w, 1e-6, rope, rd, 2, 1)
+    f = lambda u: u.view(np.float16).astype(np.float32).reshape(-1, 128)
+    assert np.array_equal(q1.reshape(-1, 128), yko.rotate128(f(q0), False, 0.0625).astype(np.float16).view(np.uint16))
+    assert np.array_equal(k1.reshape(-1, 128), yko.rotate128(f(k0), False, 0.125).astype(np.float16).view(np.uint16))
+    assert np.array_equal(v1.reshape(-1, 128), yko.rotate128(xv.reshape(-1, 128), False, 0.125).astype(np.float16).view(np.uint16))
+    # scores survive the rotation up to the fp16 rounding of the rotated rows
+    s0 = (f(q0)[:24].astype(np.float64) * f(k0)[0]).sum(1)
+    s1 = (f(q1)[:24].astype(np.float64) * f(k1)[0]).sum(1)
+    assert np.abs(s0 - s1).max() < 0.05
+
+
+def test_unrotate_out_inverts_v_rotation():
+    rng = np.random.default_rng(6)
+    v = rng.standard_normal((10, 128)).astype(np.float32)
+    rv = yko.rotate128(v, False, 0.125)
+    out = yko.unrotate_out(rv)
+    assert np.abs(_h(out) - v).max() < 2e-3

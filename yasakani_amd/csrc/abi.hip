@@ -30,7 +30,7 @@ struct yka_kv {
   size_t ws_rows = 0;              // capacity of the partial workspace in (token, split) pairs
   int* d_pos = nullptr;            // position used by the host-pointer hooks
   hipStream_t stream = nullptr;    // stream of the host-pointer hooks
-  int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0;
+  int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0, opt_unrot = 0;
   KvView view(int layer) const {
     return KvView{pool + (size_t)layer * layer_bytes, tables ? tables + (size_t)layer * n_pages : nullptr, cfg.n_kv_heads, cfg.max_ctx};
   }
@@ -99,7 +99,7 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
     AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * kD, d_pos, depth, Ms, s0, NH, S, wide_rows_per_block(Ms), kv->pm, kv->pl, kv->pacc16,
                fuse_append ? k16 : nullptr, fuse_append ? v16 : nullptr};
     if (narrow) launch_attend_narrow(A, st); else launch_attend_wide(A, st);
-    if (mode != 2) launch_combine(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD}, st);
+    if (mode != 2) launch_combine(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD, kv->opt_unrot}, st);
   }
 }
 
@@ -182,6 +182,7 @@ int yka_set_opt(yka_kv* kv, int key, int value) {
     case 1: if (value < 0 || value > kMaxSplits) throw std::runtime_error("splits must be in [0, 256]"); kv->opt_splits_narrow = value; break;
     case 2: if (value < 0 || value > kMaxSplits) throw std::runtime_error("splits must be in [0, 256]"); kv->opt_splits_wide = value; break;
     case 3: kv->opt_force_narrow = value != 0; break;
+    case 4: kv->opt_unrot = value != 0; break;
     default: throw std::runtime_error("unknown option key");
   }
   YKA_CATCH_INT
@@ -245,6 +246,54 @@ int yka_codec_probe(const uint16_t* x16, int rows, uint8_t* codes, uint16_t* sca
   HIPCHK(hipMemcpy(codes, dc.p, n / 2, hipMemcpyDeviceToHost));
   HIPCHK(hipMemcpy(scales, ds.p, (size_t)rows * kNG * 2, hipMemcpyDeviceToHost));
   HIPCHK(hipMemcpy(y, dy.p, n * 4, hipMemcpyDeviceToHost));
+  YKA_CATCH_INT
+}
+
+static void check_post(const yka_kv* kv, const yka_post_params* P) {
+  if (!P) throw std::runtime_error("null parameter block");
+  if (!P->d_qn_w16 || !P->d_kn_w16) throw std::runtime_error("null norm weights");
+  if (P->rope_dims < 0 || P->rope_dims > kD || (P->rope_dims & 1)) throw std::runtime_error("rope_dims must be even and in [0, 128]");
+  if (P->rope_dims > 0 && (!P->d_rope || P->rope_rows < 1)) throw std::runtime_error("rotary table missing");
+  (void)kv;
+}
+
+int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float* d_xk, const float* d_xv, int M, const int* d_pos,
+                  const yka_post_params* P, uint16_t* d_q16, void* hip_stream) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); check_rows(kv, M); check_post(kv, P);
+  if (!d_xq || !d_xk || !d_xv || !d_pos || !d_q16) throw std::runtime_error("null pointer");
+  launch_attn_post(PostArgs{kv->view(layer), d_xq, d_xk, d_xv, M, kv->cfg.n_heads, d_pos, P->d_qn_w16, P->d_kn_w16, P->eps,
+                            P->d_rope, P->rope_dims, P->rope_rows, P->rotate != 0, d_q16}, (hipStream_t)hip_stream);
+  HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, const float* xv, int M, int pos,
+                       const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope, int rope_dims,
+                       int rope_rows, int rotate, uint16_t* q16) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); check_rows(kv, M);
+  if (!xq || !xk || !xv || !qn_w16 || !kn_w16 || !q16) throw std::runtime_error("null pointer");
+  if (pos < 0 || (long long)pos + M > kv->cfg.max_ctx) throw std::runtime_error("rows outside the container");
+  if (rope_dims < 0 || rope_dims > kD || (rope_dims & 1)) throw std::runtime_error("rope_dims must be even and in [0, 128]");
+  if (rope_dims > 0 && (!rope || rope_rows < pos + M)) throw std::runtime_error("rotary table shorter than pos + M");
+  const size_t nq = (size_t)M * kv->cfg.n_heads * kD, nk = (size_t)M * kv->cfg.n_kv_heads * kD;
+  const size_t nr = rope_dims > 0 ? (size_t)rope_rows * rope_dims : 1;
+  DevBuf dq(nq * 4), dk(nk * 4), dv(nk * 4), dqw(kD * 2), dkw(kD * 2), dr(nr * 4), dq16(nq * 2);
+  HIPCHK(hipMemcpy(dq.p, xq, nq * 4, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dk.p, xk, nk * 4, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dv.p, xv, nk * 4, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dqw.p, qn_w16, kD * 2, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dkw.p, kn_w16, kD * 2, hipMemcpyHostToDevice));
+  if (rope_dims > 0) HIPCHK(hipMemcpy(dr.p, rope, nr * 4, hipMemcpyHostToDevice));
+  yka_post_params P{dqw.as<uint16_t>(), dkw.as<uint16_t>(), eps, dr.as<float>(), rope_dims, rope_rows, rotate};
+  check_post(kv, &P);
+  launch_set_int(kv->d_pos, pos, kv->stream);
+  launch_attn_post(PostArgs{kv->view(layer), dq.as<float>(), dk.as<float>(), dv.as<float>(), M, kv->cfg.n_heads, kv->d_pos,
+                            P.d_qn_w16, P.d_kn_w16, eps, P.d_rope, rope_dims, rope_rows, rotate != 0, dq16.as<uint16_t>()}, kv->stream);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipStreamSynchronize(kv->stream));
+  HIPCHK(hipMemcpy(q16, dq16.p, nq * 2, hipMemcpyDeviceToHost));
   YKA_CATCH_INT
 }
 

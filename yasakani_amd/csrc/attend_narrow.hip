@@ -273,12 +273,32 @@ __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
   for (int c = 0; c < 8; ++c) s_o[sl][c8 + c] = acc[c];
   if ((tid & 15) == 0) s_wsum[sl] = wsum;
   __syncthreads();
+  float y = 0.f;
   if (tid < kD) {
     float o = 0.f, L = 0.f;
 #pragma unroll
     for (int k = 0; k < 16; ++k) { o += s_o[k][tid]; L += s_wsum[k]; }
-    A.out16[((size_t)tok * A.n_heads + head) * kD + tid] = __half_as_ushort(__float2half_rn(o / L));
+    y = o / L;
   }
+  if (A.unrot) {                                   // uniform over the grid
+    // inverse signed Hadamard rotation over the row's 128 channels (threads 0..127 = two waves)
+#pragma unroll
+    for (int h = 1; h < 64; h *= 2) {
+      const float b = __shfl_xor(y, h, 64);
+      y = (tid & h) ? b - y : y + b;
+    }
+    __syncthreads();
+    if (tid < kD) s_w[tid] = y;
+    __syncthreads();
+    if (tid < kD) {
+      const float b = s_w[tid ^ 64];
+      y = (tid & 64) ? b - y : y + b;
+      uint32_t x = (uint32_t)tid + 1u;             // sign of channel tid (src/kvx_codec.cuh:28-32)
+      x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+      y = y * 0.0625f * ((x & 1u) ? -1.f : 1.f);
+    }
+  }
+  if (tid < kD) A.out16[((size_t)tok * A.n_heads + head) * kD + tid] = __half_as_ushort(__float2half_rn(y));
 }
 void launch_combine(const CombineArgs& A, hipStream_t st) {
   hipLaunchKernelGGL(combine_kernel, dim3(A.n_heads, A.M), dim3(256), 0, st, A);

@@ -30,8 +30,12 @@ __device__ __forceinline__ void quant_lane(float x, int& code, uint16_t& s16) {
 
 // Quantizes channel d (0..127) of one fp16 row and stores its share of the row at token `pos` of kv head `kvh`.
 // Must be called by all 128 lanes of two full waves (d = lane index over the row); isv selects the V planes.
+__device__ __forceinline__ void quant_store_value(const KvView& kv, int kvh, int pos, bool isv, float x, int d);
 __device__ __forceinline__ void quant_store_row(const KvView& kv, int kvh, int pos, bool isv, const uint16_t* src_row, int d) {
-  const float x = h2f_bits(src_row[d]);
+  quant_store_value(kv, kvh, pos, isv, h2f_bits(src_row[d]), d);
+}
+// the same with the (fp16-valued) channel already in a register
+__device__ __forceinline__ void quant_store_value(const KvView& kv, int kvh, int pos, bool isv, float x, int d) {
   int code; uint16_t s16;
   quant_lane(x, code, s16);
   const int nb = __shfl_xor(code, 1, 64);

@@ -50,13 +50,23 @@ struct AttnArgs {
   // before reading it (fused quantize-on-append).
   const uint16_t* k16; const uint16_t* v16;
 };
-struct CombineArgs { const float* pm; const float* pl; const uint16_t* pacc16; int S; int M; int n_heads; uint16_t* out16; };
+// unrot != 0: the output row gets the inverse signed Hadamard rotation (7 butterfly stages, x 1/16, signs) before it is
+// rounded to fp16 - the counterpart of rotating V rows on their way into the cache (src/q35_kernels.cu:1421)
+struct CombineArgs { const float* pm; const float* pl; const uint16_t* pacc16; int S; int M; int n_heads; uint16_t* out16; int unrot; };
+// projection outputs xq [M][n_heads][128], xk / xv [M][n_kv][128] fp32 -> q16 and the cache rows at *d_pos + t
+struct PostArgs {
+  KvView kv; const float* xq; const float* xk; const float* xv; int M; int n_heads; const int* d_pos;
+  const uint16_t* qn_w16; const uint16_t* kn_w16; float eps;
+  const float* rope; int rd; int rope_rows;      // rope [rope_rows][rd/2] (cos, sin) pairs; rd = 0: no rotary step
+  int rot; uint16_t* q16;
+};
 
 // launchers (each checks nothing: the C layer validates shapes first)
 void launch_append(const AppendArgs&, hipStream_t);
 void launch_attend_narrow(const AttnArgs&, hipStream_t);   // 16-row tiles: 2 tokens x 6 heads per workgroup column
 void launch_attend_wide(const AttnArgs&, hipStream_t);     // 3..64 tokens
 void launch_combine(const CombineArgs&, hipStream_t);
+void launch_attn_post(const PostArgs&, hipStream_t);
 // canonical <-> physical
 void launch_export_rows(const KvView&, int pos0, int n, uint8_t* kc, uint16_t* ks, uint8_t* vc, uint16_t* vs, hipStream_t);
 void launch_import_rows(const KvView&, int pos0, int n, const uint8_t* kc, const uint16_t* ks, const uint8_t* vc, const uint16_t* vs, hipStream_t);

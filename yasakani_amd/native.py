@@ -26,6 +26,13 @@ class KvConfig(C.Structure):
                 ("n_layers", "n_heads", "n_kv_heads", "head_dim", "max_ctx", "max_rows", "paged", "device")]
 
 
+class PostParams(C.Structure):
+    """yka_post_params: device pointers of the norm weights and of the rotary table, and the switches of the step
+    between the QKV projection and the cache."""
+    _fields_ = [("d_qn_w16", C.c_void_p), ("d_kn_w16", C.c_void_p), ("eps", C.c_float), ("d_rope", C.c_void_p),
+                ("rope_dims", C.c_int32), ("rope_rows", C.c_int32), ("rotate", C.c_int32)]
+
+
 def _load():
     path = library_path()
     if not os.path.exists(path):
@@ -45,6 +52,8 @@ def _load():
         "yka_append_attend": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
         "yka_codec_probe": (i32, [vp, i32, vp, vp, vp]),
         "yka_kvx256_probe": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
+        "yka_attn_post": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
+        "yka_attn_post_host": (i32, [vp, i32, vp, vp, vp, i32, i32, vp, vp, C.c_float, vp, i32, i32, i32, vp]),
         "yka_kv_export_rows": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_kv_import_rows": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_kv_dequant_rows": (i32, [vp, i32, i32, i32, vp, vp]),
@@ -63,7 +72,8 @@ def _load():
 
 
 EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "yka_set_opt", "yka_kv_set_page_table",
-           "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kvx256_probe", "yka_kv_export_rows",
+           "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kvx256_probe", "yka_attn_post",
+           "yka_attn_post_host", "yka_kv_export_rows",
            "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
            "yka_append_host", "yka_pass_capture", "yka_pass_launch", "yka_pass_destroy", "yka_attn_bench")
 
@@ -177,6 +187,10 @@ class KvCache:
     def append(self, layer, d_k16, d_v16, M, d_pos, stream=0):
         _chk(lib().yka_append(self._h, layer, d_k16, d_v16, M, d_pos, stream))
 
+    def attn_post(self, layer, d_xq, d_xk, d_xv, M, d_pos, params, d_q16, stream=0):
+        """Device-pointer form: projection outputs -> Q rows in d_q16, K/V rows quantized into the cache (params: PostParams)."""
+        _chk(lib().yka_attn_post(self._h, layer, d_xq, d_xk, d_xv, M, d_pos, C.byref(params), d_q16, stream))
+
     def attend(self, layer, d_q16, M, d_pos, d_out16, d_depth=None, stream=0):
         _chk(lib().yka_attend(self._h, layer, d_q16, M, d_pos, d_depth, d_out16, stream))
 
@@ -225,6 +239,23 @@ class KvCache:
         M = k16.shape[0]
         k = _u16(k16, (M, self.cfg.n_kv_heads, D)); v = _u16(v16, (M, self.cfg.n_kv_heads, D))
         _chk(lib().yka_append_host(self._h, layer, _ptr(k), _ptr(v), M, pos))
+
+    def attn_post_host(self, layer, xq, xk, xv, pos, qn_w16, kn_w16, eps, rope, rope_dims, rotate=False):
+        """Projection outputs (fp32; xq [M,n_heads,128], xk/xv [M,n_kv_heads,128]) -> RMS norm, rotary, optional
+        rotation; K/V rows are quantized into rows pos..pos+M-1, the Q rows come back as fp16 [M,n_heads,128]."""
+        M = xq.shape[0]
+        xq = np.ascontiguousarray(xq, np.float32).reshape(M, self.cfg.n_heads, D)
+        xk = np.ascontiguousarray(xk, np.float32).reshape(M, self.cfg.n_kv_heads, D)
+        xv = np.ascontiguousarray(xv, np.float32).reshape(M, self.cfg.n_kv_heads, D)
+        qw = _u16(qn_w16, (D,)); kw = _u16(kn_w16, (D,))
+        rows = 0
+        if rope_dims > 0:
+            rope = np.ascontiguousarray(rope, np.float32).reshape(-1, rope_dims // 2, 2)
+            rows = rope.shape[0]
+        q16 = np.empty((M, self.cfg.n_heads, D), np.uint16)
+        _chk(lib().yka_attn_post_host(self._h, layer, _ptr(xq), _ptr(xk), _ptr(xv), M, pos, _ptr(qw), _ptr(kw), float(eps),
+                                      _ptr(rope) if rope_dims > 0 else None, int(rope_dims), rows, int(bool(rotate)), _ptr(q16)))
+        return q16.view(np.float16)
 
     def capture_pass(self, layers, d_q16, d_k16, d_v16, M, d_pos, d_out16, d_depth=None, mode=0):
         """Records one layer call per listed layer into a graph (device addresses); returns a Pass."""
