@@ -128,6 +128,38 @@ def big_configs(native):
     return out
 
 
+def batched_decode(torch, native, kv, ctx, L, k_new, v_new, q, calls=200):
+    """Multi-stream passes on the containers already filled for the headline run: one row per stream, B streams at `ctx`
+    cached tokens each (one pass = append + attention + combine for all B rows; B x 18.9 MB of KV)."""
+    dev = torch.device("cuda:0")
+    out = {}
+    stream = torch.cuda.current_stream().cuda_stream
+    for B in (8, 16, 32):
+        if B > L:
+            continue
+        rep = (B + q.shape[0] - 1) // q.shape[0]
+        dq = torch.from_numpy(np.tile(q, (rep, 1, 1))[:B].view(np.int16).copy()).to(dev)
+        dk = torch.from_numpy(np.tile(k_new, (rep, 1, 1))[:B].view(np.int16).copy()).to(dev)
+        dv = torch.from_numpy(np.tile(v_new, (rep, 1, 1))[:B].view(np.int16).copy()).to(dev)
+        dout = torch.zeros_like(dq)
+        dpos = torch.full((B,), ctx, dtype=torch.int32, device=dev)
+        dslot = torch.arange(B, dtype=torch.int32, device=dev)
+        fn = lambda: kv.append_attend_ms(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, dpos.data_ptr(), dslot.data_ptr(), dout.data_ptr(), stream)
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(calls):
+            fn()
+        e1.record(); torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / calls
+        by = B * algorithmic_bytes(ctx, 1)
+        out[f"streams_{B}"] = {"us_per_pass": us, "us_per_row": us / B, "value_GBs": by / (us * 1e-6) / 1e9,
+                               "hbm_peak_frac": by / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
+    return out
+
+
 def append_vs_post(torch, native, kv, ctx, rows_list=(1, 64), calls=400):
     """Eager launches on torch's stream: plain quantize-on-append of fp16 rows against the fused norm + rotary + rotation +
     quantize step fed with the projection's fp32 rows (one launch each; us per call, launch cost included)."""
@@ -257,6 +289,7 @@ def main():
         a, b = out.astype(np.float64), ref16.astype(np.float64)
         line["parity_vs_cpu"] = {"max_abs": float(np.abs(a - b).max()), "rel_l2": float(np.linalg.norm(a - b) / np.linalg.norm(b))}
     if not args.no_extra:                       # last: it overwrites the rows the parity check above reads
+        line["batched_decode"] = batched_decode(torch, native, kv, ctx, L, kn, vn, q)
         line["append_vs_post"] = append_vs_post(torch, native, kv, ctx)
     kv.close()
     if args.calibrate_copy:

@@ -79,6 +79,17 @@ YKA_API int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, cons
                               const uint16_t* d_v16, int M, const int* d_pos, const uint8_t* d_depth,
                               uint16_t* d_out16, void* hip_stream);
 
+/* Multi-stream pass (batched decode): row t of the pass belongs to the stream whose KV container is d_row_slot[t]
+ * (a container index in [0, n_layers): the handle's containers are then one per stream of the layer being run) and sits
+ * at position d_row_pos[t] of it.  If d_k16 / d_v16 are given, row t of them is quantized into that row first; then row
+ * t of d_q16 attends to keys [0, d_row_pos[t]] of its container.  Rows of one stream may follow each other at
+ * consecutive positions (a stream's last token and its draft tokens).  A row whose slot or position is out of range is
+ * dropped and yields zeros.  Replaces launch_q35_attn_post_ms / launch_tb_requant_ms, launch_q35_atx_pk_ms and
+ * launch_q35_combine_ms (q35.hpp:28-35,109-112,157; q35_atxpk.hpp:18-20; kernel src/q35_atxpk_ms.cu).  The reference caps
+ * such a pass at 16 rows (Q35_SST, q35.hpp:20); here M may be up to max_rows.  Allocates nothing, synchronises nothing. */
+YKA_API int yka_append_attend_ms(yka_kv* kv, const uint16_t* d_q16, const uint16_t* d_k16, const uint16_t* d_v16, int M,
+                                 const int* d_row_pos, const int* d_row_slot, uint16_t* d_out16, void* hip_stream);
+
 /* The step between the QKV projection and the cache, fused with quantize-on-append; replaces launch_q35_attn_post
  * (q35.hpp:97-105, q35_kernels.cu:1013-1065) + launch_tb_requant (q35_kernels.cu:1084-1092) for 128-channel heads:
  * per head, Q and K rows are RMS-normalised (x / sqrt(mean x^2 + eps) * (1 + w)), get the rotary embedding on their
@@ -101,6 +112,10 @@ YKA_API int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float*
                           const int* d_pos, const yka_post_params* params, uint16_t* d_q16, void* hip_stream);
 
 /* ---- hooks with host pointers (model: src/kvx_probe.cu) ---- */
+
+/* Host-pointer form of yka_append_attend_ms (k16 / v16 may be NULL = attend only). */
+YKA_API int yka_ms_call_host(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M,
+                             const int32_t* row_pos, const int32_t* row_slot, uint16_t* out16);
 
 /* Host-pointer form of yka_attn_post: uploads everything, sets the device position to `pos`, runs, downloads q16. */
 YKA_API int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, const float* xv, int M, int pos,

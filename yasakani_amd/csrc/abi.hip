@@ -103,6 +103,24 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
   }
 }
 
+// Multi-stream pass: rows are appended first (several rows of one stream may follow each other and read each other's
+// keys), then every row attends to keys [0, pos[t]] of its own container.  One token per workgroup column.
+void do_attend_ms(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, const int* row_pos,
+                  const int* row_slot, uint16_t* out16, hipStream_t st) {
+  const int NH = kv->cfg.n_heads;
+  const RowMap R{row_pos, row_slot, kv->cfg.n_layers, kv->layer_bytes, kv->n_pages};
+  if (k16) launch_append(AppendArgs{kv->view(0), k16, v16, nullptr, M, R}, st);
+  for (int s0 = 0; s0 < M; s0 += kMaxSlice) {
+    const int Ms = std::min(kMaxSlice, M - s0);
+    int S = kv->opt_splits_narrow > 0 ? kv->opt_splits_narrow : 1024 / (kv->cfg.n_kv_heads * Ms);
+    S = std::min(std::max(2, std::min(kMaxSplits, S)), (int)(kWsPairs / (size_t)Ms));
+    RowMap Rs = R; Rs.pos += s0; Rs.slot += s0;
+    AttnArgs A{kv->view(0), q16 + (size_t)s0 * NH * kD, nullptr, nullptr, Ms, s0, NH, S, 128, kv->pm, kv->pl, kv->pacc16, nullptr, nullptr, Rs};
+    launch_attend_narrow(A, st);
+    launch_combine(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD, kv->opt_unrot}, st);
+  }
+}
+
 }  // namespace
 
 #define YKA_TRY try {
@@ -231,6 +249,37 @@ int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16
   if (!d_q16 || !d_k16 || !d_v16 || !d_pos || !d_out16) throw std::runtime_error("null pointer");
   do_attend(kv, layer, d_q16, M, d_pos, d_depth, d_out16, (hipStream_t)hip_stream, 0, d_k16, d_v16);
   HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_append_attend_ms(yka_kv* kv, const uint16_t* d_q16, const uint16_t* d_k16, const uint16_t* d_v16, int M,
+                         const int* d_row_pos, const int* d_row_slot, uint16_t* d_out16, void* hip_stream) {
+  YKA_TRY
+  on_device(kv); check_rows(kv, M);
+  if (!d_q16 || !d_row_pos || !d_row_slot || !d_out16) throw std::runtime_error("null pointer");
+  if ((d_k16 == nullptr) != (d_v16 == nullptr)) throw std::runtime_error("new K and V rows come together or not at all");
+  do_attend_ms(kv, d_q16, d_k16, d_v16, M, d_row_pos, d_row_slot, d_out16, (hipStream_t)hip_stream);
+  HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_ms_call_host(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, const int32_t* row_pos,
+                     const int32_t* row_slot, uint16_t* out16) {
+  YKA_TRY
+  on_device(kv); check_rows(kv, M);
+  if (!q16 || !row_pos || !row_slot || !out16) throw std::runtime_error("null pointer");
+  if ((k16 == nullptr) != (v16 == nullptr)) throw std::runtime_error("new K and V rows come together or not at all");
+  const size_t nq = (size_t)M * kv->cfg.n_heads * kD, nk = (size_t)M * kv->cfg.n_kv_heads * kD;
+  DevBuf dq(nq * 2), dk(nk * 2), dv(nk * 2), dout(nq * 2), dp((size_t)M * 4), dsl((size_t)M * 4);
+  HIPCHK(hipMemcpy(dq.p, q16, nq * 2, hipMemcpyHostToDevice));
+  if (k16) { HIPCHK(hipMemcpy(dk.p, k16, nk * 2, hipMemcpyHostToDevice)); HIPCHK(hipMemcpy(dv.p, v16, nk * 2, hipMemcpyHostToDevice)); }
+  HIPCHK(hipMemcpy(dp.p, row_pos, (size_t)M * 4, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dsl.p, row_slot, (size_t)M * 4, hipMemcpyHostToDevice));
+  do_attend_ms(kv, dq.as<uint16_t>(), k16 ? dk.as<uint16_t>() : nullptr, k16 ? dv.as<uint16_t>() : nullptr, M, dp.as<int>(), dsl.as<int>(),
+               dout.as<uint16_t>(), kv->stream);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipStreamSynchronize(kv->stream));
+  HIPCHK(hipMemcpy(out16, dout.p, nq * 2, hipMemcpyDeviceToHost));
   YKA_CATCH_INT
 }
 

@@ -71,20 +71,36 @@ __device__ __forceinline__ void load_tile(const uint8_t* pg, int tp, int i, int 
     R.vw[e] = *reinterpret_cast<const uint32_t*>(pg + kPageVc + (size_t)(tp + tau(g, e)) * 64 + 4 * i);
 }
 
-// grid (S, n_kv, ceil(M/2)), block 256 (4 waves).  Workgroup = (split, kv head, row tile of 2 tokens x 6 heads).
+// grid (S, n_kv, ceil(M/TPT)), block 256 (4 waves).  Workgroup = (split, kv head, row tile of TPT tokens x 6 heads):
+// TPT = 2 for a single-stream pass; MS (multi-stream pass, reference: src/q35_atxpk_ms.cu:13-33): one token per tile,
+// which reads the container and the position its row map names.
+template <bool MS>
 __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
   __shared__ float s_m[4][16], s_l[4][16];
   __shared__ float s_acc[4][16][kD + 4];
+  constexpr int TPT = MS ? 1 : 2;
   const int split = blockIdx.x, kvh = blockIdx.y, rt = blockIdx.z;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
-  const int pos = *A.d_pos;
+  int pos; bool row_ok = true;
+  if (MS) {
+    pos = A.rows.pos[rt];
+    const int slot = A.rows.slot[rt];
+    row_ok = pos >= 0 && pos < A.kv.max_ctx && slot >= 0 && slot < A.rows.n_slots;   // a bad row reads nothing and yields zeros
+    A.kv = slot_view(A.kv, A.rows, row_ok ? slot : 0);
+  } else {
+    pos = *A.d_pos;
+  }
 
-  // query row of this lane column: j = i -> (token 2*rt + i/6, head kvh*6 + i%6); columns 12..15 are padding
-  const int tl = 2 * rt + i / kG;                  // token index inside the slice
-  const bool vrow = i < 2 * kG && tl < A.M;
+  // query row of this lane column: j = i -> (token TPT*rt + i/6, head kvh*6 + i%6); the other columns are padding
+  const int tl = TPT * rt + i / kG;                // token index inside the slice
+  const bool vrow = i < TPT * kG && tl < A.M && row_ok;
   const int head = kvh * kG + i % kG;
   int len = 0;
-  if (vrow) { const int tg = A.tok0 + tl; len = pos + (A.depth ? (int)A.depth[tg] : tg) + 1; len = min(len, A.kv.max_ctx); }
+  if (vrow) {
+    if (MS) len = pos + 1;
+    else { const int tg = A.tok0 + tl; len = pos + (A.depth ? (int)A.depth[tg] : tg) + 1; }
+    len = min(len, A.kv.max_ctx);
+  }
   int maxlen = len;
 #pragma unroll
   for (int o = 1; o < 16; o <<= 1) maxlen = max(maxlen, __shfl_xor(maxlen, o, 64));
@@ -95,7 +111,7 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
   //      whose tile range holds it - the only workgroup of this kv head that will read it in this launch.  Writer and
   //      readers are waves of one workgroup, i.e. of one CU and one (write-through) L1, so workgroup-scope fences
   //      around the barrier order the stores before the loads without any cache maintenance. ----
-  if (A.k16) {
+  if (!MS && A.k16) {
     bool mine = false;
     for (int t = 0; t < A.M; ++t) {
       const int r = pos + t;
@@ -208,9 +224,9 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) s_acc[wave][i][8 * (4 * g + r) + b] = o[b][r];
   __syncthreads();
-  for (int idx = threadIdx.x; idx < 2 * kG * kD; idx += 256) {
+  for (int idx = threadIdx.x; idx < TPT * kG * kD; idx += 256) {
     const int j = idx >> 7, d = idx & (kD - 1);
-    const int tj = 2 * rt + j / kG;
+    const int tj = TPT * rt + j / kG;
     if (tj >= A.M) continue;
     const float m0 = s_m[0][j], m1 = s_m[1][j], m2 = s_m[2][j], m3 = s_m[3][j];
     const float M2 = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
@@ -224,7 +240,8 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
 }
 
 void launch_attend_narrow(const AttnArgs& A, hipStream_t st) {
-  hipLaunchKernelGGL(attend_narrow_kernel, dim3(A.S, A.kv.n_kv, (A.M + 1) / 2), dim3(256), 0, st, A);
+  if (A.rows.pos) hipLaunchKernelGGL(attend_narrow_kernel<true>, dim3(A.S, A.kv.n_kv, A.M), dim3(256), 0, st, A);
+  else hipLaunchKernelGGL(attend_narrow_kernel<false>, dim3(A.S, A.kv.n_kv, (A.M + 1) / 2), dim3(256), 0, st, A);
 }
 
 // combiner (reference: src/attention_kv4q.cu:325-332): M2 = max pm; w_s = pm_s > -1e29 ? 2^(pm_s - M2) * pl_s : 0;
@@ -278,7 +295,7 @@ __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
     float o = 0.f, L = 0.f;
 #pragma unroll
     for (int k = 0; k < 16; ++k) { o += s_o[k][tid]; L += s_wsum[k]; }
-    y = o / L;
+    y = L > 0.f ? o / L : 0.f;                     // a row that saw no key at all (a rejected row of a multi-stream pass)
   }
   if (A.unrot) {                                   // uniform over the grid
     // inverse signed Hadamard rotation over the row's 128 channels (threads 0..127 = two waves)

@@ -9,9 +9,15 @@ namespace yka {
 // Rows land at *d_pos + tok (reference: q35_kernels.cu:1038,1064 write the pass's rows before attention reads them).
 __global__ void __launch_bounds__(128) append_kernel(AppendArgs A) {
   const int tok = blockIdx.x, kvh = blockIdx.y >> 1, isv = blockIdx.y & 1, d = threadIdx.x;
+  const uint16_t* src = (isv ? A.v16 : A.k16) + ((size_t)tok * A.kv.n_kv + kvh) * kD;
+  if (A.rows.pos) {                                // multi-stream pass: the row's own container and position
+    const int pos = A.rows.pos[tok], slot = A.rows.slot[tok];
+    if (pos < 0 || pos >= A.kv.max_ctx || slot < 0 || slot >= A.rows.n_slots) return;
+    quant_store_row(slot_view(A.kv, A.rows, slot), kvh, pos, isv != 0, src, d);
+    return;
+  }
   const int pos = *A.d_pos + tok;
   if (pos < 0 || pos >= A.kv.max_ctx) return;
-  const uint16_t* src = (isv ? A.v16 : A.k16) + ((size_t)tok * A.kv.n_kv + kvh) * kD;
   quant_store_row(A.kv, kvh, pos, isv != 0, src, d);
 }
 void launch_append(const AppendArgs& A, hipStream_t st) {

@@ -32,7 +32,17 @@ struct KvView {
 };
 __host__ __device__ inline size_t kv_page_bytes(int n_kv) { return (size_t)n_kv * kPageBytes; }
 
-struct AppendArgs { KvView kv; const uint16_t* k16; const uint16_t* v16; const int* d_pos; int M; };
+// Multi-stream passes (reference: Q35MsRows, src/q35.hpp:28-35): row t of the pass belongs to the stream whose container
+// is slot[t] and sits at position pos[t] of it.  Containers are slot_bytes apart (page tables slot_pages entries apart),
+// starting from the view the arguments carry.  pos == nullptr: single-stream pass.
+struct RowMap { const int* pos = nullptr; const int* slot = nullptr; int n_slots = 0; size_t slot_bytes = 0; int slot_pages = 0; };
+__device__ __forceinline__ KvView slot_view(KvView v, const RowMap& R, int slot) {
+  v.base += (size_t)slot * R.slot_bytes;
+  if (v.table) v.table += (size_t)slot * R.slot_pages;
+  return v;
+}
+
+struct AppendArgs { KvView kv; const uint16_t* k16; const uint16_t* v16; const int* d_pos; int M; RowMap rows; };
 
 // partial results of the split-KV kernels (same roles as pm/pl/pacc of the reference, args.hpp:10):
 //   pm, pl [rows_tok][S][n_heads] fp32; pacc16 [rows_tok][S][n_heads][128] fp16 = acc / l (normalised, so that fp16
@@ -49,6 +59,7 @@ struct AttnArgs {
   // narrow kernel only.  k16/v16 != nullptr (M <= 2): the workgroup whose tiles hold a new row quantizes and stores it
   // before reading it (fused quantize-on-append).
   const uint16_t* k16; const uint16_t* v16;
+  RowMap rows;  // narrow kernel only: multi-stream pass, one token per workgroup column, no depth table, no fused append
 };
 // unrot != 0: the output row gets the inverse signed Hadamard rotation (7 butterfly stages, x 1/16, signs) before it is
 // rounded to fp16 - the counterpart of rotating V rows on their way into the cache (src/q35_kernels.cu:1421)

@@ -53,6 +53,8 @@ def _load():
         "yka_codec_probe": (i32, [vp, i32, vp, vp, vp]),
         "yka_kvx256_probe": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_attn_post": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
+        "yka_append_attend_ms": (i32, [vp, vp, vp, vp, i32, vp, vp, vp, vp]),
+        "yka_ms_call_host": (i32, [vp, vp, vp, vp, i32, vp, vp, vp]),
         "yka_attn_post_host": (i32, [vp, i32, vp, vp, vp, i32, i32, vp, vp, C.c_float, vp, i32, i32, i32, vp]),
         "yka_kv_export_rows": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_kv_import_rows": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
@@ -72,7 +74,7 @@ def _load():
 
 
 EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "yka_set_opt", "yka_kv_set_page_table",
-           "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kvx256_probe", "yka_attn_post",
+           "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kvx256_probe", "yka_attn_post", "yka_append_attend_ms", "yka_ms_call_host",
            "yka_attn_post_host", "yka_kv_export_rows",
            "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
            "yka_append_host", "yka_pass_capture", "yka_pass_launch", "yka_pass_destroy", "yka_attn_bench")
@@ -186,6 +188,23 @@ class KvCache:
     # -- launch path: device addresses --
     def append(self, layer, d_k16, d_v16, M, d_pos, stream=0):
         _chk(lib().yka_append(self._h, layer, d_k16, d_v16, M, d_pos, stream))
+
+    def append_attend_ms(self, d_q16, d_k16, d_v16, M, d_row_pos, d_row_slot, d_out16, stream=0):
+        """Multi-stream pass with device pointers: row t uses container d_row_slot[t] at position d_row_pos[t]."""
+        _chk(lib().yka_append_attend_ms(self._h, d_q16, d_k16, d_v16, M, d_row_pos, d_row_slot, d_out16, stream))
+
+    def ms_call(self, q16, k16, v16, row_pos, row_slot):
+        """Multi-stream pass with host arrays: q16 [M,n_heads,128], k16/v16 [M,n_kv_heads,128] (or None), row_pos/row_slot [M]."""
+        M = q16.shape[0]
+        q = _u16(q16, (M, self.cfg.n_heads, D))
+        k = None if k16 is None else _u16(k16, (M, self.cfg.n_kv_heads, D))
+        v = None if v16 is None else _u16(v16, (M, self.cfg.n_kv_heads, D))
+        rp = np.ascontiguousarray(row_pos, np.int32); rs = np.ascontiguousarray(row_slot, np.int32)
+        if rp.shape != (M,) or rs.shape != (M,):
+            raise ValueError("row_pos and row_slot need one entry per row")
+        out = np.empty((M, self.cfg.n_heads, D), np.uint16)
+        _chk(lib().yka_ms_call_host(self._h, _ptr(q), _ptr(k), _ptr(v), M, _ptr(rp), _ptr(rs), _ptr(out)))
+        return out.view(np.float16)
 
     def attn_post(self, layer, d_xq, d_xk, d_xv, M, d_pos, params, d_q16, stream=0):
         """Device-pointer form: projection outputs -> Q rows in d_q16, K/V rows quantized into the cache (params: PostParams)."""
