@@ -143,15 +143,18 @@ def batched_decode(torch, native, kv, ctx, L, k_new, v_new, q, calls=200):
         dv = torch.from_numpy(np.tile(v_new, (rep, 1, 1))[:B].view(np.int16).copy()).to(dev)
         dout = torch.zeros_like(dq)
         dpos = torch.full((B,), ctx, dtype=torch.int32, device=dev)
-        dslot = torch.arange(B, dtype=torch.int32, device=dev)
-        fn = lambda: kv.append_attend_ms(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, dpos.data_ptr(), dslot.data_ptr(), dout.data_ptr(), stream)
-        for _ in range(10):
-            fn()
+        # consecutive passes take different groups of B containers, so that all L containers (more than the 256 MB
+        # Infinity Cache holds) are streamed before any is read again
+        groups = [torch.arange(g * B, (g + 1) * B, dtype=torch.int32, device=dev) for g in range(L // B)]
+        fn = lambda i: kv.append_attend_ms(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, dpos.data_ptr(),
+                                           groups[i % len(groups)].data_ptr(), dout.data_ptr(), stream)
+        for i in range(10):
+            fn(i)
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
-        for _ in range(calls):
-            fn()
+        for i in range(calls):
+            fn(i)
         e1.record(); torch.cuda.synchronize()
         us = e0.elapsed_time(e1) * 1e3 / calls
         by = B * algorithmic_bytes(ctx, 1)

@@ -39,13 +39,16 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 // 8 codes of one dword -> 4 half2 in element order [n0,n4 | n1,n5 | n2,n6 | n3,n7] holding n-8 for even nibbles and
 // 16(n-8) for odd ones, all exact.  The factor 16 is undone by the query fragment.
-__device__ __forceinline__ void dq_dword_int(uint32_t w, h2* out) {
+// (w & mask) | magic written as a bit-field insert; `magic` (0x64006400, no bit inside either nibble mask) is kept opaque
+// to the optimizer so that the pair is selected as one and-or instruction
+__device__ __forceinline__ uint32_t nib(uint32_t w, uint32_t mask, uint32_t magic) { return (w & mask) | (magic & ~mask); }
+__device__ __forceinline__ void dq_dword_int(uint32_t w, h2* out, uint32_t magic) {
   const h2 c1032 = {(_Float16)1032.f, (_Float16)1032.f}, c1152 = {(_Float16)1152.f, (_Float16)1152.f};
   const uint32_t t = w >> 8;
-  out[0] = as_h2((w & 0x000f000fu) | kMagic) - c1032;
-  out[1] = as_h2((w & 0x00f000f0u) | kMagic) - c1152;
-  out[2] = as_h2((t & 0x000f000fu) | kMagic) - c1032;
-  out[3] = as_h2((t & 0x00f000f0u) | kMagic) - c1152;
+  out[0] = as_h2(nib(w, 0x000f000fu, magic)) - c1032;
+  out[1] = as_h2(nib(w, 0x00f000f0u, magic)) - c1152;
+  out[2] = as_h2(nib(t, 0x000f000fu, magic)) - c1032;
+  out[3] = as_h2(nib(t, 0x00f000f0u, magic)) - c1152;
 }
 
 struct RawTile {       // what one lane holds of a 32-key tile before dequantization
@@ -57,18 +60,28 @@ struct RawTile {       // what one lane holds of a 32-key tile before dequantiza
 // token slot e of lane group g inside a 32-key tile: the keys whose scores this lane receives from the two score MFMAs
 __device__ __forceinline__ int tau(int g, int e) { return 16 * (e >> 2) + 4 * g + (e & 3); }
 
-// pg = start of the (page, kv head) block, tp = index of the tile's first token inside the page
-__device__ __forceinline__ void load_tile(const uint8_t* pg, int tp, int i, int g, RawTile& R) {
+// Byte offsets of one lane inside a page, fixed for the whole kernel.  The page pointer and the tile's first token are
+// wave uniform, so every load is "scalar base + 32-bit lane offset + immediate".
+struct LaneOffs { uint32_t kc, ks, vs, vc; };
+__device__ __forceinline__ LaneOffs lane_offs(int i, int g) {
+  return LaneOffs{kPageKc + (uint32_t)i * 64u + 16u * g, kPageKs + 32u * g, kPageVs + ((uint32_t)(i >> 2) * kPageTok + 4u * g) * 2u,
+                  kPageVc + 256u * g + 4u * i};
+}
+// pg = start of the (page, kv head) block, tp = index of the tile's first token inside the page (both wave uniform)
+__device__ __forceinline__ void load_tile(const uint8_t* pg, int tp, const LaneOffs& L, RawTile& R) {
+  const uint8_t* c64 = pg + (uint32_t)tp * 64u;     // code rows (K and V planes) of the tile
+  const uint8_t* s8 = pg + (uint32_t)tp * 8u;       // K scale rows
+  const uint8_t* s2 = pg + (uint32_t)tp * 2u;       // V scale columns
 #pragma unroll
   for (int kt = 0; kt < 2; ++kt) {
-    R.kw[kt] = *reinterpret_cast<const uint4*>(pg + kPageKc + (size_t)(tp + 16 * kt + i) * 64 + 16 * g);
-    const uint4* sp = reinterpret_cast<const uint4*>(pg + kPageKs + (size_t)(tp + 16 * kt + 4 * g) * 8);
-    R.ks[kt][0] = sp[0]; R.ks[kt][1] = sp[1];
-    R.vs[kt] = *reinterpret_cast<const uint2*>(pg + kPageVs + ((size_t)(i >> 2) * kPageTok + tp + 16 * kt + 4 * g) * 2);
+    R.kw[kt] = *reinterpret_cast<const uint4*>(c64 + L.kc + 1024 * kt);
+    R.ks[kt][0] = *reinterpret_cast<const uint4*>(s8 + L.ks + 128 * kt);
+    R.ks[kt][1] = *reinterpret_cast<const uint4*>(s8 + L.ks + 128 * kt + 16);
+    R.vs[kt] = *reinterpret_cast<const uint2*>(s2 + L.vs + 32 * kt);
   }
 #pragma unroll
-  for (int e = 0; e < 8; ++e)
-    R.vw[e] = *reinterpret_cast<const uint32_t*>(pg + kPageVc + (size_t)(tp + tau(g, e)) * 64 + 4 * i);
+  for (int e = 0; e < 8; ++e)                        // token tau(g, e) = 16 (e >> 2) + 4 g + (e & 3)
+    R.vw[e] = *reinterpret_cast<const uint32_t*>(c64 + L.vc + (16 * (e >> 2) + (e & 3)) * 64);
 }
 
 // grid (S, n_kv, ceil(M/TPT)), block 256 (4 waves).  Workgroup = (split, kv head, row tile of TPT tokens x 6 heads):
@@ -80,7 +93,8 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
   __shared__ float s_acc[4][16][kD + 4];
   constexpr int TPT = MS ? 1 : 2;
   const int split = blockIdx.x, kvh = blockIdx.y, rt = blockIdx.z;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // a scalar: tile indices and page pointers are wave uniform
+  const int lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
   int pos; bool row_ok = true;
   if (MS) {
     pos = A.rows.pos[rt];
@@ -101,9 +115,10 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
     else { const int tg = A.tok0 + tl; len = pos + (A.depth ? (int)A.depth[tg] : tg) + 1; }
     len = min(len, A.kv.max_ctx);
   }
-  int maxlen = len;
+  int maxlen = len, minlen = vrow ? len : 0x7fffffff;
 #pragma unroll
-  for (int o = 1; o < 16; o <<= 1) maxlen = max(maxlen, __shfl_xor(maxlen, o, 64));
+  for (int o = 1; o < 16; o <<= 1) { maxlen = max(maxlen, __shfl_xor(maxlen, o, 64)); minlen = min(minlen, __shfl_xor(minlen, o, 64)); }
+  maxlen = __builtin_amdgcn_readfirstlane(maxlen); minlen = __builtin_amdgcn_readfirstlane(minlen);
   const int ntiles = (maxlen + 31) >> 5, tps = (ntiles + A.S - 1) / A.S;
   const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
 
@@ -149,9 +164,13 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
   for (int b = 0; b < 8; ++b) o[b] = f4{0.f, 0.f, 0.f, 0.f};
 
   RawTile cur;
+  const LaneOffs offs = lane_offs(i, g);
+  uint32_t magic = kMagic;
+  asm volatile("" : "+v"(magic));
   for (int T = tile0 + wave; T < tile1; T += 4) {
-    load_tile(kv_page(A.kv, kvh, T << 5), (T << 5) % kPageTok, i, g, cur);
+    load_tile(kv_page(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, cur);
     const int t0 = T << 5;
+    const bool need_mask = t0 + 32 > minlen;         // wave uniform: only the last tiles of a row can hold keys past its length
     // ---- scores: two 16-key MFMA tiles; step m contracts scale group m, its fp32 sum is scaled afterwards ----
     float s[8];
 #pragma unroll
@@ -161,7 +180,7 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         h2 k4[4];
-        dq_dword_int(w[m], k4);
+        dq_dword_int(w[m], k4, magic);
         const h8 kf = h8{k4[0][0], k4[0][1], k4[1][0], k4[1][1], k4[2][0], k4[2][1], k4[3][0], k4[3][1]};
         part[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[m], f4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
       }
@@ -171,10 +190,16 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const h2 s01 = as_h2(sw[2 * r]), s23 = as_h2(sw[2 * r + 1]);
-        const float dot = part[0][r] * (float)s01[0] + part[1][r] * (float)s01[1] + part[2][r] * (float)s23[0] + part[3][r] * (float)s23[1];
-        const int key = t0 + 16 * kt + 4 * g + r;
-        s[4 * kt + r] = key < len ? dot * sc_log2 : -INFINITY;
+        float dot = __builtin_fmaf(part[0][r], (float)s01[0], 0.f);
+        dot = __builtin_fmaf(part[1][r], (float)s01[1], dot);
+        dot = __builtin_fmaf(part[2][r], (float)s23[0], dot);
+        dot = __builtin_fmaf(part[3][r], (float)s23[1], dot);
+        s[4 * kt + r] = dot;                           // raw units; log2(e)/sqrt(d) is folded into the exponent below
       }
+    }
+    if (need_mask) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { const int key = t0 + 16 * (e >> 2) + 4 * g + (e & 3); s[e] = key < len ? s[e] : -INFINITY; }
     }
     // ---- online softmax (one running maximum per row, shared by its 4 lane groups) ----
     float tmax = s[0];
@@ -182,17 +207,18 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
     for (int e = 1; e < 8; ++e) tmax = fmaxf(tmax, s[e]);
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m_run, tmax);
-    const float alpha = exp2f(m_run - m_new);
+    const float m_new = fmaxf(m_run, tmax * sc_log2);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);    // 0 on the first tile (m_run = -1e30): nothing to rescale yet
+    const bool first = m_run < -1e29f;
     m_run = m_new;
-    if (__any(alpha != 1.f)) {
+    if (__any(alpha != 1.f && !first)) {
       l_run *= alpha;
 #pragma unroll
       for (int b = 0; b < 8; ++b) { o[b][0] *= alpha; o[b][1] *= alpha; o[b][2] *= alpha; o[b][3] *= alpha; }
     }
     h8 pf;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) { const float p = exp2f(s[e] - m_new); l_run += p; pf[e] = (_Float16)p; }
+    for (int e = 0; e < 8; ++e) { const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], sc_log2, -m_new)); l_run += p; pf[e] = (_Float16)p; }
     // ---- O^T += V^T P^T : 8 MFMAs, MFMA b covers channels 8*i' + b ----
     h2 va[8][4];
 #pragma unroll
@@ -204,9 +230,9 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
 #pragma unroll
       for (int bb = 0; bb < 4; ++bb) {
         // byte bb of both tokens side by side: low half = token 2pe, high half = token 2pe+1
-        const uint32_t x = ((w0 >> (8 * bb)) & 0xffu) | (((w1 >> (8 * bb)) & 0xffu) << 16);
-        va[2 * bb][pe] = (as_h2((x & 0x000f000fu) | kMagic) - c1032) * s2;
-        va[2 * bb + 1][pe] = (as_h2((x & 0x00f000f0u) | kMagic) - c1152) * s2q;
+        const uint32_t x = __builtin_amdgcn_perm(w1, w0, 0x0c040c00u + bb * 0x00010001u);
+        va[2 * bb][pe] = (as_h2(nib(x, 0x000f000fu, magic)) - c1032) * s2;
+        va[2 * bb + 1][pe] = (as_h2(nib(x, 0x00f000f0u, magic)) - c1152) * s2q;
       }
     }
 #pragma unroll
