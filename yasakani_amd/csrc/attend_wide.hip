@@ -173,23 +173,34 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
       for (int r = 0; r < 16; ++r) o[rt][dt][r] = 0.f;
   }
 
-  Raw raw;
+  Raw raw0, raw1;                              // raw codes of the next two tiles: loads run two tiles ahead of their use
   KScales sc;
   const LaneOffs offs = lane_offs(tid, h);
   uint32_t magic = kMagic;
   asm volatile("" : "+v"(magic));
+  auto load_tile_raw = [&](int T, Raw& r) { load_raw(kv_page(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, r); };
   if (tile0 < tile1) {
-    load_raw(kv_page(A.kv, kvh, tile0 << 5), (tile0 << 5) % kPageTok, offs, raw);
+    load_tile_raw(tile0, raw0);
     load_kscales(kv_page(A.kv, kvh, tile0 << 5), (tile0 << 5) % kPageTok, offs, sc);
-    dequant_to_lds(lds[0], tid, raw, magic);
-    if (tile0 + 1 < tile1) load_raw(kv_page(A.kv, kvh, (tile0 + 1) << 5), ((tile0 + 1) << 5) % kPageTok, offs, raw);
+    dequant_to_lds(lds[0], tid, raw0, magic);
+    if (tile0 + 1 < tile1) load_tile_raw(tile0 + 1, raw1);
+    if (tile0 + 2 < tile1) load_tile_raw(tile0 + 2, raw0);
   }
   __syncthreads();
-  for (int T = tile0; T < tile1; ++T) {
-    const int cb = (T - tile0) & 1;
+  // One tile: `rs` holds the raw codes of tile T+1, which are dequantized into the other LDS buffer and replaced by the
+  // request for tile T+3; cb (the LDS buffer of tile T) is a literal at both call sites.
+  auto tile_step = [&](const int T, const int cb, Raw& rs) {
+    // all K fragments of tile T are requested before anything else, so that their LDS latency runs under the
+    // dequantization of tile T+1
+    h8 kfr[8];
+    if (nrt > 0) {
+#pragma unroll
+      for (int c = 0; c < 8; ++c)
+        kfr[c] = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(lds[cb] + kLdsK + j * kKPitch + (4 * (c >> 1) + 2 * (c & 1) + h) * 16));
+    }
     if (T + 1 < tile1) {
-      dequant_to_lds(lds[cb ^ 1], tid, raw, magic);                   // tile T+1 (loaded one iteration ago)
-      if (T + 2 < tile1) load_raw(kv_page(A.kv, kvh, (T + 2) << 5), ((T + 2) << 5) % kPageTok, offs, raw);
+      dequant_to_lds(lds[cb ^ 1], tid, rs, magic);
+      if (T + 3 < tile1) load_tile_raw(T + 3, rs);
     }
     const uint8_t* buf = lds[cb];
     const int t0 = T << 5;
@@ -201,8 +212,7 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
       float s[RT][16];
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
-        const h8 k0 = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsK + j * kKPitch + (4 * m + h) * 16));
-        const h8 k1 = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsK + j * kKPitch + (4 * m + 2 + h) * 16));
+        const h8 k0 = kfr[2 * m], k1 = kfr[2 * m + 1];
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
           {                                    // row tiles past the wave's last row run on zero queries; nothing of them is stored
@@ -222,6 +232,11 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
           }
         }
       }
+      // all V fragments are requested here: their LDS latency runs under the softmax arithmetic
+      h8 vfr[8];
+#pragma unroll
+      for (int c = 0; c < 8; ++c)
+        vfr[c] = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsV + (32 * (c >> 1) + j) * kVPitch + (16 * (c & 1) + 8 * h) * 2));
 #pragma unroll
       for (int rt = 0; rt < RT; ++rt) {
         {
@@ -264,13 +279,17 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
       for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-          const h8 vf = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsV + (32 * dt + j) * kVPitch + (16 * u + 8 * h) * 2));
+          const h8 vf = vfr[2 * dt + u];
 #pragma unroll
           for (int rt = 0; rt < RT; ++rt)
             o[rt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[rt][u], o[rt][dt], 0, 0, 0);
         }
     }
     __syncthreads();
+  };
+  for (int T = tile0; T < tile1; T += 2) {
+    tile_step(T, 0, raw1);
+    if (T + 1 < tile1) tile_step(T + 1, 1, raw0);
   }
   // ---- partials: normalised fp16.  o[dt][4a+b] of lane (row j, half h) is V-image row 32dt + 8a + 4h + b, i.e.
   //      channel 64(a&1) + 32h + 8b + 4(a>>1) + dt: for each (a&1, b) the lane owns 8 consecutive channels.
