@@ -168,7 +168,7 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
   uint32_t magic = kMagic;
   asm volatile("" : "+v"(magic));
   for (int T = tile0 + wave; T < tile1; T += 4) {
-    load_tile(kv_page(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, cur);
+    load_tile(kv_page_uniform(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, cur);
     const int t0 = T << 5;
     const bool need_mask = t0 + 32 > minlen;         // wave uniform: only the last tiles of a row can hold keys past its length
     // ---- scores: two 16-key MFMA tiles; step m contracts scale group m, its fp32 sum is scaled afterwards ----

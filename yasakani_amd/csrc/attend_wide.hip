@@ -178,10 +178,10 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
   const LaneOffs offs = lane_offs(tid, h);
   uint32_t magic = kMagic;
   asm volatile("" : "+v"(magic));
-  auto load_tile_raw = [&](int T, Raw& r) { load_raw(kv_page(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, r); };
+  auto load_tile_raw = [&](int T, Raw& r) { load_raw(kv_page_uniform(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, r); };
   if (tile0 < tile1) {
     load_tile_raw(tile0, raw0);
-    load_kscales(kv_page(A.kv, kvh, tile0 << 5), (tile0 << 5) % kPageTok, offs, sc);
+    load_kscales(kv_page_uniform(A.kv, kvh, tile0 << 5), (tile0 << 5) % kPageTok, offs, sc);
     dequant_to_lds(lds[0], tid, raw0, magic);
     if (tile0 + 1 < tile1) load_tile_raw(tile0 + 1, raw1);
     if (tile0 + 2 < tile1) load_tile_raw(tile0 + 2, raw0);
@@ -273,7 +273,7 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
         }
       }
       // scales of the next tile: requested now, needed after the next barrier
-      if (T + 1 < tile1) load_kscales(kv_page(A.kv, kvh, (T + 1) << 5), ((T + 1) << 5) % kPageTok, offs, sc);
+      if (T + 1 < tile1) load_kscales(kv_page_uniform(A.kv, kvh, (T + 1) << 5), ((T + 1) << 5) % kPageTok, offs, sc);
       // ---- O^T += V^T P^T : d-tile dt (32 rows of the V image), k-step u (16 tokens) ----
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)

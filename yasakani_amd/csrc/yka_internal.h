@@ -95,4 +95,16 @@ __device__ __forceinline__ uint8_t* kv_page(const KvView& kv, int kvh, int t) {
   return kv.base + (size_t)(pp * kv.n_kv + kvh) * kPageBytes;
 }
 
+// The same for a token index that is uniform over the wave (the attention kernels' tile loops).  The page-table entry is
+// fetched through the scalar data path: a vector load would share its completion counter with the tile loads a wave
+// keeps in flight, so waiting for the entry would wait for all of them.  (Read only; the table is written by the host.)
+__device__ __forceinline__ uint8_t* kv_page_uniform(const KvView& kv, int kvh, int t) {
+  const int lp = t / kPageTok;
+  int pp = lp;
+  if (kv.table) {
+    asm volatile("s_load_dword %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=s"(pp) : "s"(kv.table), "s"(lp * 4) : "memory");
+  }
+  return kv.base + (size_t)(pp * kv.n_kv + kvh) * kPageBytes;
+}
+
 }  // namespace yka
