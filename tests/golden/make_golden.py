@@ -6,7 +6,7 @@ comes from the reference: the fixtures freeze the oracle's outputs on small seed
 has been pinned by tests/test_oracle_*.py), so that (i) a later change of the oracle is noticed and (ii) the GPU
 tests can compare against committed data.
 
-    python tests/golden/make_golden.py        # rewrites codec_v1.npz and attention_v1.npz
+    python tests/golden/make_golden.py        # rewrites codec_v1.npz, attention_v1.npz, row256_v1.npz and post_v1.npz
 """
 import os
 import sys
@@ -56,8 +56,54 @@ def attention_fixture():
     np.savez_compressed(os.path.join(HERE, "attention_v1.npz"), **cases)
 
 
+def row256_fixture():
+    """The reference's own 256-channel row format: rotation, flat int4 (MSB-first words, fp32 scale) and int8 rows."""
+    rng = np.random.default_rng(20261126)
+    x = (rng.standard_normal((24, 256)) * (10.0 ** rng.uniform(-3, 2, (24, 1)))).astype(np.float32)
+    x[0] = 0.0
+    x[1] = 0.0; x[1, 200] = -3.0
+    x[2] = np.round(x[2] * 4)
+    out = {"x": x}
+    for mode in (0, 1):
+        for rot in (0, 1):
+            q8, words, scales, y = yko.kvx_probe256(x, mode, rot)
+            tag = f"m{mode}r{rot}"
+            out[tag + ".scales_bits"] = scales.view(np.uint32)
+            out[tag + ".y_bits"] = y.view(np.uint32)
+            if mode == 0:
+                out[tag + ".q8"] = q8
+            else:
+                out[tag + ".words"] = words
+    np.savez_compressed(os.path.join(HERE, "row256_v1.npz"), **out)
+
+
+def post_fixture():
+    """The step between the QKV projection and the cache: fp32 rows in, fp16 Q rows and int4 cache rows out."""
+    rng = np.random.default_rng(20261127)
+    M, rd, pos, ctx = 6, 32, 250, 512
+    xq = (rng.standard_normal((M, 24, 128)) * 2).astype(np.float32)
+    xk = (rng.standard_normal((M, 4, 128)) * 0.7).astype(np.float32)
+    xk[:, :, [3, 40, 77, 120]] *= 8
+    xv = rng.standard_normal((M, 4, 128)).astype(np.float32)
+    xq[1] = 0; xk[1] = 0; xv[1] = 0
+    qw = (rng.standard_normal(128) * 0.1).astype(np.float16).view(np.uint16)
+    kw = (rng.standard_normal(128) * 0.1).astype(np.float16).view(np.uint16)
+    rope = yko.rope_table(ctx, rd)
+    out = {"xq": xq, "xk": xk, "xv": xv, "qw": qw, "kw": kw, "rope": rope, "rd": np.int32(rd), "pos": np.int32(pos),
+           "eps": np.float32(1e-6), "ctx": np.int32(ctx)}
+    for rot in (0, 1):
+        q16, k16, v16 = yko.attn_post(xq, xk, xv, qw, kw, 1e-6, rope, rd, pos, rot)
+        c = yko.Cache(ctx)
+        c.append(k16, v16, pos)
+        sl = slice(pos, pos + M)
+        out.update({f"r{rot}.q16": q16, f"r{rot}.kc": c.kc[:, sl], f"r{rot}.ks": c.ks[:, sl], f"r{rot}.vc": c.vc[:, sl], f"r{rot}.vs": c.vs[:, sl]})
+    np.savez_compressed(os.path.join(HERE, "post_v1.npz"), **out)
+
+
 if __name__ == "__main__":
     codec_fixture()
     attention_fixture()
-    for f in ("codec_v1.npz", "attention_v1.npz"):
+    row256_fixture()
+    post_fixture()
+    for f in ("codec_v1.npz", "attention_v1.npz", "row256_v1.npz", "post_v1.npz"):
         print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

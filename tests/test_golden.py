@@ -62,3 +62,53 @@ def test_gpu_reproduces_attention_fixture(native, case):
     assert (got[0] == g[f"{case}.kc"][:, ctx:]).all() and (got[1] == g[f"{case}.ks"][:, ctx:]).all()
     assert (got[2] == g[f"{case}.vc"][:, ctx:]).all() and (got[3] == g[f"{case}.vs"][:, ctx:]).all()
     assert_attn_close(out, g[f"{case}.out32"], case)
+
+
+# ---- the reference's own 256-channel row format, and the step between the QKV projection and the cache ----
+
+def _check_row256(probe, g):
+    for mode in (0, 1):
+        for rot in (0, 1):
+            q8, words, scales, y = probe(g["x"], mode, rot)
+            tag = f"m{mode}r{rot}"
+            assert (scales.view(np.uint32) == g[tag + ".scales_bits"]).all(), tag
+            assert (y.view(np.uint32) == g[tag + ".y_bits"]).all(), tag
+            if mode == 0:
+                assert (q8 == g[tag + ".q8"]).all(), tag
+            else:
+                assert (words == g[tag + ".words"]).all(), tag
+
+
+def test_oracle_reproduces_row256_fixture(oracle):
+    _check_row256(oracle.kvx_probe256, _load("row256_v1.npz"))
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_row256_fixture(native):
+    _check_row256(native.kvx256_probe, _load("row256_v1.npz"))
+
+
+def test_oracle_reproduces_post_fixture(oracle):
+    g = _load("post_v1.npz")
+    M, pos, ctx = g["xq"].shape[0], int(g["pos"]), int(g["ctx"])
+    for rot in (0, 1):
+        q16, k16, v16 = oracle.attn_post(g["xq"], g["xk"], g["xv"], g["qw"], g["kw"], float(g["eps"]), g["rope"], int(g["rd"]), pos, rot)
+        c = oracle.Cache(ctx)
+        c.append(k16, v16, pos)
+        sl = slice(pos, pos + M)
+        assert (q16 == g[f"r{rot}.q16"]).all()
+        for name, arr in (("kc", c.kc), ("ks", c.ks), ("vc", c.vc), ("vs", c.vs)):
+            assert (arr[:, sl] == g[f"r{rot}.{name}"]).all(), name
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_post_fixture(native):
+    g = _load("post_v1.npz")
+    M, pos, ctx = g["xq"].shape[0], int(g["pos"]), int(g["ctx"])
+    for rot in (0, 1):
+        with native.KvCache(max_ctx=ctx) as kv:
+            q16 = kv.attn_post_host(0, g["xq"], g["xk"], g["xv"], pos, g["qw"], g["kw"], float(g["eps"]), g["rope"], int(g["rd"]), rotate=bool(rot))
+            got = kv.export_rows(0, pos, M)
+        assert (q16.view(np.uint16) == g[f"r{rot}.q16"]).all()
+        for arr, name in zip(got, ("kc", "ks", "vc", "vs")):
+            assert (arr == g[f"r{rot}.{name}"]).all(), name
