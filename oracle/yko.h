@@ -19,6 +19,8 @@
  *                            split-count independence, uniform-V / dominant-key
  *                            closed forms, window == single rows
  *   yko_attend_f64           pinned: same closed forms + numpy
+ *   (both, cache format 1)   pinned: numpy softmax on rows decoded with numpy bit unpacking, split independence,
+ *                            window == single rows, uniform-V / dominant-key closed forms (head_dim 256)
  *   yko_combine              pinned: algebraic identity vs unsplit evaluation,
  *                            empty-split sentinel
  *   yko_kvx_sign             pinned: independent arbitrary-precision evaluation of the integer hash
@@ -86,7 +88,14 @@ void yko_unrotate_out(const float* y32, int rows, uint16_t* out16);
 typedef struct {
   int n_heads, n_kv_heads, head_dim, max_ctx;
   uint8_t* kc; uint16_t* ks; uint8_t* vc; uint16_t* vs;
+  /* fmt 0: the format above.  fmt 1 (head_dim 256 only): the reference's own rows - kc/vc point to uint32 words
+   * [kvh][max_ctx][32] (4-bit fields, MSB first), ks/vs to float scales [kvh][max_ctx], one per row
+   * (src/kvq_fast.cuh:194-198,226-233).  Append widens the fp16 inputs to fp32 and encodes them with
+   * yko_flat4_encode256; attention decodes rows with yko_flat4_decode256. */
+  int fmt;
 } yko_cache;
+/* row `row` (= kvh * max_ctx + token) of K (isv 0) or V (isv 1), dequantized to fp32 */
+void yko_cache_row(const yko_cache* c, int isv, size_t row, float* out);
 
 /* quantize-on-append (reference ordering: src/engine35.cpp:911-913 - rows are written before attention reads them;
  * row placement src/q35_kernels.cu:1038,1064): k16/v16 [M][kvh][dim] -> rows pos..pos+M-1 */

@@ -26,7 +26,7 @@ def build(force=False):
 
 class _Cache(C.Structure):
     _fields_ = [("n_heads", C.c_int), ("n_kv_heads", C.c_int), ("head_dim", C.c_int), ("max_ctx", C.c_int),
-                ("kc", C.c_void_p), ("ks", C.c_void_p), ("vc", C.c_void_p), ("vs", C.c_void_p)]
+                ("kc", C.c_void_p), ("ks", C.c_void_p), ("vc", C.c_void_p), ("vs", C.c_void_p), ("fmt", C.c_int)]
 
 
 _lib = None
@@ -120,18 +120,25 @@ def unpack_nibbles(bytes_):
 
 
 class Cache:
-    """Canonical cache image of one layer: kc/vc [kvh, max_ctx, 64] u8, ks/vs [kvh, max_ctx, 4] u16."""
+    """Canonical cache image of one layer.  head_dim 128: kc/vc [kvh, max_ctx, 64] u8, ks/vs [kvh, max_ctx, 4] u16
+    (int4 in 32-channel groups with fp16 scales).  head_dim 256: the reference's own rows - kc/vc [kvh, max_ctx, 32] u32
+    (MSB-first 4-bit fields), ks/vs [kvh, max_ctx] f32, one scale per row."""
 
     def __init__(self, max_ctx, n_heads=24, n_kv_heads=4, head_dim=D):
         self.n_heads, self.n_kv_heads, self.head_dim, self.max_ctx = n_heads, n_kv_heads, head_dim, max_ctx
-        self.kc = np.zeros((n_kv_heads, max_ctx, head_dim // 2), np.uint8)
+        self.fmt = 1 if head_dim == 256 else 0
+        if self.fmt:
+            self.kc = np.zeros((n_kv_heads, max_ctx, 32), np.uint32)
+            self.ks = np.zeros((n_kv_heads, max_ctx), np.float32)
+        else:
+            self.kc = np.zeros((n_kv_heads, max_ctx, head_dim // 2), np.uint8)
+            self.ks = np.zeros((n_kv_heads, max_ctx, head_dim // GROUP), np.uint16)
         self.vc = np.zeros_like(self.kc)
-        self.ks = np.zeros((n_kv_heads, max_ctx, head_dim // GROUP), np.uint16)
         self.vs = np.zeros_like(self.ks)
 
     def _c(self):
         return _Cache(self.n_heads, self.n_kv_heads, self.head_dim, self.max_ctx,
-                      self.kc.ctypes.data, self.ks.ctypes.data, self.vc.ctypes.data, self.vs.ctypes.data)
+                      self.kc.ctypes.data, self.ks.ctypes.data, self.vc.ctypes.data, self.vs.ctypes.data, self.fmt)
 
     def append(self, k16, v16, pos):
         k = _as_u16(k16); v = _as_u16(v16)

@@ -32,7 +32,7 @@ static inline float dot16(const float* a, const float* b, int D) {
  *   mn = max(m, s); e = exp(min(m,s) - mn); a = s > m ? e : 1; b = s > m ? 1 : e; l = l*a + b; acc = acc*a + b*v. */
 static void split_task(const yko_cache* c, const float* qf /* [M][NH][D], pre-scaled */, int M, int pos, const uint8_t* depth,
                        int kvh, int split, int splits_arg, int Smax, float* pm, float* pl, float* pacc) {
-  const int D = c->head_dim, NH = c->n_heads, G = NH / c->n_kv_heads, ng = D / YKO_GROUP;
+  const int D = c->head_dim, NH = c->n_heads, G = NH / c->n_kv_heads;
   int lo_all = 0x7fffffff, hi_all = 0;
   int* lo = (int*)malloc(sizeof(int) * 2 * (size_t)M);
   int* hi = lo + M;
@@ -50,8 +50,8 @@ static void split_task(const yko_cache* c, const float* qf /* [M][NH][D], pre-sc
   float kd[YKO_MAXD], vd[YKO_MAXD];
   for (int key = lo_all; key < hi_all; ++key) {
     const size_t row = (size_t)kvh * c->max_ctx + key;
-    yko_dequant_rows(c->kc + row * (D / 2), c->ks + row * ng, 1, D, kd);
-    yko_dequant_rows(c->vc + row * (D / 2), c->vs + row * ng, 1, D, vd);
+    yko_cache_row(c, 0, row, kd);
+    yko_cache_row(c, 1, row, vd);
     for (int t = 0; t < M; ++t) {
       if (key < lo[t] || key >= hi[t]) continue;
       for (int i = 0; i < G; ++i) {
@@ -134,7 +134,7 @@ void yko_attend_f32(const yko_cache* c, const uint16_t* q16, int M, int pos, con
 
 /* textbook: scores in double, subtract the row maximum, exponentiate, normalise, weight V */
 void yko_attend_f64(const yko_cache* c, const uint16_t* q16, int M, int pos, const uint8_t* depth, double* out64) {
-  const int D = c->head_dim, NH = c->n_heads, KVH = c->n_kv_heads, G = NH / KVH, ng = D / YKO_GROUP;
+  const int D = c->head_dim, NH = c->n_heads, KVH = c->n_kv_heads, G = NH / KVH;
   const double qs = 1.0 / sqrt((double)D);
   int maxlen = 0;
   for (int t = 0; t < M; ++t) { const int l = row_len(pos, depth, t); if (l > maxlen) maxlen = l; }
@@ -148,7 +148,7 @@ void yko_attend_f64(const yko_cache* c, const uint16_t* q16, int M, int pos, con
       double mx = -INFINITY;
       for (int key = 0; key < len; ++key) {
         const size_t row = (size_t)kvh * c->max_ctx + key;
-        yko_dequant_rows(c->kc + row * (D / 2), c->ks + row * ng, 1, D, kd);
+        yko_cache_row(c, 0, row, kd);
         double s = 0.0;
         for (int d = 0; d < D; ++d) s += (double)yko_h2f(q[d]) * (double)kd[d];
         s *= qs; sc[key] = s; if (s > mx) mx = s;
@@ -158,7 +158,7 @@ void yko_attend_f64(const yko_cache* c, const uint16_t* q16, int M, int pos, con
       for (int key = 0; key < len; ++key) {
         const double w = exp(sc[key] - mx); L += w;
         const size_t row = (size_t)kvh * c->max_ctx + key;
-        yko_dequant_rows(c->vc + row * (D / 2), c->vs + row * ng, 1, D, kd);
+        yko_cache_row(c, 1, row, kd);
         for (int d = 0; d < D; ++d) o[d] += w * (double)kd[d];
       }
       for (int d = 0; d < D; ++d) o[d] /= L;

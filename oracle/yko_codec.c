@@ -100,12 +100,32 @@ void yko_dequant_rows(const uint8_t* codes, const uint16_t* scales, int rows, in
 
 /* rows pos..pos+M-1 of every KV head are (over)written before any row of the pass is read
  * (src/engine35.cpp:911-913; row index src/q35_kernels.cu:42) */
+void yko_cache_row(const yko_cache* c, int isv, size_t row, float* out) {
+  const int D = c->head_dim;
+  if (c->fmt == 1) {
+    const uint32_t* words = (const uint32_t*)(isv ? c->vc : c->kc) + row * 32;
+    yko_flat4_decode256(words, ((const float*)(isv ? c->vs : c->ks))[row], out);
+  } else {
+    const int ng = D / YKO_GROUP;
+    yko_dequant_rows((isv ? c->vc : c->kc) + row * (D / 2), (isv ? c->vs : c->ks) + row * ng, 1, D, out);
+  }
+}
+
 void yko_append(yko_cache* c, const uint16_t* k16, const uint16_t* v16, int M, int pos) {
   const int D = c->head_dim, ng = D / YKO_GROUP, KVH = c->n_kv_heads;
   for (int t = 0; t < M; ++t)
     for (int h = 0; h < KVH; ++h) {
       const size_t row = (size_t)h * c->max_ctx + (size_t)(pos + t);
       const size_t src = ((size_t)t * KVH + h) * D;
+      if (c->fmt == 1) {                 /* D == 256: the reference's row codec on the fp32 value of every fp16 input */
+        float x[256];
+        for (int isv = 0; isv < 2; ++isv) {
+          const uint16_t* s16 = (isv ? v16 : k16) + src;
+          for (int d = 0; d < 256; ++d) x[d] = yko_h2f(s16[d]);
+          yko_flat4_encode256(x, (uint32_t*)(isv ? c->vc : c->kc) + row * 32, (float*)(isv ? c->vs : c->ks) + row, NULL);
+        }
+        continue;
+      }
       yko_quant_rows(k16 + src, 1, D, c->kc + row * (D / 2), c->ks + row * ng);
       yko_quant_rows(v16 + src, 1, D, c->vc + row * (D / 2), c->vs + row * ng);
     }
