@@ -13,8 +13,15 @@
  * One caller at a time per handle; any host thread may call (the device of the handle is made current first,
  * as on_gpu does in c_api.cpp:22-31).
  *
- * Fixed format: head_dim 128; symmetric signed int4 codes stored as q+8, two per byte, even channel in the low
- * nibble; one fp16 scale per (token, kv head, 32-channel group); Q, new K/V and outputs are fp16 bit patterns.
+ * Formats, selected by head_dim at open:
+ *   128: symmetric signed int4 codes stored as q+8, two per byte, even channel in the low nibble; one fp16 scale per
+ *        (token, kv head, 32-channel group) - the measured format; every entry point below exists for it;
+ *   256: the reference's own rows - flat int4 with ONE fp32 scale per (token, kv head) row, 4-bit fields MSB first in
+ *        32 uint32 words (kvq_fast.cuh:194-198,226-233; decode kvq_attn.cuh:33-37,53-54).  Open / close / options /
+ *        page table / append / attend / append_attend / layer_call_host / append_host / replicate / captured passes /
+ *        attn_bench work on it; its canonical image goes through yka_kv_export_rows256 / yka_kv_import_rows256; the
+ *        other entry points return an error.
+ * Q, new K/V and outputs are fp16 bit patterns, [rows][heads][head_dim].
  */
 #ifndef YKA_ABI_H
 #define YKA_ABI_H
@@ -31,7 +38,7 @@ typedef struct yka_kv_config {
   int32_t n_layers;    /* KV containers (the reference keeps one per full-attention layer, engine35.cpp:303-329) */
   int32_t n_heads;     /* query heads (24) */
   int32_t n_kv_heads;  /* KV heads (4); n_heads / n_kv_heads must be 6 */
-  int32_t head_dim;    /* 128 */
+  int32_t head_dim;    /* 128, or 256 for the reference's own rows */
   int32_t max_ctx;     /* tokens reserved per layer; multiple of 256 */
   int32_t max_rows;    /* most query rows one call may carry (64 = kVerifyMax, engine35.hpp:157; up to 2048 = PM_ for prefill) */
   int32_t paged;       /* 0: token t of a KV head lives in page t/256; 1: pages go through a per-layer page table */
@@ -140,6 +147,10 @@ YKA_API int yka_kvx256_probe(const float* x, int rows, int mode, int rot, int8_t
 YKA_API int yka_kv_export_rows(yka_kv* kv, int layer, int pos0, int n, uint8_t* kc, uint16_t* ks, uint8_t* vc, uint16_t* vs);
 YKA_API int yka_kv_import_rows(yka_kv* kv, int layer, int pos0, int n, const uint8_t* kc, const uint16_t* ks,
                                const uint8_t* vc, const uint16_t* vs);
+/* The same for head_dim 256: kw/vw [n_kv_heads][n][32] uint32 words, ks/vs [n_kv_heads][n] fp32 row scales. */
+YKA_API int yka_kv_export_rows256(yka_kv* kv, int layer, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs);
+YKA_API int yka_kv_import_rows256(yka_kv* kv, int layer, int pos0, int n, const uint32_t* kw, const float* ks,
+                                  const uint32_t* vw, const float* vs);
 /* dequantize rows on the GPU (decoder probe, replaces tba_unpack_kernel's use in yskn_tbp_pack_unpack,
  * kvx_probe.cu:123-170): k, v [n_kv_heads][n][128] fp32 */
 YKA_API int yka_kv_dequant_rows(yka_kv* kv, int layer, int pos0, int n, float* k, float* v);

@@ -1,0 +1,97 @@
+"""The reference's own rows on the GPU (head_dim 256, flat int4, one fp32 scale per row, MSB-first words) against the
+oracle: appended words and scales bit-exact, attention outputs within the attention bars."""
+import numpy as np
+import pytest
+
+from tolerances import assert_attn_close
+
+pytestmark = pytest.mark.gpu
+NH, KVH, D = 24, 4, 256
+
+
+def _inputs(seed, ctx, M):
+    rng = np.random.default_rng(seed)
+    q = rng.standard_normal((M, NH, D)).astype(np.float16)
+    k = rng.standard_normal((ctx + M, KVH, D)).astype(np.float32)
+    k[:, :, [5, 77, 130, 201]] *= 8                       # outlier channels
+    v = rng.standard_normal((ctx + M, KVH, D)).astype(np.float16)
+    return q, k.astype(np.float16), v
+
+
+def _fill(kv, ref, k, v, ctx):
+    for p in range(0, ctx, 64):
+        n = min(64, ctx - p)
+        kv.append_host(0, k[p:p + n], v[p:p + n], p)
+    if ctx:
+        ref.append(k[:ctx], v[:ctx], 0)
+
+
+@pytest.mark.parametrize("paged", [False, True])
+def test_append_bit_exact_and_image_round_trip(native, oracle, paged):
+    ctx = 300
+    q, k, v = _inputs(1, ctx, 4)
+    k[7] = 0; v[7] = 0                                    # zero rows: scale 1, every field 8
+    k[9, :, 1:] = 0                                       # one non-zero element per row
+    ref = oracle.Cache(512, NH, KVH, D)
+    with native.KvCache(n_layers=2, head_dim=D, max_ctx=512, paged=paged) as kv:
+        if paged:
+            kv.set_page_table(np.array([1, 0], np.int32))
+        _fill(kv, ref, k, v, ctx)
+        kw, ks, vw, vs = kv.export_rows(0, 0, ctx)
+        assert np.array_equal(kw, ref.kc[:, :ctx]) and np.array_equal(vw, ref.vc[:, :ctx])
+        assert np.array_equal(ks.view(np.uint32), ref.ks[:, :ctx].view(np.uint32))
+        assert np.array_equal(vs.view(np.uint32), ref.vs[:, :ctx].view(np.uint32))
+        assert np.all(kw[:, 7] == 0x88888888) and np.all(ks[:, 7] == 1.0)
+        kv.import_rows(1, 100, kw[:, :50], ks[:, :50], vw[:, :50], vs[:, :50])
+        back = kv.export_rows(1, 100, 50)
+        for a, b in zip(back, (kw[:, :50], ks[:, :50], vw[:, :50], vs[:, :50])):
+            assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("ctx,M", [(0, 1), (0, 5), (31, 1), (32, 2), (257, 3), (1000, 1), (1000, 16), (4096, 1), (2500, 64)])
+def test_attention_matches_oracle(native, oracle, ctx, M):
+    q, k, v = _inputs(10 + ctx + M, ctx, M)
+    max_ctx = ((ctx + M + 255) // 256) * 256
+    ref = oracle.Cache(max_ctx, NH, KVH, D)
+    with native.KvCache(head_dim=D, max_ctx=max_ctx) as kv:
+        _fill(kv, ref, k, v, ctx)
+        out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx)
+        got = kv.export_rows(0, ctx, M)
+    ref.append(k[ctx:], v[ctx:], ctx)
+    assert np.array_equal(got[0], ref.kc[:, ctx:ctx + M]) and np.array_equal(got[3].view(np.uint32), ref.vs[:, ctx:ctx + M].view(np.uint32))
+    assert_attn_close(out, ref.attend_f32(q, ctx, threads=8), f"ctx={ctx} M={M}")
+
+
+def test_depth_table_splits_and_pages(native, oracle):
+    ctx, M = 700, 6
+    q, k, v = _inputs(77, ctx, M)
+    depth = np.array([0, 1, 1, 2, 2, 3], np.uint8)
+    ref = oracle.Cache(1024, NH, KVH, D)
+    outs = []
+    for paged in (False, True):
+        with native.KvCache(head_dim=D, max_ctx=1024, paged=paged) as kv:
+            if paged:
+                kv.set_page_table(np.array([2, 0, 3, 1], np.int32))
+            _fill(kv, ref if not paged else oracle.Cache(1024, NH, KVH, D), k, v, ctx)
+            outs.append(kv.layer_call(0, q, k[ctx:], v[ctx:], ctx, depth=depth))
+            if not paged:
+                kv.set_opt(1, 3)
+                few = kv.layer_call(0, q, None, None, ctx, depth=depth)
+                kv.set_opt(1, 97)
+                many = kv.layer_call(0, q, None, None, ctx, depth=depth)
+    ref.append(k[ctx:], v[ctx:], ctx)
+    expect = ref.attend_f32(q, ctx, depth=depth)
+    assert_attn_close(outs[0], expect, "depth table")
+    assert np.array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))      # paged == contiguous, bit for bit
+    assert_attn_close(few, expect, "3 splits"); assert_attn_close(many, expect, "97 splits")
+
+
+def test_entry_points_of_the_other_format_refuse(native):
+    with native.KvCache(head_dim=D, max_ctx=256) as kv:
+        with pytest.raises(native.YkaError, match="128"):
+            kv.dequant_rows(0, 0, 1)
+        with pytest.raises(native.YkaError, match="128"):
+            kv.ms_call(np.zeros((1, NH, 128), np.float16), None, None, [0], [0])
+    with native.KvCache(max_ctx=256) as kv:
+        with pytest.raises(native.YkaError, match="256"):
+            native._chk(native.lib().yka_kv_export_rows256(kv._h, 0, 0, 1, None, None, None, None))

@@ -31,6 +31,8 @@ struct yka_kv {
   int* d_pos = nullptr;            // position used by the host-pointer hooks
   hipStream_t stream = nullptr;    // stream of the host-pointer hooks
   int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0, opt_unrot = 0;
+  bool r256() const { return cfg.head_dim == 256; }   // the reference's own rows (attend256.hip); otherwise the 128-channel format
+  int D() const { return cfg.head_dim; }
   KvView view(int layer) const {
     return KvView{pool + (size_t)layer * layer_bytes, tables ? tables + (size_t)layer * n_pages : nullptr, cfg.n_kv_heads, cfg.max_ctx};
   }
@@ -82,7 +84,11 @@ void check_rows(const yka_kv* kv, int M) {
 }
 
 void do_append(yka_kv* kv, int layer, const uint16_t* k16, const uint16_t* v16, int M, const int* d_pos, hipStream_t st) {
-  launch_append(AppendArgs{kv->view(layer), k16, v16, d_pos, M}, st);
+  if (kv->r256()) launch_append256(AppendArgs{kv->view(layer), k16, v16, d_pos, M}, st);
+  else launch_append(AppendArgs{kv->view(layer), k16, v16, d_pos, M}, st);
+}
+void need_128(const yka_kv* kv) {
+  if (kv->r256()) throw std::runtime_error("this entry point exists for head_dim 128 only");
 }
 
 // mode 0: attention + combine; 2: attention kernel alone.  k16/v16 != nullptr asks for quantize-on-append as well:
@@ -90,6 +96,19 @@ void do_append(yka_kv* kv, int layer, const uint16_t* k16, const uint16_t* v16, 
 void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_pos, const uint8_t* depth, uint16_t* out16,
                hipStream_t st, int mode = 0, const uint16_t* k16 = nullptr, const uint16_t* v16 = nullptr) {
   const int NH = kv->cfg.n_heads;
+  if (kv->r256()) {
+    // 256-channel rows: append first, then row tiles of 2 tokens x 6 heads for every width; two workgroups per CU
+    if (k16) do_append(kv, layer, k16, v16, M, d_pos, st);
+    for (int s0 = 0; s0 < M; s0 += kMaxSlice) {
+      const int Ms = std::min(kMaxSlice, M - s0), tiles = (Ms + 1) / 2;
+      int S = kv->opt_splits_narrow > 0 ? kv->opt_splits_narrow : 512 / (kv->cfg.n_kv_heads * tiles);
+      S = std::min(std::max(2, std::min(kMaxSplits, S)), (int)(kWsPairs / (size_t)Ms));
+      AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * 256, d_pos, depth, Ms, s0, NH, S, 0, kv->pm, kv->pl, kv->pacc16, nullptr, nullptr};
+      launch_attend256(A, st);
+      if (mode != 2) launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, 0}, st);
+    }
+    return;
+  }
   const bool fuse_append = k16 && M <= 2;
   if (k16 && !fuse_append) do_append(kv, layer, k16, v16, M, d_pos, st);
   for (int s0 = 0; s0 < M; s0 += kMaxSlice) {   // 64-row slices, as attn_block cuts wide passes (engine35.cpp:935-947)
@@ -146,7 +165,7 @@ yka_kv* yka_kv_open(const yka_kv_config* cfg) {
   yka_kv* kv = nullptr;
   try {
     if (!cfg) throw std::runtime_error("null config");
-    if (cfg->head_dim != kD) throw std::runtime_error("head_dim must be 128");
+    if (cfg->head_dim != kD && cfg->head_dim != 256) throw std::runtime_error("head_dim must be 128 (int4 in 32-channel groups) or 256 (the reference's own rows)");
     if (cfg->n_kv_heads < 1 || cfg->n_heads != cfg->n_kv_heads * kG) throw std::runtime_error("n_heads must be 6 * n_kv_heads");
     if (cfg->n_layers < 1) throw std::runtime_error("n_layers must be >= 1");
     if (cfg->max_ctx < kPageTok || cfg->max_ctx % kPageTok) throw std::runtime_error("max_ctx must be a positive multiple of 256");
@@ -158,7 +177,7 @@ yka_kv* yka_kv_open(const yka_kv_config* cfg) {
     kv = new yka_kv();
     kv->cfg = *cfg;
     kv->n_pages = cfg->max_ctx / kPageTok;
-    kv->layer_bytes = (size_t)kv->n_pages * kv_page_bytes(cfg->n_kv_heads);
+    kv->layer_bytes = cfg->head_dim == 256 ? (size_t)kv->n_pages * cfg->n_kv_heads * kPage256Bytes : (size_t)kv->n_pages * kv_page_bytes(cfg->n_kv_heads);
     HIPCHK(hipMalloc((void**)&kv->pool, kv->layer_bytes * cfg->n_layers));
     HIPCHK(hipMemset(kv->pool, 0, kv->layer_bytes * cfg->n_layers));   // zero scales: unwritten rows decode to finite values
     if (cfg->paged) {
@@ -171,7 +190,7 @@ yka_kv* yka_kv_open(const yka_kv_config* cfg) {
     const size_t np = kv->ws_rows * cfg->n_heads;
     HIPCHK(hipMalloc((void**)&kv->pm, np * 4));
     HIPCHK(hipMalloc((void**)&kv->pl, np * 4));
-    HIPCHK(hipMalloc((void**)&kv->pacc16, np * kD * 2));
+    HIPCHK(hipMalloc((void**)&kv->pacc16, np * cfg->head_dim * 2));
     HIPCHK(hipMalloc((void**)&kv->d_pos, 4));
     HIPCHK(hipMemset(kv->d_pos, 0, 4));
     HIPCHK(hipStreamCreateWithFlags(&kv->stream, hipStreamNonBlocking));
@@ -255,7 +274,7 @@ int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16
 int yka_append_attend_ms(yka_kv* kv, const uint16_t* d_q16, const uint16_t* d_k16, const uint16_t* d_v16, int M,
                          const int* d_row_pos, const int* d_row_slot, uint16_t* d_out16, void* hip_stream) {
   YKA_TRY
-  on_device(kv); check_rows(kv, M);
+  on_device(kv); need_128(kv); check_rows(kv, M);
   if (!d_q16 || !d_row_pos || !d_row_slot || !d_out16) throw std::runtime_error("null pointer");
   if ((d_k16 == nullptr) != (d_v16 == nullptr)) throw std::runtime_error("new K and V rows come together or not at all");
   do_attend_ms(kv, d_q16, d_k16, d_v16, M, d_row_pos, d_row_slot, d_out16, (hipStream_t)hip_stream);
@@ -266,7 +285,7 @@ int yka_append_attend_ms(yka_kv* kv, const uint16_t* d_q16, const uint16_t* d_k1
 int yka_ms_call_host(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, const int32_t* row_pos,
                      const int32_t* row_slot, uint16_t* out16) {
   YKA_TRY
-  on_device(kv); check_rows(kv, M);
+  on_device(kv); need_128(kv); check_rows(kv, M);
   if (!q16 || !row_pos || !row_slot || !out16) throw std::runtime_error("null pointer");
   if ((k16 == nullptr) != (v16 == nullptr)) throw std::runtime_error("new K and V rows come together or not at all");
   const size_t nq = (size_t)M * kv->cfg.n_heads * kD, nk = (size_t)M * kv->cfg.n_kv_heads * kD;
@@ -309,7 +328,7 @@ static void check_post(const yka_kv* kv, const yka_post_params* P) {
 int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float* d_xk, const float* d_xv, int M, const int* d_pos,
                   const yka_post_params* P, uint16_t* d_q16, void* hip_stream) {
   YKA_TRY
-  on_device(kv); check_layer(kv, layer); check_rows(kv, M); check_post(kv, P);
+  on_device(kv); need_128(kv); check_layer(kv, layer); check_rows(kv, M); check_post(kv, P);
   if (!d_xq || !d_xk || !d_xv || !d_pos || !d_q16) throw std::runtime_error("null pointer");
   launch_attn_post(PostArgs{kv->view(layer), d_xq, d_xk, d_xv, M, kv->cfg.n_heads, d_pos, P->d_qn_w16, P->d_kn_w16, P->eps,
                             P->d_rope, P->rope_dims, P->rope_rows, P->rotate != 0, d_q16}, (hipStream_t)hip_stream);
@@ -321,7 +340,7 @@ int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, 
                        const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope, int rope_dims,
                        int rope_rows, int rotate, uint16_t* q16) {
   YKA_TRY
-  on_device(kv); check_layer(kv, layer); check_rows(kv, M);
+  on_device(kv); need_128(kv); check_layer(kv, layer); check_rows(kv, M);
   if (!xq || !xk || !xv || !qn_w16 || !kn_w16 || !q16) throw std::runtime_error("null pointer");
   if (pos < 0 || (long long)pos + M > kv->cfg.max_ctx) throw std::runtime_error("rows outside the container");
   if (rope_dims < 0 || rope_dims > kD || (rope_dims & 1)) throw std::runtime_error("rope_dims must be even and in [0, 128]");
@@ -371,7 +390,7 @@ static void check_range(const yka_kv* kv, int pos0, int n) {
 
 int yka_kv_export_rows(yka_kv* kv, int layer, int pos0, int n, uint8_t* kc, uint16_t* ks, uint8_t* vc, uint16_t* vs) {
   YKA_TRY
-  on_device(kv); check_layer(kv, layer); check_range(kv, pos0, n);
+  on_device(kv); need_128(kv); check_layer(kv, layer); check_range(kv, pos0, n);
   if (!kc || !ks || !vc || !vs) throw std::runtime_error("null pointer");
   const size_t rows = (size_t)kv->cfg.n_kv_heads * n;
   DevBuf dkc(rows * 64), dvc(rows * 64), dks(rows * kNG * 2), dvs(rows * kNG * 2);
@@ -388,7 +407,7 @@ int yka_kv_export_rows(yka_kv* kv, int layer, int pos0, int n, uint8_t* kc, uint
 
 int yka_kv_import_rows(yka_kv* kv, int layer, int pos0, int n, const uint8_t* kc, const uint16_t* ks, const uint8_t* vc, const uint16_t* vs) {
   YKA_TRY
-  on_device(kv); check_layer(kv, layer); check_range(kv, pos0, n);
+  on_device(kv); need_128(kv); check_layer(kv, layer); check_range(kv, pos0, n);
   if (!kc || !ks || !vc || !vs) throw std::runtime_error("null pointer");
   const size_t rows = (size_t)kv->cfg.n_kv_heads * n;
   DevBuf dkc(rows * 64), dvc(rows * 64), dks(rows * kNG * 2), dvs(rows * kNG * 2);
@@ -403,9 +422,41 @@ int yka_kv_import_rows(yka_kv* kv, int layer, int pos0, int n, const uint8_t* kc
   YKA_CATCH_INT
 }
 
-int yka_kv_dequant_rows(yka_kv* kv, int layer, int pos0, int n, float* k, float* v) {
+int yka_kv_export_rows256(yka_kv* kv, int layer, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs) {
   YKA_TRY
   on_device(kv); check_layer(kv, layer); check_range(kv, pos0, n);
+  if (!kv->r256()) throw std::runtime_error("this entry point exists for head_dim 256 only");
+  if (!kw || !ks || !vw || !vs) throw std::runtime_error("null pointer");
+  const size_t rows = (size_t)kv->cfg.n_kv_heads * n;
+  DevBuf dkw(rows * 128), dvw(rows * 128), dks(rows * 4), dvs(rows * 4);
+  HIPCHK(hipDeviceSynchronize());
+  launch_export_rows256(kv->view(layer), pos0, n, dkw.as<uint32_t>(), dks.as<float>(), dvw.as<uint32_t>(), dvs.as<float>(), nullptr);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipDeviceSynchronize());
+  HIPCHK(hipMemcpy(kw, dkw.p, rows * 128, hipMemcpyDeviceToHost)); HIPCHK(hipMemcpy(vw, dvw.p, rows * 128, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(ks, dks.p, rows * 4, hipMemcpyDeviceToHost)); HIPCHK(hipMemcpy(vs, dvs.p, rows * 4, hipMemcpyDeviceToHost));
+  YKA_CATCH_INT
+}
+
+int yka_kv_import_rows256(yka_kv* kv, int layer, int pos0, int n, const uint32_t* kw, const float* ks, const uint32_t* vw, const float* vs) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); check_range(kv, pos0, n);
+  if (!kv->r256()) throw std::runtime_error("this entry point exists for head_dim 256 only");
+  if (!kw || !ks || !vw || !vs) throw std::runtime_error("null pointer");
+  const size_t rows = (size_t)kv->cfg.n_kv_heads * n;
+  DevBuf dkw(rows * 128), dvw(rows * 128), dks(rows * 4), dvs(rows * 4);
+  HIPCHK(hipMemcpy(dkw.p, kw, rows * 128, hipMemcpyHostToDevice)); HIPCHK(hipMemcpy(dvw.p, vw, rows * 128, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dks.p, ks, rows * 4, hipMemcpyHostToDevice)); HIPCHK(hipMemcpy(dvs.p, vs, rows * 4, hipMemcpyHostToDevice));
+  HIPCHK(hipDeviceSynchronize());
+  launch_import_rows256(kv->view(layer), pos0, n, dkw.as<uint32_t>(), dks.as<float>(), dvw.as<uint32_t>(), dvs.as<float>(), nullptr);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipDeviceSynchronize());
+  YKA_CATCH_INT
+}
+
+int yka_kv_dequant_rows(yka_kv* kv, int layer, int pos0, int n, float* k, float* v) {
+  YKA_TRY
+  on_device(kv); need_128(kv); check_layer(kv, layer); check_range(kv, pos0, n);
   if (!k || !v) throw std::runtime_error("null pointer");
   const size_t ne = (size_t)kv->cfg.n_kv_heads * n * kD;
   DevBuf dk(ne * 4), dv(ne * 4);
@@ -437,7 +488,7 @@ int yka_layer_call_host(yka_kv* kv, int layer, const uint16_t* q16, const uint16
   on_device(kv); check_layer(kv, layer); check_rows(kv, M);
   if (!q16 || !out16 || ((k16 == nullptr) != (v16 == nullptr))) throw std::runtime_error("bad pointer arguments");
   if (pos < 0 || (long long)pos + M > kv->cfg.max_ctx) throw std::runtime_error("pos + M exceeds max_ctx");
-  const size_t nq = (size_t)M * kv->cfg.n_heads * kD, nk = (size_t)M * kv->cfg.n_kv_heads * kD;
+  const size_t nq = (size_t)M * kv->cfg.n_heads * kv->D(), nk = (size_t)M * kv->cfg.n_kv_heads * kv->D();
   DevBuf dq(nq * 2), dk(nk * 2), dv(nk * 2), dout(nq * 2), dd((size_t)M);
   hipStream_t st = kv->stream;
   HIPCHK(hipMemcpy(dq.p, q16, nq * 2, hipMemcpyHostToDevice));
@@ -458,7 +509,7 @@ int yka_append_host(yka_kv* kv, int layer, const uint16_t* k16, const uint16_t* 
   on_device(kv); check_layer(kv, layer);
   if (!k16 || !v16 || M < 1) throw std::runtime_error("bad argument");
   if (pos < 0 || (long long)pos + M > kv->cfg.max_ctx) throw std::runtime_error("pos + M exceeds max_ctx");
-  const size_t nk = (size_t)M * kv->cfg.n_kv_heads * kD;
+  const size_t nk = (size_t)M * kv->cfg.n_kv_heads * kv->D();
   DevBuf dk(nk * 2), dv(nk * 2);
   HIPCHK(hipMemcpy(dk.p, k16, nk * 2, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dv.p, v16, nk * 2, hipMemcpyHostToDevice));
@@ -525,7 +576,7 @@ int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const u
     if (!q16 || !ms || reps < 1 || mode < 0 || mode > 2) throw std::runtime_error("bad argument");
     if (mode == 0 && (!k16 || !v16)) throw std::runtime_error("mode 0 needs k16 and v16");
     if (pos < 0 || (long long)pos + M > kv->cfg.max_ctx) throw std::runtime_error("pos + M exceeds max_ctx");
-    const size_t nq = (size_t)M * kv->cfg.n_heads * kD, nk = (size_t)M * kv->cfg.n_kv_heads * kD;
+    const size_t nq = (size_t)M * kv->cfg.n_heads * kv->D(), nk = (size_t)M * kv->cfg.n_kv_heads * kv->D();
     DevBuf dq(nq * 2), dk(nk * 2), dv(nk * 2), dout(nq * 2);
     hipStream_t st = kv->stream;
     HIPCHK(hipMemcpy(dq.p, q16, nq * 2, hipMemcpyHostToDevice));

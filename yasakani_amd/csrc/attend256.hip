@@ -1,0 +1,296 @@
+// The reference's own KV rows on gfx950: head_dim 256, flat int4 with ONE fp32 scale per row, 4-bit fields MSB first in
+// 32-bit words (src/kvq_fast.cuh:194-198,226-233; decode src/kvq_attn.cuh:33-37,53-54).  Quantize-on-append, the
+// canonical image, split-KV attention for row tiles of 2 tokens x 6 heads, and the combiner.
+//
+// Page of one (page, kv head): 256 tokens, 67584 bytes
+//   +0      K words  [256][32] uint32      +65536  K scales [256] fp32
+//   +32768  V words  [256][32] uint32      +66560  V scales [256] fp32
+// Attention follows the 128-channel narrow kernel (same MFMA 16x16x32 layouts: S^T = K Q^T leaves one query row per lane
+// column, which is the B-operand layout of O^T += V^T P^T), with what one scale per row allows:
+//   * the score of a key is (sum over 256 channels of q * code) * scale: 8 chained MFMAs and ONE multiply;
+//   * V codes stay exact integers in the MFMA; the V scale of a key is folded into its probability (p * scale, rounded
+//     to fp16 once), the softmax denominator uses the unscaled p.
+// Nibble -> fp16: ((w >> s) & 0x000f000f) | 0x64006400 is (1024 + n) in both halves; minus 1032 gives n - 8.  Shift s
+// selects elements 7 - s/4 (low half) and 3 - s/4 (high half) of the word, so a word yields its 8 codes in the order
+// [7,3,6,2,5,1,4,0]; the query fragments are loaded in the same order.
+#include "yka_internal.h"
+#include <hip/hip_fp16.h>
+
+namespace yka {
+namespace {
+
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+
+constexpr int kD2 = 256;
+constexpr int kP2Kw = 0, kP2Vw = 32768, kP2Ks = 65536, kP2Vs = 66560;
+constexpr uint32_t kMagic = 0x64006400u;
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ h2 as_h2(uint32_t u) { return __builtin_bit_cast(h2, u); }
+__device__ __forceinline__ uint32_t nib(uint32_t w, uint32_t magic) { return (w & 0x000f000fu) | (magic & ~0x000f000fu); }
+
+// start of the (page, kv head) block of token t; t uniform over the wave (table entry through the scalar path)
+__device__ __forceinline__ uint8_t* page256(const KvView& kv, int kvh, int t) {
+  const int lp = t / kPageTok;
+  int pp = lp;
+  if (kv.table) asm volatile("s_load_dword %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=s"(pp) : "s"(kv.table), "s"(lp * 4) : "memory");
+  return kv.base + (size_t)(pp * kv.n_kv + kvh) * kPage256Bytes;
+}
+
+// ---- quantize-on-append: grid (M, n_kv * 2), block 256 = one row, thread = channel ----
+__global__ void __launch_bounds__(256) append256_kernel(AppendArgs A) {
+  __shared__ float red[4];
+  __shared__ uint8_t fld[256];
+  const int tok = blockIdx.x, kvh = blockIdx.y >> 1, isv = blockIdx.y & 1, d = threadIdx.x;
+  const int pos = *A.d_pos + tok;
+  if (pos < 0 || pos >= A.kv.max_ctx) return;
+  const uint16_t* src = (isv ? A.v16 : A.k16) + ((size_t)tok * A.kv.n_kv + kvh) * kD2;
+  const float x = __half2float(__ushort_as_half(src[d]));
+  float am = fabsf(x);
+#pragma unroll
+  for (int o = 32; o; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, 64));
+  if ((d & 63) == 0) red[d >> 6] = am;
+  __syncthreads();
+  am = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  float s7 = __fdiv_rn(am, 7.f);
+  if (s7 == 0.f) s7 = 1.f;
+  float q = rintf(__fdiv_rn(x, s7));
+  q = fminf(fmaxf(q, -7.f), 7.f);
+  fld[d] = (uint8_t)((int)q + 8);
+  __syncthreads();
+  uint8_t* pg = page256(A.kv, kvh, pos);
+  const int tp = pos % kPageTok;
+  if (d < 32) {                                  // word d = fields 8d .. 8d+7, the first in the top nibble
+    uint32_t w = 0u;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) w |= (uint32_t)fld[8 * d + k] << (28 - 4 * k);
+    reinterpret_cast<uint32_t*>(pg + (isv ? kP2Vw : kP2Kw))[tp * 32 + d] = w;
+  }
+  if (d == 0) reinterpret_cast<float*>(pg + (isv ? kP2Vs : kP2Ks))[tp] = s7;
+}
+
+// ---- canonical image <-> pages: grid (n, n_kv), block 64: lanes 0..31 move K words, 32..63 V words ----
+template <bool IMPORT>
+__global__ void __launch_bounds__(64) xfer256_kernel(KvView kv, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs) {
+  const int t = blockIdx.x, kvh = blockIdx.y, j = threadIdx.x & 31, isv = threadIdx.x >> 5;
+  uint8_t* pg = page256(kv, kvh, pos0 + t);
+  const int tp = (pos0 + t) % kPageTok;
+  uint32_t* pw = reinterpret_cast<uint32_t*>(pg + (isv ? kP2Vw : kP2Kw)) + tp * 32 + j;
+  float* ps = reinterpret_cast<float*>(pg + (isv ? kP2Vs : kP2Ks)) + tp;
+  const size_t row = (size_t)kvh * n + t;
+  uint32_t* cw = (isv ? vw : kw) + row * 32 + j;
+  float* cs = (isv ? vs : ks) + row;
+  if (IMPORT) { *pw = *cw; if (j == 0) *ps = *cs; }
+  else { *cw = *pw; if (j == 0) *cs = *ps; }
+}
+
+struct Raw256 {        // what one lane holds of a 32-key tile
+  uint4 kw[2][2];      // K words of key 16kt + (lane & 15): words 8g .. 8g+7 (g = lane >> 4) = channels 64g .. 64g+63
+  f4 ksc[2], vsc[2];   // scales of the 4 keys whose scores this lane receives: keys 16kt + 4g + r
+  uint32_t vw[2][8];   // V word (lane & 15) + 16 hh of token tau(g, e)
+};
+struct Offs256 { uint32_t kw, sc, vw; };
+
+__device__ __forceinline__ void load_tile256(const uint8_t* pg, int tp, const Offs256& L, Raw256& R) {
+  const uint8_t* rows = pg + (uint32_t)tp * 128u;          // code rows of the tile (K and V planes)
+  const uint8_t* sc = pg + (uint32_t)tp * 4u;              // scale entries of the tile
+#pragma unroll
+  for (int kt = 0; kt < 2; ++kt) {
+    R.kw[kt][0] = *reinterpret_cast<const uint4*>(rows + kP2Kw + L.kw + 2048 * kt);
+    R.kw[kt][1] = *reinterpret_cast<const uint4*>(rows + kP2Kw + L.kw + 2048 * kt + 16);
+    R.ksc[kt] = *reinterpret_cast<const f4*>(sc + kP2Ks + L.sc + 64 * kt);
+    R.vsc[kt] = *reinterpret_cast<const f4*>(sc + kP2Vs + L.sc + 64 * kt);
+  }
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+    for (int e = 0; e < 8; ++e)                             // token tau(g, e) = 16 (e >> 2) + 4 g + (e & 3)
+      R.vw[hh][e] = *reinterpret_cast<const uint32_t*>(rows + kP2Vw + L.vw + (16 * (e >> 2) + (e & 3)) * 128 + 64 * hh);
+}
+
+}  // namespace
+
+// grid (S, n_kv, ceil(M/2)), block 256 (4 waves, 2 waves per SIMD).  Workgroup = (split, kv head, 2 tokens x 6 heads).
+__global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
+  __shared__ float s_m[4][16], s_l[4][16];
+  __shared__ float s_acc[4][16][kD2 + 4];
+  const int split = blockIdx.x, kvh = blockIdx.y, rt = blockIdx.z;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
+  const int pos = *A.d_pos;
+  const int tl = 2 * rt + i / kG;
+  const bool vrow = i < 2 * kG && tl < A.M;
+  const int head = kvh * kG + i % kG;
+  int len = 0;
+  if (vrow) { const int tg = A.tok0 + tl; len = min(pos + (A.depth ? (int)A.depth[tg] : tg) + 1, A.kv.max_ctx); }
+  int maxlen = len, minlen = vrow ? len : 0x7fffffff;
+#pragma unroll
+  for (int o = 1; o < 16; o <<= 1) { maxlen = max(maxlen, __shfl_xor(maxlen, o, 64)); minlen = min(minlen, __shfl_xor(minlen, o, 64)); }
+  maxlen = __builtin_amdgcn_readfirstlane(maxlen); minlen = __builtin_amdgcn_readfirstlane(minlen);
+  const int ntiles = (maxlen + 31) >> 5, tps = (ntiles + A.S - 1) / A.S;
+  const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
+
+  // Q fragments: k-step t of 8, lane (row i, group g), element e <-> channel 64g + 8t + [7,3,6,2,5,1,4,0][e]
+  h8 qf[8];
+  {
+    const uint16_t* qrow = A.q16 + ((size_t)tl * A.n_heads + head) * kD2 + 64 * g;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      uint4 u = vrow ? *reinterpret_cast<const uint4*>(qrow + 8 * t) : make_uint4(0, 0, 0, 0);
+      const h8 c = __builtin_bit_cast(h8, u);
+      qf[t] = h8{c[7], c[3], c[6], c[2], c[5], c[1], c[4], c[0]};
+    }
+  }
+  const float sc_log2 = kLog2e * 0.0625f;          // log2(e) / sqrt(256)
+  const h2 c1032 = {(_Float16)1032.f, (_Float16)1032.f};
+  uint32_t magic = kMagic;
+  asm volatile("" : "+v"(magic));
+  const Offs256 offs{(uint32_t)i * 128u + 32u * g, 16u * g, 512u * g + 4u * i};
+
+  float m_run = -1e30f, l_run = 0.f;
+  f4 o[16];
+#pragma unroll
+  for (int b = 0; b < 16; ++b) o[b] = f4{0.f, 0.f, 0.f, 0.f};
+
+  Raw256 cur;
+  for (int T = tile0 + wave; T < tile1; T += 4) {
+    load_tile256(page256(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, cur);
+    const int t0 = T << 5;
+    const bool need_mask = t0 + 32 > minlen;
+    // ---- scores: per 16-key tile 8 chained MFMAs (one per word of the lane), then one multiply by the key's scale ----
+    float s[8];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      const uint32_t w[8] = {cur.kw[kt][0].x, cur.kw[kt][0].y, cur.kw[kt][0].z, cur.kw[kt][0].w,
+                             cur.kw[kt][1].x, cur.kw[kt][1].y, cur.kw[kt][1].z, cur.kw[kt][1].w};
+      f4 part = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int t = 0; t < 8; ++t) {
+        const h2 p0 = as_h2(nib(w[t], magic)) - c1032, p1 = as_h2(nib(w[t] >> 4, magic)) - c1032;
+        const h2 p2 = as_h2(nib(w[t] >> 8, magic)) - c1032, p3 = as_h2(nib(w[t] >> 12, magic)) - c1032;
+        const h8 kf = h8{p0[0], p0[1], p1[0], p1[1], p2[0], p2[1], p3[0], p3[1]};
+        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[t], part, 0, 0, 0);
+      }
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s[4 * kt + r] = part[r] * cur.ksc[kt][r];      // key t0 + 16kt + 4g + r against row i
+    }
+    if (need_mask) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { const int key = t0 + 16 * (e >> 2) + 4 * g + (e & 3); s[e] = key < len ? s[e] : -INFINITY; }
+    }
+    // ---- online softmax (one running maximum per row, shared by its 4 lane groups) ----
+    float tmax = s[0];
+#pragma unroll
+    for (int e = 1; e < 8; ++e) tmax = fmaxf(tmax, s[e]);
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax * sc_log2);
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    const bool first = m_run < -1e29f;
+    m_run = m_new;
+    if (__any(alpha != 1.f && !first)) {
+      l_run *= alpha;
+#pragma unroll
+      for (int b = 0; b < 16; ++b) { o[b][0] *= alpha; o[b][1] *= alpha; o[b][2] *= alpha; o[b][3] *= alpha; }
+    }
+    h8 pf;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], sc_log2, -m_new));
+      l_run += p;
+      pf[e] = (_Float16)(p * cur.vsc[e >> 2][e & 3]);       // the V scale of the key rides on its probability
+    }
+    // ---- O^T += V^T P^T: word (lane & 15) + 16 hh of 8 tokens; byte bb of those words holds elements 7-2bb (low
+    //      nibble) and 6-2bb (high nibble): accumulator hh*8 + element covers channels 8 * word + element ----
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+      for (int bb = 0; bb < 4; ++bb) {
+        h2 lo[4], hi[4];
+#pragma unroll
+        for (int pe = 0; pe < 4; ++pe) {
+          const uint32_t x = __builtin_amdgcn_perm(cur.vw[hh][2 * pe + 1], cur.vw[hh][2 * pe], 0x0c040c00u + bb * 0x00010001u);
+          lo[pe] = as_h2(nib(x, magic)) - c1032;
+          hi[pe] = as_h2(nib(x >> 4, magic)) - c1032;
+        }
+        const h8 vlo = h8{lo[0][0], lo[0][1], lo[1][0], lo[1][1], lo[2][0], lo[2][1], lo[3][0], lo[3][1]};
+        const h8 vhi = h8{hi[0][0], hi[0][1], hi[1][0], hi[1][1], hi[2][0], hi[2][1], hi[3][0], hi[3][1]};
+        o[hh * 8 + 7 - 2 * bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vlo, pf, o[hh * 8 + 7 - 2 * bb], 0, 0, 0);
+        o[hh * 8 + 6 - 2 * bb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vhi, pf, o[hh * 8 + 6 - 2 * bb], 0, 0, 0);
+      }
+  }
+  // ---- merge the 4 waves, write one partial per (row, split): o[hh*8 + el][r] = channel 8 (4g + r + 16 hh) + el of row i ----
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+  if (g == 0) { s_m[wave][i] = m_run; s_l[wave][i] = l_run; }
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+    for (int el = 0; el < 8; ++el)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s_acc[wave][i][8 * (4 * g + r + 16 * hh) + el] = o[hh * 8 + el][r];
+  __syncthreads();
+  for (int idx = threadIdx.x; idx < 2 * kG * kD2; idx += 256) {
+    const int j = idx >> 8, d = idx & (kD2 - 1);
+    const int tj = 2 * rt + j / kG;
+    if (tj >= A.M) continue;
+    const float m0 = s_m[0][j], m1 = s_m[1][j], m2 = s_m[2][j], m3 = s_m[3][j];
+    const float M2 = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
+    const float w0 = exp2f(m0 - M2), w1 = exp2f(m1 - M2), w2 = exp2f(m2 - M2), w3 = exp2f(m3 - M2);
+    const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
+    const float L = w0 * s_l[0][j] + w1 * s_l[1][j] + w2 * s_l[2][j] + w3 * s_l[3][j];
+    const float acc = w0 * s_acc[0][j][d] + w1 * s_acc[1][j][d] + w2 * s_acc[2][j][d] + w3 * s_acc[3][j][d];
+    A.pacc16[p * kD2 + d] = __half_as_ushort(__float2half_rn(L > 0.f ? acc / L : 0.f));
+    if (d == 0) { A.pm[p] = M2; A.pl[p] = L; }
+  }
+}
+
+// combiner (src/attention_kv4q.cu:325-332) for 256-channel rows: grid (n_heads, M), block 256 = one channel per thread
+__global__ void __launch_bounds__(256) combine256_kernel(CombineArgs A) {
+  __shared__ float s_w[256];
+  __shared__ float s_red[4];
+  const int head = blockIdx.x, tok = blockIdx.y, tid = threadIdx.x;
+  const size_t p0 = (size_t)tok * A.S * A.n_heads + head;
+  float pmv = -1e30f, plv = 0.f;
+  if (tid < A.S) { pmv = A.pm[p0 + (size_t)tid * A.n_heads]; plv = A.pl[p0 + (size_t)tid * A.n_heads]; }
+  float M2 = pmv;
+#pragma unroll
+  for (int o = 32; o; o >>= 1) M2 = fmaxf(M2, __shfl_xor(M2, o, 64));
+  if ((tid & 63) == 0) s_red[tid >> 6] = M2;
+  __syncthreads();
+  M2 = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+  s_w[tid] = (tid < A.S && pmv > -1e29f) ? exp2f(pmv - M2) * plv : 0.f;
+  __syncthreads();
+  const uint16_t* src = A.pacc16 + p0 * kD2 + tid;
+  const size_t stride = (size_t)A.n_heads * kD2;
+  float acc = 0.f, L = 0.f;
+  for (int s0 = 0; s0 < A.S; s0 += 8) {           // 8 loads in flight
+    uint16_t u[8]; float w[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { const int sp = s0 + k; w[k] = sp < A.S ? s_w[sp] : 0.f; u[k] = sp < A.S ? src[(size_t)sp * stride] : (uint16_t)0; }
+#pragma unroll
+    for (int k = 0; k < 8; ++k) { acc += w[k] * __half2float(__ushort_as_half(u[k])); L += w[k]; }
+  }
+  A.out16[((size_t)tok * A.n_heads + head) * kD2 + tid] = __half_as_ushort(__float2half_rn(L > 0.f ? acc / L : 0.f));
+}
+
+void launch_append256(const AppendArgs& A, hipStream_t st) {
+  hipLaunchKernelGGL(append256_kernel, dim3(A.M, A.kv.n_kv * 2), dim3(256), 0, st, A);
+}
+void launch_attend256(const AttnArgs& A, hipStream_t st) {
+  hipLaunchKernelGGL(attend256_kernel, dim3(A.S, A.kv.n_kv, (A.M + 1) / 2), dim3(256), 0, st, A);
+}
+void launch_combine256(const CombineArgs& A, hipStream_t st) {
+  hipLaunchKernelGGL(combine256_kernel, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
+}
+void launch_export_rows256(const KvView& kv, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs, hipStream_t st) {
+  hipLaunchKernelGGL(xfer256_kernel<false>, dim3(n, kv.n_kv), dim3(64), 0, st, kv, pos0, n, kw, ks, vw, vs);
+}
+void launch_import_rows256(const KvView& kv, int pos0, int n, const uint32_t* kw, const float* ks, const uint32_t* vw, const float* vs, hipStream_t st) {
+  hipLaunchKernelGGL(xfer256_kernel<true>, dim3(n, kv.n_kv), dim3(64), 0, st, kv, pos0, n, const_cast<uint32_t*>(kw), const_cast<float*>(ks),
+                     const_cast<uint32_t*>(vw), const_cast<float*>(vs));
+}
+
+}  // namespace yka

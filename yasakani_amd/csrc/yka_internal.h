@@ -20,6 +20,7 @@ constexpr int kPageTok = 256;    // tokens per page
 //   +34816  V scales [4][256]   fp16, group major (4 consecutive tokens of one group are 8 contiguous bytes)
 constexpr int kPageKc = 0, kPageVc = 16384, kPageKs = 32768, kPageVs = 34816, kPageBytes = 36864;
 __host__ __device__ inline int k_phys_dword(int logical) { return 4 * (logical & 3) + (logical >> 2); }
+constexpr int kPage256Bytes = 67584;   // page of the 256-channel row format (attend256.hip): 256 x (128 + 128) code bytes + 2 x 256 fp32 scales
 constexpr int kMaxSlice = 64;    // rows per attention slice (kVerifyMax of the reference, engine35.hpp:157)
 
 // One layer's container.  The page of token t of kv head h starts at
@@ -78,6 +79,12 @@ void launch_attend_narrow(const AttnArgs&, hipStream_t);   // 16-row tiles: 2 to
 void launch_attend_wide(const AttnArgs&, hipStream_t);     // 3..64 tokens
 void launch_combine(const CombineArgs&, hipStream_t);
 void launch_attn_post(const PostArgs&, hipStream_t);
+// the reference's own rows, head_dim 256 (attend256.hip): same argument structs, 67584-byte pages
+void launch_append256(const AppendArgs&, hipStream_t);
+void launch_attend256(const AttnArgs&, hipStream_t);       // row tiles of 2 tokens x 6 heads for every width
+void launch_combine256(const CombineArgs&, hipStream_t);
+void launch_export_rows256(const KvView&, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs, hipStream_t);
+void launch_import_rows256(const KvView&, int pos0, int n, const uint32_t* kw, const float* ks, const uint32_t* vw, const float* vs, hipStream_t);
 // canonical <-> physical
 void launch_export_rows(const KvView&, int pos0, int n, uint8_t* kc, uint16_t* ks, uint8_t* vc, uint16_t* vs, hipStream_t);
 void launch_import_rows(const KvView&, int pos0, int n, const uint8_t* kc, const uint16_t* ks, const uint8_t* vc, const uint16_t* vs, hipStream_t);

@@ -53,6 +53,8 @@ def _load():
         "yka_codec_probe": (i32, [vp, i32, vp, vp, vp]),
         "yka_kvx256_probe": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_attn_post": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
+        "yka_kv_export_rows256": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
+        "yka_kv_import_rows256": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_append_attend_ms": (i32, [vp, vp, vp, vp, i32, vp, vp, vp, vp]),
         "yka_ms_call_host": (i32, [vp, vp, vp, vp, i32, vp, vp, vp]),
         "yka_attn_post_host": (i32, [vp, i32, vp, vp, vp, i32, i32, vp, vp, C.c_float, vp, i32, i32, i32, vp]),
@@ -75,7 +77,7 @@ def _load():
 
 EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "yka_set_opt", "yka_kv_set_page_table",
            "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kvx256_probe", "yka_attn_post", "yka_append_attend_ms", "yka_ms_call_host",
-           "yka_attn_post_host", "yka_kv_export_rows",
+           "yka_attn_post_host", "yka_kv_export_rows", "yka_kv_export_rows256", "yka_kv_import_rows256",
            "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
            "yka_append_host", "yka_pass_capture", "yka_pass_launch", "yka_pass_destroy", "yka_attn_bench")
 
@@ -219,6 +221,11 @@ class KvCache:
     # -- hooks: host arrays --
     def export_rows(self, layer, pos0, n):
         kvh = self.cfg.n_kv_heads
+        if self.cfg.head_dim == 256:        # words [kvh, n, 32] u32 and row scales [kvh, n] f32
+            kw = np.empty((kvh, n, 32), np.uint32); vw = np.empty_like(kw)
+            ks = np.empty((kvh, n), np.float32); vs = np.empty_like(ks)
+            _chk(lib().yka_kv_export_rows256(self._h, layer, pos0, n, _ptr(kw), _ptr(ks), _ptr(vw), _ptr(vs)))
+            return kw, ks, vw, vs
         kc = np.empty((kvh, n, D // 2), np.uint8); vc = np.empty_like(kc)
         ks = np.empty((kvh, n, NG), np.uint16); vs = np.empty_like(ks)
         _chk(lib().yka_kv_export_rows(self._h, layer, pos0, n, _ptr(kc), _ptr(ks), _ptr(vc), _ptr(vs)))
@@ -227,6 +234,13 @@ class KvCache:
     def import_rows(self, layer, pos0, kc, ks, vc, vs):
         kvh = self.cfg.n_kv_heads
         n = kc.shape[1]
+        if self.cfg.head_dim == 256:
+            kw = np.ascontiguousarray(kc, np.uint32); vw = np.ascontiguousarray(vc, np.uint32)
+            fs = np.ascontiguousarray(ks, np.float32); gs = np.ascontiguousarray(vs, np.float32)
+            if kw.shape != (kvh, n, 32) or vw.shape != kw.shape or fs.shape != (kvh, n) or gs.shape != fs.shape:
+                raise ValueError("expected words [kvh, n, 32] and scales [kvh, n]")
+            _chk(lib().yka_kv_import_rows256(self._h, layer, pos0, n, _ptr(kw), _ptr(fs), _ptr(vw), _ptr(gs)))
+            return
         kc = np.ascontiguousarray(kc, np.uint8); vc = np.ascontiguousarray(vc, np.uint8)
         ks = _u16(ks, (kvh, n, NG)); vs = _u16(vs, (kvh, n, NG))
         if kc.shape != (kvh, n, D // 2) or vc.shape != kc.shape:
@@ -245,18 +259,18 @@ class KvCache:
     def layer_call(self, layer, q16, k16, v16, pos, depth=None):
         """One layer call with host arrays: q16 [M,n_heads,128], k16/v16 [M,n_kv_heads,128] fp16 (or None = attend only)."""
         M = q16.shape[0]
-        q = _u16(q16, (M, self.cfg.n_heads, D))
-        k = None if k16 is None else _u16(k16, (M, self.cfg.n_kv_heads, D))
-        v = None if v16 is None else _u16(v16, (M, self.cfg.n_kv_heads, D))
+        q = _u16(q16, (M, self.cfg.n_heads, self.cfg.head_dim))
+        k = None if k16 is None else _u16(k16, (M, self.cfg.n_kv_heads, self.cfg.head_dim))
+        v = None if v16 is None else _u16(v16, (M, self.cfg.n_kv_heads, self.cfg.head_dim))
         dep = None if depth is None else np.ascontiguousarray(depth, np.uint8)
-        out = np.empty((M, self.cfg.n_heads, D), np.uint16)
+        out = np.empty((M, self.cfg.n_heads, self.cfg.head_dim), np.uint16)
         _chk(lib().yka_layer_call_host(self._h, layer, _ptr(q), _ptr(k), _ptr(v), M, pos, _ptr(dep), _ptr(out)))
         return out.view(np.float16)
 
     def append_host(self, layer, k16, v16, pos):
         """Quantize host rows k16/v16 [M,n_kv_heads,128] into rows pos..pos+M-1."""
         M = k16.shape[0]
-        k = _u16(k16, (M, self.cfg.n_kv_heads, D)); v = _u16(v16, (M, self.cfg.n_kv_heads, D))
+        k = _u16(k16, (M, self.cfg.n_kv_heads, self.cfg.head_dim)); v = _u16(v16, (M, self.cfg.n_kv_heads, self.cfg.head_dim))
         _chk(lib().yka_append_host(self._h, layer, _ptr(k), _ptr(v), M, pos))
 
     def attn_post_host(self, layer, xq, xk, xv, pos, qn_w16, kn_w16, eps, rope, rope_dims, rotate=False):
@@ -287,11 +301,11 @@ class KvCache:
     def bench(self, q16, k16, v16, pos, mode=0, use_graph=True, reps=20):
         """Timed sweeps over all layers; returns (ms per sweep [reps], out of the last layer call)."""
         M = q16.shape[0]
-        q = _u16(q16, (M, self.cfg.n_heads, D))
-        k = None if k16 is None else _u16(k16, (M, self.cfg.n_kv_heads, D))
-        v = None if v16 is None else _u16(v16, (M, self.cfg.n_kv_heads, D))
+        q = _u16(q16, (M, self.cfg.n_heads, self.cfg.head_dim))
+        k = None if k16 is None else _u16(k16, (M, self.cfg.n_kv_heads, self.cfg.head_dim))
+        v = None if v16 is None else _u16(v16, (M, self.cfg.n_kv_heads, self.cfg.head_dim))
         ms = np.zeros(reps, np.float32)
-        out = np.empty((M, self.cfg.n_heads, D), np.uint16)
+        out = np.empty((M, self.cfg.n_heads, self.cfg.head_dim), np.uint16)
         _chk(lib().yka_attn_bench(self._h, _ptr(q), _ptr(k), _ptr(v), M, pos, mode, int(bool(use_graph)), reps, _ptr(ms), _ptr(out)))
         return ms, out.view(np.float16)
 
