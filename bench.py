@@ -109,6 +109,34 @@ def small_decode(native, ctx=4096, L=128):
             "hbm_peak_frac": by / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
 
 
+def r256_figures(native, ctx=32768, L=16):
+    """The reference's own rows (head_dim 256, one fp32 scale per row): 1,056 B per token per layer, 16 containers of
+    34.6 MB.  One layer call = append + attention (row tiles of 2 tokens) + combine."""
+    rng = np.random.default_rng(256)
+    D2 = 256
+    k = rng.standard_normal((4096 + 64, KVH, D2)).astype(np.float16)
+    v = rng.standard_normal((4096 + 64, KVH, D2)).astype(np.float16)
+    q = rng.standard_normal((64, NH, D2)).astype(np.float16)
+    kv = native.KvCache(n_layers=L, head_dim=D2, max_ctx=ctx + 256, max_rows=64)
+    for p in range(0, ctx, 64):                       # 4096 distinct rows tiled over the context
+        s0 = p % 4096
+        kv.append_host(0, k[s0:s0 + 64], v[s0:s0 + 64], p)
+    kv.replicate_layer(0)
+    out = {}
+    token_bytes = KVH * 2 * (128 + 4)
+    for rows in (1, 16, 64):
+        ms, _ = kv.bench(q[:rows], k[4096:4096 + rows], v[4096:4096 + rows], ctx, mode=0, use_graph=True, reps=10)
+        us = float(np.median(ms)) * 1e3 / L
+        ms2, _ = kv.bench(q[:rows], None, None, ctx, mode=2, use_graph=True, reps=10)
+        k_us = float(np.median(ms2)) * 1e3 / L
+        by = ctx * token_bytes + rows * (2 * token_bytes + 2 * KVH * D2 * 2 + 2 * NH * D2 * 2)
+        out[f"rows_{rows}"] = {"us_per_layer": us, "kernel_us": k_us, "value_GBs": by / (us * 1e-6) / 1e9,
+                               "kernel_hbm_frac": by / (k_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                               "kernel_tflops": 4.0 * rows * NH * D2 * ctx / (k_us * 1e-6) / 1e12}
+    kv.close()
+    return out
+
+
 def big_configs(native):
     """Secondary figures for the two large configurations: a 2048-row prefill chunk on 131072 cached tokens (cut into
     64-row slices inside the library) and decode / verify-64 on 262144 tokens in shuffled 256-token pages."""
@@ -326,6 +354,7 @@ def main():
         line["calibration_copy_bytes"] = 256 << 20
     if not args.no_extra:
         line["other_configs"] = big_configs(native)
+        line["reference_rows_head_dim_256"] = r256_figures(native)
     print(json.dumps(line))
 
 

@@ -247,10 +247,12 @@ __global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
   }
 }
 
-// combiner (src/attention_kv4q.cu:325-332) for 256-channel rows: grid (n_heads, M), block 256 = one channel per thread
+// combiner (src/attention_kv4q.cu:325-332) for 256-channel rows: grid (n_heads, M), block 256 = 8 split lanes x 32 channel
+// lanes of 8 channels; the split lanes run in parallel (4 loads in flight each) and are summed through LDS.  S <= 256.
 __global__ void __launch_bounds__(256) combine256_kernel(CombineArgs A) {
   __shared__ float s_w[256];
-  __shared__ float s_red[4];
+  __shared__ float s_o[8][kD2 + 4];
+  __shared__ float s_wsum[8];
   const int head = blockIdx.x, tok = blockIdx.y, tid = threadIdx.x;
   const size_t p0 = (size_t)tok * A.S * A.n_heads + head;
   float pmv = -1e30f, plv = 0.f;
@@ -258,22 +260,41 @@ __global__ void __launch_bounds__(256) combine256_kernel(CombineArgs A) {
   float M2 = pmv;
 #pragma unroll
   for (int o = 32; o; o >>= 1) M2 = fmaxf(M2, __shfl_xor(M2, o, 64));
-  if ((tid & 63) == 0) s_red[tid >> 6] = M2;
+  if ((tid & 63) == 0) s_wsum[tid >> 6] = M2;
   __syncthreads();
-  M2 = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+  M2 = fmaxf(fmaxf(s_wsum[0], s_wsum[1]), fmaxf(s_wsum[2], s_wsum[3]));
+  __syncthreads();
   s_w[tid] = (tid < A.S && pmv > -1e29f) ? exp2f(pmv - M2) * plv : 0.f;
   __syncthreads();
-  const uint16_t* src = A.pacc16 + p0 * kD2 + tid;
+  const int sl = tid >> 5, c8 = (tid & 31) * 8;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float wsum = 0.f;
+  const uint16_t* src = A.pacc16 + p0 * kD2 + c8;
   const size_t stride = (size_t)A.n_heads * kD2;
-  float acc = 0.f, L = 0.f;
-  for (int s0 = 0; s0 < A.S; s0 += 8) {           // 8 loads in flight
-    uint16_t u[8]; float w[8];
+  for (int s0 = sl; s0 < A.S; s0 += 32) {
+    uint4 u[4]; float w[4];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) { const int sp = s0 + k; w[k] = sp < A.S ? s_w[sp] : 0.f; u[k] = sp < A.S ? src[(size_t)sp * stride] : (uint16_t)0; }
+    for (int k = 0; k < 4; ++k) {
+      const int sp = s0 + 8 * k;
+      w[k] = sp < A.S ? s_w[sp] : 0.f;
+      u[k] = sp < A.S ? *reinterpret_cast<const uint4*>(src + (size_t)sp * stride) : make_uint4(0, 0, 0, 0);
+    }
 #pragma unroll
-    for (int k = 0; k < 8; ++k) { acc += w[k] * __half2float(__ushort_as_half(u[k])); L += w[k]; }
+    for (int k = 0; k < 4; ++k) {
+      const h8 v = __builtin_bit_cast(h8, u[k]);
+#pragma unroll
+      for (int c = 0; c < 8; ++c) acc[c] += w[k] * (float)v[c];
+      wsum += w[k];
+    }
   }
-  A.out16[((size_t)tok * A.n_heads + head) * kD2 + tid] = __half_as_ushort(__float2half_rn(L > 0.f ? acc / L : 0.f));
+#pragma unroll
+  for (int c = 0; c < 8; ++c) s_o[sl][c8 + c] = acc[c];
+  if ((tid & 31) == 0) s_wsum[sl] = wsum;
+  __syncthreads();
+  float o = 0.f, L = 0.f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) { o += s_o[k][tid]; L += s_wsum[k]; }
+  A.out16[((size_t)tok * A.n_heads + head) * kD2 + tid] = __half_as_ushort(__float2half_rn(L > 0.f ? o / L : 0.f));
 }
 
 void launch_append256(const AppendArgs& A, hipStream_t st) {
