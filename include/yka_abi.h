@@ -57,7 +57,8 @@ YKA_API const char* yka_build_info(void);
  * key 1: split count of the narrow kernel (decode, rows of at most 2 tokens; at most 256); key 2: split count of the wide kernel;
  * key 3: 1 forces the narrow kernel for every width (cross-check of the wide kernel), 0 = automatic;
  * key 4: 1 = attention outputs get the inverse signed Hadamard rotation before they are rounded to fp16 (for caches
- *        filled by yka_attn_post with rotate = 1; the reference un-rotates in its output step, q35_kernels.cu:1421). */
+ *        filled by yka_attn_post or yka_append256_f32 with rotate = 1; the reference un-rotates in its output step,
+ *        q35_kernels.cu:1421). */
 YKA_API int yka_set_opt(yka_kv* kv, int key, int value);
 
 /* Paged mode: logical page p of `layer` (-1 = every layer) lives in physical page h_table[p]; n_pages = max_ctx/256
@@ -97,6 +98,16 @@ YKA_API int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, cons
 YKA_API int yka_append_attend_ms(yka_kv* kv, const uint16_t* d_q16, const uint16_t* d_k16, const uint16_t* d_v16, int M,
                                  const int* d_row_pos, const int* d_row_slot, uint16_t* d_out16, void* hip_stream);
 
+/* head_dim 256: quantize-on-append from fp32 rows, d_k32 / d_v32 [M][n_kv_heads][256].  With rotate != 0 every row first
+ * gets the signed Walsh-Hadamard rotation (kvx_codec.cuh:28-49), then the flat int4 row codec - the arithmetic of
+ * kvx_rotate followed by the flat mode of the row quantizer (q35_kernels.cu:1036,1060; kvq_fast.cuh:194-198), bit for
+ * bit.  Allocates nothing, synchronises nothing. */
+YKA_API int yka_append256_f32(yka_kv* kv, int layer, const float* d_k32, const float* d_v32, int M, const int* d_pos,
+                              int rotate, void* hip_stream);
+/* head_dim 256: rotated query rows, d_x32 [rows][256] fp32 -> d_q16 [rows][256] fp16 (q35_kernels.cu:1060,1062 with fp16
+ * in the place of the reference's bf16).  Attention over a rotated cache then needs option key 4 (outputs un-rotated). */
+YKA_API int yka_rotate_q256(const float* d_x32, int rows, uint16_t* d_q16, void* hip_stream);
+
 /* The step between the QKV projection and the cache, fused with quantize-on-append; replaces launch_q35_attn_post
  * (q35.hpp:97-105, q35_kernels.cu:1013-1065) + launch_tb_requant (q35_kernels.cu:1084-1092) for 128-channel heads:
  * per head, Q and K rows are RMS-normalised (x / sqrt(mean x^2 + eps) * (1 + w)), get the rotary embedding on their
@@ -123,6 +134,10 @@ YKA_API int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float*
 /* Host-pointer form of yka_append_attend_ms (k16 / v16 may be NULL = attend only). */
 YKA_API int yka_ms_call_host(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M,
                              const int32_t* row_pos, const int32_t* row_slot, uint16_t* out16);
+
+/* Host-pointer forms of yka_append256_f32 and yka_rotate_q256. */
+YKA_API int yka_append256_f32_host(yka_kv* kv, int layer, const float* k32, const float* v32, int M, int pos, int rotate);
+YKA_API int yka_rotate_q256_host(const float* x32, int rows, uint16_t* q16);
 
 /* Host-pointer form of yka_attn_post: uploads everything, sets the device position to `pos`, runs, downloads q16. */
 YKA_API int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, const float* xv, int M, int pos,

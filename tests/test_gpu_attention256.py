@@ -95,3 +95,47 @@ def test_entry_points_of_the_other_format_refuse(native):
     with native.KvCache(max_ctx=256) as kv:
         with pytest.raises(native.YkaError, match="256"):
             native._chk(native.lib().yka_kv_export_rows256(kv._h, 0, 0, 1, None, None, None, None))
+
+
+def test_rotated_rows_and_unrotated_outputs(native, oracle):
+    """fp32 rows -> signed Hadamard rotation -> flat int4 rows (the reference's kvx_rotate + row quantizer), rotated Q rows,
+    attention, outputs rotated back."""
+    ctx, M = 500, 5
+    rng = np.random.default_rng(2024)
+    k32 = rng.standard_normal((ctx + M, KVH, D)).astype(np.float32)
+    k32[:, :, [5, 77, 130, 201]] *= 8
+    v32 = rng.standard_normal((ctx + M, KVH, D)).astype(np.float32)
+    q32 = rng.standard_normal((M, NH, D)).astype(np.float32)
+    n = ctx + M
+    ref = oracle.Cache(768, NH, KVH, D)
+    for h in range(KVH):
+        ref.kc[h, :n], ref.ks[h, :n], _ = oracle.flat4_encode256(oracle.kvx_rotate256(k32[:, h]))
+        ref.vc[h, :n], ref.vs[h, :n], _ = oracle.flat4_encode256(oracle.kvx_rotate256(v32[:, h]))
+    qrot = oracle.kvx_rotate256(q32.reshape(-1, D)).astype(np.float16).reshape(M, NH, D)
+    got_q = native.rotate_q256(q32)
+    assert np.array_equal(got_q.view(np.uint16), qrot.view(np.uint16))
+    with native.KvCache(head_dim=D, max_ctx=768) as kv:
+        for p in range(0, n, 64):
+            m = min(64, n - p)
+            kv.append256_f32_host(0, k32[p:p + m], v32[p:p + m], p, rotate=True)
+        kw, ks, vw, vs = kv.export_rows(0, 0, n)
+        assert np.array_equal(kw, ref.kc[:, :n]) and np.array_equal(vw, ref.vc[:, :n])
+        assert np.array_equal(ks.view(np.uint32), ref.ks[:, :n].view(np.uint32)) and np.array_equal(vs.view(np.uint32), ref.vs[:, :n].view(np.uint32))
+        kv.set_opt(4, 1)
+        out = kv.layer_call(0, got_q, None, None, ctx)
+        kv.set_opt(4, 0)
+        raw = kv.layer_call(0, got_q, None, None, ctx)
+    _, o32 = ref.attend_f32(qrot, ctx, want_f32=True)
+    expect = oracle.kvx_rotate256(o32.reshape(-1, D), inverse=True).astype(np.float16).reshape(M, NH, D)
+    assert_attn_close(out, expect, "un-rotated outputs")
+    assert_attn_close(raw, o32, "outputs left in the rotated basis")
+    # the whole pipeline approximates plain attention on the unrotated fp32 data (int4 noise only); a wrong factor or a
+    # missing sign in either rotation would show as an error of order 1
+    worst = 0.0
+    for t in range(M):
+        for h in (0, 7, 23):
+            s = k32[:ctx + t + 1, h // 6].astype(np.float64) @ q32[t, h].astype(np.float64) / 16.0
+            p = np.exp(s - s.max()); p /= p.sum()
+            plain = p @ v32[:ctx + t + 1, h // 6].astype(np.float64)
+            worst = max(worst, np.linalg.norm(out[t, h].astype(np.float64) - plain) / np.linalg.norm(plain))
+    assert worst < 0.35, worst

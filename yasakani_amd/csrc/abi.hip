@@ -105,7 +105,7 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
       S = std::min(std::max(2, std::min(kMaxSplits, S)), (int)(kWsPairs / (size_t)Ms));
       AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * 256, d_pos, depth, Ms, s0, NH, S, 0, kv->pm, kv->pl, kv->pacc16, nullptr, nullptr};
       launch_attend256(A, st);
-      if (mode != 2) launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, 0}, st);
+      if (mode != 2) launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, kv->opt_unrot}, st);
     }
     return;
   }
@@ -419,6 +419,59 @@ int yka_kv_import_rows(yka_kv* kv, int layer, int pos0, int n, const uint8_t* kc
   launch_import_rows(kv->view(layer), pos0, n, dkc.as<uint8_t>(), dks.as<uint16_t>(), dvc.as<uint8_t>(), dvs.as<uint16_t>(), nullptr);
   HIPCHK(hipGetLastError());
   HIPCHK(hipDeviceSynchronize());
+  YKA_CATCH_INT
+}
+
+int yka_append256_f32(yka_kv* kv, int layer, const float* d_k32, const float* d_v32, int M, const int* d_pos, int rotate, void* hip_stream) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); check_rows(kv, M);
+  if (!kv->r256()) throw std::runtime_error("this entry point exists for head_dim 256 only");
+  if (!d_k32 || !d_v32 || !d_pos) throw std::runtime_error("null pointer");
+  AppendArgs A{kv->view(layer), nullptr, nullptr, d_pos, M};
+  A.k32 = d_k32; A.v32 = d_v32; A.rot = rotate != 0;
+  launch_append256(A, (hipStream_t)hip_stream);
+  HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_rotate_q256(const float* d_x32, int rows, uint16_t* d_q16, void* hip_stream) {
+  YKA_TRY
+  if (!d_x32 || !d_q16 || rows < 1) throw std::runtime_error("bad argument");
+  launch_rotate_q256(d_x32, rows, d_q16, (hipStream_t)hip_stream);
+  HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_append256_f32_host(yka_kv* kv, int layer, const float* k32, const float* v32, int M, int pos, int rotate) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); check_rows(kv, M);
+  if (!kv->r256()) throw std::runtime_error("this entry point exists for head_dim 256 only");
+  if (!k32 || !v32) throw std::runtime_error("null pointer");
+  if (pos < 0 || (long long)pos + M > kv->cfg.max_ctx) throw std::runtime_error("pos + M exceeds max_ctx");
+  const size_t nk = (size_t)M * kv->cfg.n_kv_heads * 256;
+  DevBuf dk(nk * 4), dv(nk * 4);
+  HIPCHK(hipMemcpy(dk.p, k32, nk * 4, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dv.p, v32, nk * 4, hipMemcpyHostToDevice));
+  HIPCHK(hipDeviceSynchronize());
+  launch_set_int(kv->d_pos, pos, kv->stream);
+  AppendArgs A{kv->view(layer), nullptr, nullptr, kv->d_pos, M};
+  A.k32 = dk.as<float>(); A.v32 = dv.as<float>(); A.rot = rotate != 0;
+  launch_append256(A, kv->stream);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipStreamSynchronize(kv->stream));
+  YKA_CATCH_INT
+}
+
+int yka_rotate_q256_host(const float* x32, int rows, uint16_t* q16) {
+  YKA_TRY
+  if (!x32 || !q16 || rows < 1) throw std::runtime_error("bad argument");
+  const size_t n = (size_t)rows * 256;
+  DevBuf dx(n * 4), dq(n * 2);
+  HIPCHK(hipMemcpy(dx.p, x32, n * 4, hipMemcpyHostToDevice));
+  launch_rotate_q256(dx.as<float>(), rows, dq.as<uint16_t>(), nullptr);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipDeviceSynchronize());
+  HIPCHK(hipMemcpy(q16, dq.p, n * 2, hipMemcpyDeviceToHost));
   YKA_CATCH_INT
 }
 

@@ -14,6 +14,7 @@
 // selects elements 7 - s/4 (low half) and 3 - s/4 (high half) of the word, so a word yields its 8 codes in the order
 // [7,3,6,2,5,1,4,0]; the query fragments are loaded in the same order.
 #include "yka_internal.h"
+#include "rot256_device.h"
 #include <hip/hip_fp16.h>
 
 namespace yka {
@@ -42,12 +43,14 @@ __device__ __forceinline__ uint8_t* page256(const KvView& kv, int kvh, int t) {
 // ---- quantize-on-append: grid (M, n_kv * 2), block 256 = one row, thread = channel ----
 __global__ void __launch_bounds__(256) append256_kernel(AppendArgs A) {
   __shared__ float red[4];
+  __shared__ float buf[256];
   __shared__ uint8_t fld[256];
   const int tok = blockIdx.x, kvh = blockIdx.y >> 1, isv = blockIdx.y & 1, d = threadIdx.x;
   const int pos = *A.d_pos + tok;
   if (pos < 0 || pos >= A.kv.max_ctx) return;
-  const uint16_t* src = (isv ? A.v16 : A.k16) + ((size_t)tok * A.kv.n_kv + kvh) * kD2;
-  const float x = __half2float(__ushort_as_half(src[d]));
+  const size_t e = ((size_t)tok * A.kv.n_kv + kvh) * kD2 + d;
+  float x = A.k32 ? (isv ? A.v32 : A.k32)[e] : __half2float(__ushort_as_half((isv ? A.v16 : A.k16)[e]));
+  if (A.rot) x = rotate256(x, buf, false);
   float am = fabsf(x);
 #pragma unroll
   for (int o = 32; o; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, 64));
@@ -72,6 +75,13 @@ __global__ void __launch_bounds__(256) append256_kernel(AppendArgs A) {
 }
 
 // ---- canonical image <-> pages: grid (n, n_kv), block 64: lanes 0..31 move K words, 32..63 V words ----
+// rotated query rows: grid rows, block 256
+__global__ void __launch_bounds__(256) rotate_q256_kernel(const float* x32, uint16_t* q16) {
+  __shared__ float buf[256];
+  const size_t e = (size_t)blockIdx.x * kD2 + threadIdx.x;
+  q16[e] = __half_as_ushort(__float2half_rn(rotate256(x32[e], buf, false)));
+}
+
 template <bool IMPORT>
 __global__ void __launch_bounds__(64) xfer256_kernel(KvView kv, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs) {
   const int t = blockIdx.x, kvh = blockIdx.y, j = threadIdx.x & 31, isv = threadIdx.x >> 5;
@@ -294,11 +304,16 @@ __global__ void __launch_bounds__(256) combine256_kernel(CombineArgs A) {
   float o = 0.f, L = 0.f;
 #pragma unroll
   for (int k = 0; k < 8; ++k) { o += s_o[k][tid]; L += s_wsum[k]; }
-  A.out16[((size_t)tok * A.n_heads + head) * kD2 + tid] = __half_as_ushort(__float2half_rn(L > 0.f ? o / L : 0.f));
+  float y = L > 0.f ? __fdiv_rn(o, L) : 0.f;
+  if (A.unrot) y = rotate256(y, s_w, true);        // inverse of the rotation of the V rows (src/q35_kernels.cu:1421); s_w is free again
+  A.out16[((size_t)tok * A.n_heads + head) * kD2 + tid] = __half_as_ushort(__float2half_rn(y));
 }
 
 void launch_append256(const AppendArgs& A, hipStream_t st) {
   hipLaunchKernelGGL(append256_kernel, dim3(A.M, A.kv.n_kv * 2), dim3(256), 0, st, A);
+}
+void launch_rotate_q256(const float* x32, int rows, uint16_t* q16, hipStream_t st) {
+  hipLaunchKernelGGL(rotate_q256_kernel, dim3(rows), dim3(256), 0, st, x32, q16);
 }
 void launch_attend256(const AttnArgs& A, hipStream_t st) {
   hipLaunchKernelGGL(attend256_kernel, dim3(A.S, A.kv.n_kv, (A.M + 1) / 2), dim3(256), 0, st, A);

@@ -43,7 +43,10 @@ __device__ __forceinline__ KvView slot_view(KvView v, const RowMap& R, int slot)
   return v;
 }
 
-struct AppendArgs { KvView kv; const uint16_t* k16; const uint16_t* v16; const int* d_pos; int M; RowMap rows; };
+// k32 / v32 / rot: 256-channel rows only (attend256.hip) - fp32 source rows instead of fp16 ones, and the signed Hadamard
+// rotation applied to every row before it is quantized (src/q35_kernels.cu:1036,1060 + launch_tb_requant)
+struct AppendArgs { KvView kv; const uint16_t* k16; const uint16_t* v16; const int* d_pos; int M; RowMap rows;
+                    const float* k32 = nullptr; const float* v32 = nullptr; int rot = 0; };
 
 // partial results of the split-KV kernels (same roles as pm/pl/pacc of the reference, args.hpp:10):
 //   pm, pl [rows_tok][S][n_heads] fp32; pacc16 [rows_tok][S][n_heads][128] fp16 = acc / l (normalised, so that fp16
@@ -81,6 +84,7 @@ void launch_combine(const CombineArgs&, hipStream_t);
 void launch_attn_post(const PostArgs&, hipStream_t);
 // the reference's own rows, head_dim 256 (attend256.hip): same argument structs, 67584-byte pages
 void launch_append256(const AppendArgs&, hipStream_t);
+void launch_rotate_q256(const float* x32, int rows, uint16_t* q16, hipStream_t);   // rotated query rows, rounded to fp16
 void launch_attend256(const AttnArgs&, hipStream_t);       // row tiles of 2 tokens x 6 heads for every width
 void launch_combine256(const CombineArgs&, hipStream_t);
 void launch_export_rows256(const KvView&, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs, hipStream_t);

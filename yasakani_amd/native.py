@@ -54,6 +54,10 @@ def _load():
         "yka_kvx256_probe": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_attn_post": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
         "yka_kv_export_rows256": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
+        "yka_append256_f32": (i32, [vp, i32, vp, vp, i32, vp, i32, vp]),
+        "yka_rotate_q256": (i32, [vp, i32, vp, vp]),
+        "yka_append256_f32_host": (i32, [vp, i32, vp, vp, i32, i32, i32]),
+        "yka_rotate_q256_host": (i32, [vp, i32, vp]),
         "yka_kv_import_rows256": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_append_attend_ms": (i32, [vp, vp, vp, vp, i32, vp, vp, vp, vp]),
         "yka_ms_call_host": (i32, [vp, vp, vp, vp, i32, vp, vp, vp]),
@@ -78,6 +82,7 @@ def _load():
 EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "yka_set_opt", "yka_kv_set_page_table",
            "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kvx256_probe", "yka_attn_post", "yka_append_attend_ms", "yka_ms_call_host",
            "yka_attn_post_host", "yka_kv_export_rows", "yka_kv_export_rows256", "yka_kv_import_rows256",
+           "yka_append256_f32", "yka_rotate_q256", "yka_append256_f32_host", "yka_rotate_q256_host",
            "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
            "yka_append_host", "yka_pass_capture", "yka_pass_launch", "yka_pass_destroy", "yka_attn_bench")
 
@@ -123,6 +128,15 @@ def codec_probe(x16):
     y = np.empty((rows, D), np.float32)
     _chk(lib().yka_codec_probe(_ptr(x), rows, _ptr(codes), _ptr(scales), _ptr(y)))
     return codes, scales, y
+
+
+def rotate_q256(x32):
+    """Rotated query rows: x32 [..., 256] fp32 -> fp16 of the signed Walsh-Hadamard rotation of every row."""
+    x = np.ascontiguousarray(x32, np.float32)
+    rows = x.size // 256
+    q = np.empty(x.shape, np.uint16)
+    _chk(lib().yka_rotate_q256_host(_ptr(x), rows, _ptr(q)))
+    return q.view(np.float16)
 
 
 def kvx256_probe(x, mode, rot):
@@ -190,6 +204,13 @@ class KvCache:
     # -- launch path: device addresses --
     def append(self, layer, d_k16, d_v16, M, d_pos, stream=0):
         _chk(lib().yka_append(self._h, layer, d_k16, d_v16, M, d_pos, stream))
+
+    def append256_f32_host(self, layer, k32, v32, pos, rotate=False):
+        """head_dim 256: quantize fp32 rows k32/v32 [M,n_kv_heads,256] into rows pos..pos+M-1, rotating each row first if asked."""
+        M = k32.shape[0]
+        k = np.ascontiguousarray(k32, np.float32).reshape(M, self.cfg.n_kv_heads, 256)
+        v = np.ascontiguousarray(v32, np.float32).reshape(M, self.cfg.n_kv_heads, 256)
+        _chk(lib().yka_append256_f32_host(self._h, layer, _ptr(k), _ptr(v), M, pos, int(bool(rotate))))
 
     def append_attend_ms(self, d_q16, d_k16, d_v16, M, d_row_pos, d_row_slot, d_out16, stream=0):
         """Multi-stream pass with device pointers: row t uses container d_row_slot[t] at position d_row_pos[t]."""
