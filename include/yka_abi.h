@@ -108,6 +108,16 @@ YKA_API int yka_append256_f32(yka_kv* kv, int layer, const float* d_k32, const f
  * in the place of the reference's bf16).  Attention over a rotated cache then needs option key 4 (outputs un-rotated). */
 YKA_API int yka_rotate_q256(const float* d_x32, int rows, uint16_t* d_q16, void* hip_stream);
 
+/* The step after attention for 256-channel heads; replaces the output part of launch_q35_combine (q35.hpp:153-156,
+ * q35_kernels.cu:1420-1428 with a8_group512_tail, a8_prologue.cuh:87-98,122-133), fp16 where the reference rounds to bf16:
+ * per token and per pair of heads (512 values) y * f16(sigmoid(gate)) -> f16 -> x sign -> 512-point Hadamard transform
+ * x 1/sqrt(512) -> f16 -> one scale alpha = max|v| / 127 and int8 codes.  d_y16 = attention outputs [M][n_heads][256]
+ * (what yka_attend wrote, un-rotated if option key 4 is set), d_gate16 the same shape, d_signs [n_heads * 256] (+1/-1),
+ * d_qx [M][n_heads * 256] int8, d_alpha [M][n_heads * 256 / 512] fp32.  The interleaved small-batch layout of the
+ * reference's int8 operand (a8_lo_off, a8_prologue.cuh:121) is not produced.  Allocates nothing, synchronises nothing. */
+YKA_API int yka_attn_out256(const uint16_t* d_y16, const uint16_t* d_gate16, const int8_t* d_signs, int M, int n_heads,
+                            int8_t* d_qx, float* d_alpha, void* hip_stream);
+
 /* The step between the QKV projection and the cache, fused with quantize-on-append; replaces launch_q35_attn_post
  * (q35.hpp:97-105, q35_kernels.cu:1013-1065) + launch_tb_requant (q35_kernels.cu:1084-1092) for 128-channel heads:
  * per head, Q and K rows are RMS-normalised (x / sqrt(mean x^2 + eps) * (1 + w)), get the rotary embedding on their
@@ -135,6 +145,9 @@ YKA_API int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float*
 YKA_API int yka_ms_call_host(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M,
                              const int32_t* row_pos, const int32_t* row_slot, uint16_t* out16);
 
+/* Host-pointer form of yka_attn_out256. */
+YKA_API int yka_attn_out256_host(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads,
+                                 int8_t* qx, float* alpha);
 /* Host-pointer forms of yka_append256_f32 and yka_rotate_q256. */
 YKA_API int yka_append256_f32_host(yka_kv* kv, int layer, const float* k32, const float* v32, int M, int pos, int rotate);
 YKA_API int yka_rotate_q256_host(const float* x32, int rows, uint16_t* q16);

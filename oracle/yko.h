@@ -30,6 +30,8 @@
  *   yko_flat4_decode256      independent numpy restatement; packing against numpy.unpackbits on the
  *                            big-endian byte image of the words
  *   yko_int8_encode256       pinned: closed-form properties, independent numpy restatement
+ *   yko_attn_out256          pinned: scipy Sylvester matrix of order 512 (exact on integer inputs with an open gate),
+ *                            numpy fp64 sigmoid gate within the fp16 roundings, closed forms of the int8 groups
  *   yko_rotate128            pinned: scipy Sylvester matrix (exact on integer rows), forward x inverse = identity,
  *                            q.k invariance
  *   yko_attn_post            pinned: numpy fp64 RMS normalisation and complex-multiplication rotary form within the
@@ -73,6 +75,9 @@ void yko_flat4_decode256(const uint32_t* words32, float scale, float* y);   /* s
 void yko_int8_encode256(const float* x, int8_t* q, float* scale);        /* src/kvx_codec.cuh:50-69 */
 /* round trip of the reference's codec probe (src/kvx_probe.cu:7-20); mode 0 int8 rows, mode 1 flat int4 */
 void yko_kvx_probe256(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, float* y);
+/* the step after attention for 256-channel heads: sigmoid gate, signs, 512-point Hadamard transform, int8 groups of 512
+ * (src/q35_kernels.cu:1420-1428, src/a8_prologue.cuh:87-98,122-133) */
+void yko_attn_out256(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads, int8_t* qx, float* alpha);
 
 /* ---- between the QKV projection and the cache (yko_post.c; src/q35_kernels.cu:1013-1065 for 128-channel heads) ---- */
 void yko_rotate128(const float* x, float* y, int inverse, float factor);

@@ -59,6 +59,7 @@ def lib():
         L.yko_flat4_decode256.argtypes = [vp, C.c_float, vp]
         L.yko_int8_encode256.argtypes = [vp, vp, vp]
         L.yko_kvx_probe256.argtypes = [vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp]
+        L.yko_attn_out256.argtypes = [vp, vp, vp, C.c_int, C.c_int, vp, vp]
         L.yko_rotate128.argtypes = [vp, vp, C.c_int, C.c_float]
         L.yko_attn_post.argtypes = [vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, C.c_float, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp]
         L.yko_unrotate_out.argtypes = [vp, C.c_int, vp]
@@ -292,3 +293,14 @@ def unrotate_out(y32):
     out = np.empty(y32.shape, np.uint16)
     lib().yko_unrotate_out(_p(y32), int(y32.size // 128), _p(out))
     return out
+
+
+def attn_out256(y16, gate16, signs):
+    """the step after attention for 256-channel heads: y16, gate16 [M, n_heads, 256] fp16, signs [n_heads*256] int8
+    -> (qx [M, n_heads*256] int8, alpha [M, n_heads*256/512] f32)"""
+    y = _as_u16(y16); g = _as_u16(gate16)
+    M, H, _ = y.shape
+    sg = np.ascontiguousarray(signs, np.int8)
+    qx = np.empty((M, H * 256), np.int8); alpha = np.empty((M, H * 256 // 512), np.float32)
+    lib().yko_attn_out256(_p(y), _p(g), _p(sg), M, H, _p(qx), _p(alpha))
+    return qx, alpha

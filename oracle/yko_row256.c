@@ -102,3 +102,40 @@ void yko_kvx_probe256(const float* x, int rows, int mode, int rot, int8_t* q8, u
     if (rot) yko_kvx_rotate256(dq, y + (size_t)r * 256, 1); else memcpy(y + (size_t)r * 256, dq, sizeof dq);
   }
 }
+
+/* ---- the step after attention for 256-channel heads (src/q35_kernels.cu:1420-1428, src/a8_prologue.cuh:87-98,122-133),
+ *      with fp16 in the place of the reference's bf16 roundings ----
+ * Per token and per pair of heads (512 consecutive values e = head * 256 + d):
+ *   sg = f16(1 / (1 + expf(-gate)));  y2 = f16(y * sg);  u = y2 * sign[e]
+ *   v  = f16(H512(u) * 2^-4.5)        (Sylvester Hadamard transform: stages h = 1 .. 256, the element whose index has bit h
+ *                                      set becomes partner - self, the other self + partner; 0.0441941738... = 1/sqrt(512))
+ *   alpha = max|v| / 127;  q = alpha > 0 ? rint(v / alpha) : 0, clamped to +-127
+ * y16: attention outputs [M][n_heads][256] fp16 (already rotated back and rounded by the combiner); gate16 the same shape;
+ * signs [n_heads * 256] (+1 / -1); qx [M][n_heads * 256] int8; alpha [M][n_heads * 256 / 512]. */
+static float f16r_(float x) { return yko_h2f(yko_f2h(x)); }
+void yko_attn_out256(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads, int8_t* qx, float* alpha) {
+  const int N = n_heads * 256, nb = N / 512;
+  for (int t = 0; t < M; ++t)
+    for (int b = 0; b < nb; ++b) {
+      float a[512], c[512];
+      for (int i = 0; i < 512; ++i) {
+        const size_t e = (size_t)t * N + (size_t)b * 512 + i;
+        const float sg = f16r_(1.f / (1.f + expf(-yko_h2f(gate16[e]))));
+        const float y2 = f16r_(yko_h2f(y16[e]) * sg);
+        a[i] = y2 * (float)signs[b * 512 + i];
+      }
+      for (int h = 1; h < 512; h *= 2) {
+        for (int i = 0; i < 512; ++i) { const float self = a[i], other = a[i ^ h]; c[i] = (i & h) ? other - self : self + other; }
+        memcpy(a, c, sizeof a);
+      }
+      float am = 0.f;
+      for (int i = 0; i < 512; ++i) { a[i] = f16r_(a[i] * 0.044194173824159216f); am = fmaxf(am, fabsf(a[i])); }
+      const float al = am / 127.f;
+      alpha[(size_t)t * nb + b] = al;
+      for (int i = 0; i < 512; ++i) {
+        int q = al > 0.f ? (int)rintf(a[i] / al) : 0;
+        q = q < -127 ? -127 : (q > 127 ? 127 : q);
+        qx[(size_t)t * N + (size_t)b * 512 + i] = (int8_t)q;
+      }
+    }
+}

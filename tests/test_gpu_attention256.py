@@ -139,3 +139,22 @@ def test_rotated_rows_and_unrotated_outputs(native, oracle):
             plain = p @ v32[:ctx + t + 1, h // 6].astype(np.float64)
             worst = max(worst, np.linalg.norm(out[t, h].astype(np.float64) - plain) / np.linalg.norm(plain))
     assert worst < 0.35, worst
+
+
+def test_output_step_gate_hadamard_int8(native, oracle):
+    rng = np.random.default_rng(31)
+    M, H = 7, 24
+    y = rng.standard_normal((M, H, D)).astype(np.float16)
+    gate = (rng.standard_normal((M, H, D)) * 3).astype(np.float16)
+    signs = rng.choice(np.array([-1, 1], np.int8), size=H * D)
+    y[2, 6:8] = 0                                          # a zero group: scale 0, codes 0
+    y[3] = np.round(y[3].astype(np.float32) * 2); gate[3] = 60.0   # integers with the gate open: every operation exact
+    qx, alpha = native.attn_out256(y, gate, signs)
+    rq, ra = oracle.attn_out256(y, gate, signs)
+    assert np.array_equal(qx[3], rq[3]) and np.array_equal(alpha[3].view(np.uint32), ra[3].view(np.uint32))
+    assert alpha[2, 3] == 0 and not qx[2, 1536:2048].any()
+    # elsewhere the only operation that may differ between device and host is expf inside the sigmoid, whose result is
+    # rounded to fp16 right away: scales agree to fp16 resolution, codes differ by at most one step and almost never
+    assert np.allclose(alpha, ra, rtol=2e-3, atol=0)
+    diff = np.abs(qx.astype(np.int32) - rq.astype(np.int32))
+    assert diff.max() <= 1 and (diff != 0).mean() < 0.01, (diff.max(), (diff != 0).mean())

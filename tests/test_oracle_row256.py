@@ -118,3 +118,44 @@ def test_probe_round_trip_error(mode, rot):
     if mode == 1 and not rot:
         w, s, xq = yko.flat4_encode256(x)
         assert np.array_equal(words, w) and np.array_equal(scales, s) and np.array_equal(y, xq)
+
+
+# ---- the step after attention: sigmoid gate, signs, 512-point Hadamard transform, int8 groups of 512 ----
+
+def test_attn_out_transform_is_sylvester_512_exact_on_integers():
+    from scipy.linalg import hadamard as had
+    rng = np.random.default_rng(21)
+    M, H = 2, 24
+    y = rng.integers(-4, 5, size=(M, H, 256)).astype(np.float16)
+    gate = np.full((M, H, 256), 60.0, np.float16)          # sigmoid(60) rounds to 1: the gate is open
+    signs = rng.choice(np.array([-1, 1], np.int8), size=H * 256)
+    qx, alpha = yko.attn_out256(y, gate, signs)
+    u = (y.astype(np.float64).reshape(M, -1) * signs).reshape(M, -1, 512)
+    v = (u @ had(512).astype(np.float64)) * np.float32(0.044194173824159216)
+    v = v.astype(np.float32).astype(np.float16).astype(np.float32)      # integer sums are exact; one fp32 product, one fp16 rounding
+    al = (np.abs(v).max(-1) / np.float32(127)).astype(np.float32)
+    assert np.array_equal(alpha, al)
+    q = np.clip(np.rint((v / al[..., None]).astype(np.float32)), -127, 127).astype(np.int8)
+    assert np.array_equal(qx, q.reshape(M, -1))
+    assert np.all(np.abs(qx.reshape(M, -1, 512)).max(-1) == 127)
+
+
+def test_attn_out_gate_and_zero_group():
+    rng = np.random.default_rng(22)
+    M, H = 3, 24
+    y = rng.standard_normal((M, H, 256)).astype(np.float16)
+    gate = (rng.standard_normal((M, H, 256)) * 3).astype(np.float16)
+    signs = rng.choice(np.array([-1, 1], np.int8), size=H * 256)
+    y[1, 4:6] = 0                                          # one whole group of 512 is zero: alpha 0, codes 0
+    qx, alpha = yko.attn_out256(y, gate, signs)
+    assert alpha[1, 2] == 0 and np.all(qx[1, 1024:1536] == 0)
+    from scipy.linalg import hadamard as had
+    sg = 1.0 / (1.0 + np.exp(-gate.astype(np.float64)))
+    u = (y.astype(np.float64) * sg).reshape(M, -1) * signs
+    v = (u.reshape(M, -1, 512) @ had(512).astype(np.float64)) / np.sqrt(512.0)
+    deq = qx.reshape(M, -1, 512).astype(np.float64) * alpha[..., None]
+    # three fp16 roundings and an 8-bit grid: 127 levels over the group's range
+    err = np.abs(deq - v).max(-1)
+    assert np.all(err <= np.abs(v).max(-1) * (0.5 / 127 + 4e-3) + 1e-6)
+    # the transform is orthonormal: the energy of a group survives up to the quantization error
+    assert np.allclose(np.linalg.norm(deq, axis=-1), np.linalg.norm(u.reshape(M, -1, 512), axis=-1), rtol=0.02, atol=1e-6)

@@ -475,6 +475,33 @@ int yka_rotate_q256_host(const float* x32, int rows, uint16_t* q16) {
   YKA_CATCH_INT
 }
 
+int yka_attn_out256(const uint16_t* d_y16, const uint16_t* d_gate16, const int8_t* d_signs, int M, int n_heads, int8_t* d_qx,
+                    float* d_alpha, void* hip_stream) {
+  YKA_TRY
+  if (!d_y16 || !d_gate16 || !d_signs || !d_qx || !d_alpha) throw std::runtime_error("null pointer");
+  if (M < 1 || n_heads < 2 || (n_heads & 1)) throw std::runtime_error("M must be positive and n_heads even");
+  launch_attn_out256(d_y16, d_gate16, d_signs, M, n_heads, d_qx, d_alpha, (hipStream_t)hip_stream);
+  HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_attn_out256_host(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads, int8_t* qx, float* alpha) {
+  YKA_TRY
+  if (!y16 || !gate16 || !signs || !qx || !alpha) throw std::runtime_error("null pointer");
+  if (M < 1 || n_heads < 2 || (n_heads & 1)) throw std::runtime_error("M must be positive and n_heads even");
+  const size_t n = (size_t)M * n_heads * 256, ng = n / 512;
+  DevBuf dy(n * 2), dg(n * 2), ds((size_t)n_heads * 256), dq(n), da(ng * 4);
+  HIPCHK(hipMemcpy(dy.p, y16, n * 2, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dg.p, gate16, n * 2, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(ds.p, signs, (size_t)n_heads * 256, hipMemcpyHostToDevice));
+  launch_attn_out256(dy.as<uint16_t>(), dg.as<uint16_t>(), ds.as<int8_t>(), M, n_heads, dq.as<int8_t>(), da.as<float>(), nullptr);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipDeviceSynchronize());
+  HIPCHK(hipMemcpy(qx, dq.p, n, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(alpha, da.p, ng * 4, hipMemcpyDeviceToHost));
+  YKA_CATCH_INT
+}
+
 int yka_kv_export_rows256(yka_kv* kv, int layer, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs) {
   YKA_TRY
   on_device(kv); check_layer(kv, layer); check_range(kv, pos0, n);

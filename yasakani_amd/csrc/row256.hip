@@ -6,6 +6,7 @@
 // One workgroup of 256 threads (4 waves) per row, thread d owns channel d.
 #include "yka_internal.h"
 #include "rot256_device.h"
+#include <hip/hip_fp16.h>
 
 namespace yka {
 namespace {
@@ -66,7 +67,58 @@ __global__ void __launch_bounds__(256) row256_decode_kernel(int mode, int rot, c
   y[(size_t)row * 256 + d] = v;
 }
 
+// The step after attention for 256-channel heads (src/q35_kernels.cu:1420-1428, src/a8_prologue.cuh:87-98,122-133), fp16 in
+// the place of the reference's bf16 roundings: sigmoid gate, signs, 512-point Hadamard transform x 1/sqrt(512), fp16
+// rounding, int8 with one scale per group of 512.  grid (n_heads / 2, M), block 512: thread = element of the group.
+__global__ void __launch_bounds__(512) attn_out256_kernel(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int n_heads,
+                                                          int8_t* qx, float* alpha) {
+  __shared__ float buf[512];
+  __shared__ float red[8];
+  const int blk = blockIdx.x, tok = blockIdx.y, tid = threadIdx.x;
+  const int N = n_heads * 256;
+  const size_t e = (size_t)tok * N + (size_t)blk * 512 + tid;
+  const float gate = __half2float(__ushort_as_half(gate16[e]));
+  float sg = __fdiv_rn(1.f, __fadd_rn(1.f, expf(-gate)));
+  asm volatile("" : "+v"(sg));                     // two roundings (fp32, then fp16), never one of the exact quotient
+  sg = __half2float(__float2half_rn(sg));
+  float y2 = __fmul_rn(__half2float(__ushort_as_half(y16[e])), sg);
+  asm volatile("" : "+v"(y2));
+  y2 = __half2float(__float2half_rn(y2));
+  float v = __fmul_rn(y2, (float)signs[blk * 512 + tid]);
+#pragma unroll
+  for (int h = 1; h < 64; h *= 2) {
+    const float q = __shfl_xor(v, h, 64);
+    v = (tid & h) ? __fsub_rn(q, v) : __fadd_rn(v, q);
+  }
+#pragma unroll
+  for (int h = 64; h < 512; h *= 2) {
+    __syncthreads();
+    buf[tid] = v;
+    __syncthreads();
+    const float q = buf[tid ^ h];
+    v = (tid & h) ? __fsub_rn(q, v) : __fadd_rn(v, q);
+  }
+  v = __fmul_rn(v, 0.044194173824159216f);
+  asm volatile("" : "+v"(v));
+  v = __half2float(__float2half_rn(v));
+  float am = fabsf(v);
+#pragma unroll
+  for (int o = 32; o; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, 64));
+  if ((tid & 63) == 0) red[tid >> 6] = am;
+  __syncthreads();
+  am = fmaxf(fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3])), fmaxf(fmaxf(red[4], red[5]), fmaxf(red[6], red[7])));
+  const float al = __fdiv_rn(am, 127.f);
+  if (tid == 0) alpha[(size_t)tok * (N / 512) + blk] = al;
+  int q = al > 0.f ? __float2int_rn(__fdiv_rn(v, al)) : 0;
+  q = max(-127, min(127, q));
+  qx[e] = (int8_t)q;
+}
+
 }  // namespace
+
+void launch_attn_out256(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads, int8_t* qx, float* alpha, hipStream_t st) {
+  hipLaunchKernelGGL(attn_out256_kernel, dim3(n_heads / 2, M), dim3(512), 0, st, y16, gate16, signs, n_heads, qx, alpha);
+}
 
 void launch_row256_encode(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, hipStream_t st) {
   hipLaunchKernelGGL(row256_encode_kernel, dim3(rows), dim3(256), 0, st, x, mode, rot, q8, words, scales);

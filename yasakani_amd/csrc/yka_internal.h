@@ -98,6 +98,8 @@ void launch_set_int(int* p, int v, hipStream_t);
 // the reference's own 256-channel row format (row256.hip): mode 0 = int8 rows, 1 = flat int4 (32 MSB-first words per row)
 void launch_row256_encode(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, hipStream_t);
 void launch_row256_decode(int rows, int mode, int rot, const int8_t* q8, const uint32_t* words, const float* scales, float* y, hipStream_t);
+// the step after attention for 256-channel heads: gate, signs, 512-point Hadamard transform, int8 groups of 512 (n_heads even)
+void launch_attn_out256(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads, int8_t* qx, float* alpha, hipStream_t);
 
 // start of the (page, kv head) block that holds token t
 __device__ __forceinline__ uint8_t* kv_page(const KvView& kv, int kvh, int t) {

@@ -55,6 +55,8 @@ def _load():
         "yka_attn_post": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
         "yka_kv_export_rows256": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_append256_f32": (i32, [vp, i32, vp, vp, i32, vp, i32, vp]),
+        "yka_attn_out256": (i32, [vp, vp, vp, i32, i32, vp, vp, vp]),
+        "yka_attn_out256_host": (i32, [vp, vp, vp, i32, i32, vp, vp]),
         "yka_rotate_q256": (i32, [vp, i32, vp, vp]),
         "yka_append256_f32_host": (i32, [vp, i32, vp, vp, i32, i32, i32]),
         "yka_rotate_q256_host": (i32, [vp, i32, vp]),
@@ -82,7 +84,7 @@ def _load():
 EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "yka_set_opt", "yka_kv_set_page_table",
            "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kvx256_probe", "yka_attn_post", "yka_append_attend_ms", "yka_ms_call_host",
            "yka_attn_post_host", "yka_kv_export_rows", "yka_kv_export_rows256", "yka_kv_import_rows256",
-           "yka_append256_f32", "yka_rotate_q256", "yka_append256_f32_host", "yka_rotate_q256_host",
+           "yka_attn_out256", "yka_attn_out256_host", "yka_append256_f32", "yka_rotate_q256", "yka_append256_f32_host", "yka_rotate_q256_host",
            "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
            "yka_append_host", "yka_pass_capture", "yka_pass_launch", "yka_pass_destroy", "yka_attn_bench")
 
@@ -128,6 +130,20 @@ def codec_probe(x16):
     y = np.empty((rows, D), np.float32)
     _chk(lib().yka_codec_probe(_ptr(x), rows, _ptr(codes), _ptr(scales), _ptr(y)))
     return codes, scales, y
+
+
+def attn_out256(y16, gate16, signs):
+    """The step after attention for 256-channel heads: y16, gate16 [M, n_heads, 256] fp16, signs [n_heads*256] int8 ->
+    (qx [M, n_heads*256] int8, alpha [M, n_heads*256/512] f32)."""
+    y = np.ascontiguousarray(y16); g = np.ascontiguousarray(gate16)
+    M, H, _ = y.shape
+    y = _u16(y, (M, H, 256)); g = _u16(g, (M, H, 256))
+    sg = np.ascontiguousarray(signs, np.int8)
+    if sg.shape != (H * 256,):
+        raise ValueError("signs needs n_heads * 256 entries")
+    qx = np.empty((M, H * 256), np.int8); alpha = np.empty((M, H * 256 // 512), np.float32)
+    _chk(lib().yka_attn_out256_host(_ptr(y), _ptr(g), _ptr(sg), M, H, _ptr(qx), _ptr(alpha)))
+    return qx, alpha
 
 
 def rotate_q256(x32):
