@@ -36,7 +36,7 @@ __device__ __forceinline__ uint32_t nib(uint32_t w, uint32_t magic) { return (w 
 __device__ __forceinline__ uint8_t* page256(const KvView& kv, int kvh, int t) {
   const int lp = t / kPageTok;
   int pp = lp;
-  if (kv.table) asm volatile("s_load_dword %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=s"(pp) : "s"(kv.table), "s"(lp * 4) : "memory");
+  if (kv.table) pp = table_entry_scalar(kv.table, lp);
   return kv.base + (size_t)(pp * kv.n_kv + kvh) * kPage256Bytes;
 }
 

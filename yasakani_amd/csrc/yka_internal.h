@@ -108,15 +108,25 @@ __device__ __forceinline__ uint8_t* kv_page(const KvView& kv, int kvh, int t) {
   return kv.base + (size_t)(pp * kv.n_kv + kvh) * kPageBytes;
 }
 
+// table[index] through the scalar data path; pointer and index are forced into scalar registers (they are uniform over
+// the wave by contract, but the compiler cannot always prove it, e.g. inside a branch on a wave-uniform condition)
+__device__ __forceinline__ int table_entry_scalar(const int32_t* table, int index) {
+  const uint64_t a = (uint64_t)(uintptr_t)table;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  const uint64_t base = ((uint64_t)hi << 32) | lo;
+  const int off = __builtin_amdgcn_readfirstlane(index * 4);
+  int v;
+  asm volatile("s_load_dword %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(base), "s"(off) : "memory");
+  return v;
+}
+
 // The same for a token index that is uniform over the wave (the attention kernels' tile loops).  The page-table entry is
 // fetched through the scalar data path: a vector load would share its completion counter with the tile loads a wave
 // keeps in flight, so waiting for the entry would wait for all of them.  (Read only; the table is written by the host.)
 __device__ __forceinline__ uint8_t* kv_page_uniform(const KvView& kv, int kvh, int t) {
   const int lp = t / kPageTok;
   int pp = lp;
-  if (kv.table) {
-    asm volatile("s_load_dword %0, %1, %2\n\ts_waitcnt lgkmcnt(0)" : "=s"(pp) : "s"(kv.table), "s"(lp * 4) : "memory");
-  }
+  if (kv.table) pp = table_entry_scalar(kv.table, lp);
   return kv.base + (size_t)(pp * kv.n_kv + kvh) * kPageBytes;
 }
 
