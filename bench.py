@@ -310,8 +310,11 @@ def main():
 
     us, gbs, roof, out = measure(M, args.steps, args.warmup)
     line = {
-        "metric": f"effective KV GB/s per layer call, int4-KV GQA verify-{M} at {ctx} ctx" if M > 1 else
-                  f"effective KV GB/s per layer call, int4-KV GQA decode at {ctx} ctx",
+        # the headline workload carries BASELINE.json's metric text verbatim; `value` is its effective-KV-GB/s component,
+        # `us_per_layer` and `hbm_peak_frac` are the other two
+        "metric": ("\u00b5s/layer + effective KV GB/s (% HBM peak), int4-KV GQA verify-64 at 32k ctx" if (M, ctx) == (64, 32768) else
+                   f"\u00b5s/layer + effective KV GB/s (% HBM peak), int4-KV GQA verify-{M} at {ctx} ctx" if M > 1 else
+                   f"\u00b5s/layer + effective KV GB/s (% HBM peak), int4-KV GQA decode at {ctx} ctx"),
         "value": gbs, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": us / 1e3, "us_per_layer": us, "hbm_peak_frac": gbs / HBM_PEAK_GBS,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
