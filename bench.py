@@ -271,6 +271,8 @@ def main():
     ap.add_argument("--rows", type=int, default=64, help="query rows of the window (64 = headline; 1 = decode)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary decode / verify-16 / verify-32 lines")
+    ap.add_argument("--batched-only", action="store_true",
+                    help="run only the multi-stream (batched decode) passes and print their figures (for profiling that kernel)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three device-to-device copies of 256 MiB (a kernel of known traffic, for scaling FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -308,6 +310,10 @@ def main():
         roof["hbm_frac"] = by / (k_us * 1e-6) / 1e9 / HBM_PEAK_GBS
         return us, by / (us * 1e-6) / 1e9, roof, out
 
+    if args.batched_only:
+        print(json.dumps({"batched_decode": batched_decode(torch, native, kv, ctx, L, kn, vn, q, calls=max(8, args.steps // 8))}))
+        kv.close()
+        return
     us, gbs, roof, out = measure(M, args.steps, args.warmup)
     line = {
         # the headline workload carries BASELINE.json's metric text verbatim; `value` is its effective-KV-GB/s component,
