@@ -285,6 +285,9 @@ void launch_attend_narrow(const AttnArgs& A, hipStream_t st) {
 // combiner (reference: src/attention_kv4q.cu:325-332): M2 = max pm; w_s = pm_s > -1e29 ? 2^(pm_s - M2) * pl_s : 0;
 // y = sum w_s * (acc_s / l_s) / sum w_s.  grid (n_heads, M), block 256: 16 lanes x 8 channels cover a row, 16 split
 // lanes run in parallel and are summed through LDS.  S <= 256.
+// kInFlight = partial rows a split lane requests before it uses any: 16 covers 256 splits in one memory round trip (few,
+// long workgroups: decode); 4 keeps the register count low where thousands of workgroups run (wide windows).
+template <int kInFlight>
 __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
   __shared__ float s_w[256];
   __shared__ float s_o[16][kD + 4];
@@ -308,16 +311,16 @@ __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
   // 16 split lanes; each takes splits sl, sl+16, ...; loads are issued 4 at a time so that their latencies overlap
   const uint16_t* src = A.pacc16 + p0 * kD + c8;
   const size_t stride = (size_t)A.n_heads * kD;
-  for (int s0 = sl; s0 < A.S; s0 += 64) {
-    uint4 u[4]; float w[4];
+  for (int s0 = sl; s0 < A.S; s0 += 16 * kInFlight) {
+    uint4 u[kInFlight]; float w[kInFlight];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < kInFlight; ++k) {
       const int sp = s0 + 16 * k;
       w[k] = sp < A.S ? s_w[sp] : 0.f;
       u[k] = sp < A.S ? *reinterpret_cast<const uint4*>(src + (size_t)sp * stride) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < kInFlight; ++k) {
       const h8 v = __builtin_bit_cast(h8, u[k]);
 #pragma unroll
       for (int c = 0; c < 8; ++c) acc[c] += w[k] * (float)v[c];
@@ -356,7 +359,8 @@ __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
   if (tid < kD) A.out16[((size_t)tok * A.n_heads + head) * kD + tid] = __half_as_ushort(__float2half_rn(y));
 }
 void launch_combine(const CombineArgs& A, hipStream_t st) {
-  hipLaunchKernelGGL(combine_kernel, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
+  if (A.S > 64) hipLaunchKernelGGL(combine_kernel<16>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
+  else hipLaunchKernelGGL(combine_kernel<4>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
 }
 
 }  // namespace yka
