@@ -15,15 +15,16 @@
 //   * the running maximum of a row is only raised when a score exceeds it by more than 2^8: accumulators stay in
 //     their registers untouched on almost every tile;
 //   * LDS is double buffered: tile n+1 is dequantized while tile n is consumed; one barrier per tile.
-// LDS image of one tile (18944 bytes):
+// LDS image of one tile (19456 bytes):
 //   K  [32 keys][272 B]   chunk 4m+g of a key = channels 32m+8g..+7 in the order n0,n4,n1,n5,n2,n6,n3,n7; the 272-byte
 //                          pitch makes the lanes of a fragment read hit distinct banks
 //   V  [128 rows][80 B]   channel 8*dw+c lives in row 16*sigma(c)+dw, sigma(c) = 2*(c&3) + (c>>2): the 16 lanes that
 //                          dequantize one byte position write 16 consecutive rows, and an output lane ends up with runs
 //                          of 8 consecutive channels.  Inside a row token 16u+8a+4h+b sits at position 16u+8h+4a+b, so
 //                          the 8 tokens an MFMA lane needs are 16 contiguous bytes
-// The K group scales are not staged: every lane needs the scales of 16 keys x 4 groups, the same for all 32 lanes of a
-// wave half, so they come straight from the page's scale plane (L1/L2 resident) one tile ahead and stay in registers.
+//   S  [4 groups][4 a][2 h][4 b] fp32   K group scale of key 8a+4h+b: every lane needs the scales of 16 keys x 4 groups,
+//                          the same for all 32 lanes of a wave half; converted to fp32 once per workgroup, each lane reads
+//                          four of them per instruction (a broadcast read) and multiplies with a plain fp32 FMA
 // Partial results leave through the same LDS after the last tile so that every store writes whole 256-byte rows.
 #include "yka_internal.h"
 #include <hip/hip_fp16.h>
@@ -42,7 +43,7 @@ __device__ __forceinline__ uint32_t as_u32(h2 h) { return __builtin_bit_cast(uin
 constexpr uint32_t kMagic = 0x64006400u;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kKPitch = 272, kVPitch = 80;
-constexpr int kLdsK = 0, kLdsV = 32 * kKPitch, kLdsBuf = kLdsV + 128 * kVPitch;   // 18944
+constexpr int kLdsK = 0, kLdsV = 32 * kKPitch, kLdsS = kLdsV + 128 * kVPitch, kLdsBuf = kLdsS + 512;   // 19456
 constexpr int NT = 256;                        // threads per workgroup
 constexpr float kRaise = 8.f;                  // log2 slack before a running maximum is raised
 
@@ -50,6 +51,7 @@ struct Raw {                                   // one thread's share of a raw 32
   uint32_t kw[2];
   uint32_t vw[2];
   uint32_t vs;
+  uint32_t ks;                                 // threads 0..127: fp16 scale of (key tid/4, group tid%4)
 };
 
 // Byte offsets of one thread inside a page, fixed for the whole kernel; the page pointer and the tile's first token
@@ -57,8 +59,9 @@ struct Raw {                                   // one thread's share of a raw 32
 struct LaneOffs { uint32_t k, v, vs, ks; };
 __device__ __forceinline__ LaneOffs lane_offs(int tid, int h) {
   const uint32_t pair = tid >> 4, dw = tid & 15;
+  (void)h;
   return LaneOffs{(uint32_t)tid * 4u, kPageVc + pair * 128u + dw * 4u, kPageVs + (dw >> 2) * (kPageTok * 2u) + pair * 4u,
-                  kPageKs + (uint32_t)h * 32u};
+                  kPageKs + (uint32_t)tid * 2u};
 }
 __device__ __forceinline__ void load_raw(const uint8_t* pg, int tp, const LaneOffs& L, Raw& R) {
   const uint8_t* kt = pg + (uint32_t)tp * 64u;            // K and V code rows of the tile start here (+ plane offset)
@@ -67,6 +70,7 @@ __device__ __forceinline__ void load_raw(const uint8_t* pg, int tp, const LaneOf
   R.vw[0] = *reinterpret_cast<const uint32_t*>(kt + L.v);
   R.vw[1] = *reinterpret_cast<const uint32_t*>(kt + L.v + 64);
   R.vs = *reinterpret_cast<const uint32_t*>(pg + (uint32_t)tp * 2u + L.vs);
+  if (L.k < 128 * 4) R.ks = *reinterpret_cast<const uint16_t*>(pg + (uint32_t)tp * 8u + L.ks);   // waves 0 and 1 only
 }
 
 // (w & mask) | magic as one bit-field insert: `magic` (0x64006400, no bit inside either nibble mask) is kept opaque to
@@ -86,6 +90,10 @@ __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw&
     o.w = as_u32(as_h2(nib(t, 0x00f000f0u, magic)) - c1152);
     *reinterpret_cast<uint4*>(buf + kLdsK + key * kKPitch + (4 * (p & 3) + (p >> 2)) * 16) = o;
   }
+  if (tid < 128) {                                                   // K group scales as fp32, [group][a][h][b] for key 8a+4h+b
+    const int key = tid >> 2, m = tid & 3;
+    reinterpret_cast<float*>(buf + kLdsS)[m * 32 + (key >> 3) * 8 + (key & 7)] = (float)__builtin_bit_cast(_Float16, (uint16_t)R.ks);
+  }
   {
     const int pair = tid >> 4, dw = tid & 15;
     const int t0 = 2 * pair;                                         // token 16u + 8a + 4h + b -> position 16u + 8h + 4a + b
@@ -103,17 +111,6 @@ __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw&
       *reinterpret_cast<uint32_t*>(vb + 16 * (2 * (c0 & 3) + (c0 >> 2)) * kVPitch) = as_u32(lo);
       *reinterpret_cast<uint32_t*>(vb + 16 * (2 * (c1 & 3) + (c1 >> 2)) * kVPitch) = as_u32(hi);
     }
-  }
-}
-
-// group scales of the 16 keys whose scores a lane of half h receives: keys 8a + 4h + b of the tile, 4 fp16 each
-struct KScales { uint4 v[4][2]; };
-__device__ __forceinline__ void load_kscales(const uint8_t* pg, int tp, const LaneOffs& L, KScales& K) {
-  const uint8_t* st = pg + (uint32_t)tp * 8u;
-#pragma unroll
-  for (int a = 0; a < 4; ++a) {
-    K.v[a][0] = *reinterpret_cast<const uint4*>(st + L.ks + 64 * a);
-    K.v[a][1] = *reinterpret_cast<const uint4*>(st + L.ks + 64 * a + 16);
   }
 }
 
@@ -174,14 +171,12 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
   }
 
   Raw raw0, raw1;                              // raw codes of the next two tiles: loads run two tiles ahead of their use
-  KScales sc;
   const LaneOffs offs = lane_offs(tid, h);
   uint32_t magic = kMagic;
   asm volatile("" : "+v"(magic));
   auto load_tile_raw = [&](int T, Raw& r) { load_raw(kv_page_uniform(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, r); };
   if (tile0 < tile1) {
     load_tile_raw(tile0, raw0);
-    load_kscales(kv_page_uniform(A.kv, kvh, tile0 << 5), (tile0 << 5) % kPageTok, offs, sc);
     dequant_to_lds(lds[0], tid, raw0, magic);
     if (tile0 + 1 < tile1) load_tile_raw(tile0 + 1, raw1);
     if (tile0 + 2 < tile1) load_tile_raw(tile0 + 2, raw0);
@@ -213,6 +208,9 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         const h8 k0 = kfr[2 * m], k1 = kfr[2 * m + 1];
+        float4 sc4[4];                         // fp32 scales of group m for the lane's 16 keys, the same for all 32 lanes of a half
+#pragma unroll
+        for (int a = 0; a < 4; ++a) sc4[a] = *reinterpret_cast<const float4*>(buf + kLdsS + ((m * 4 + a) * 2 + h) * 16);
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt) {
           {                                    // row tiles past the wave's last row run on zero queries; nothing of them is stored
@@ -224,10 +222,8 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
             // part[r]: key 8(r/4) + 4h + r%4 of the tile against row j
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-              const int a = r >> 2, b = r & 3;
-              const uint32_t w2 = (&sc.v[a][b >> 1].x)[2 * (b & 1) + (m >> 1)];   // halfwords 4b+m, 4b+m+1 pair
-              const _Float16 sh = as_h2(w2)[m & 1];
-              s[rt][r] = __builtin_fmaf(part[r], (float)sh, m == 0 ? 0.f : s[rt][r]);
+              const float sh = (&sc4[r >> 2].x)[r & 3];
+              s[rt][r] = m == 0 ? part[r] * sh : __builtin_fmaf(part[r], sh, s[rt][r]);
             }
           }
         }
@@ -272,8 +268,6 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
           l_run[rt] += lsum;
         }
       }
-      // scales of the next tile: requested now, needed after the next barrier
-      if (T + 1 < tile1) load_kscales(kv_page_uniform(A.kv, kvh, (T + 1) << 5), ((T + 1) << 5) % kPageTok, offs, sc);
       // ---- O^T += V^T P^T : d-tile dt (32 rows of the V image), k-step u (16 tokens) ----
 #pragma unroll
       for (int dt = 0; dt < 4; ++dt)
