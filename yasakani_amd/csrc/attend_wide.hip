@@ -28,6 +28,7 @@
 // Partial results leave through the same LDS after the last tile so that every store writes whole 256-byte rows.
 #include "yka_internal.h"
 #include <hip/hip_fp16.h>
+#include <type_traits>
 
 namespace yka {
 
@@ -51,7 +52,7 @@ struct Raw {                                   // one thread's share of a raw 32
   uint32_t kw[2];
   uint32_t vw[2];
   uint32_t vs;
-  uint32_t ks;                                 // threads 0..127: fp16 scale of (key tid/4, group tid%4)
+  uint32_t ks;                                 // fp16 scale of (key (tid & 127) / 4, group tid % 4)
 };
 
 // Byte offsets of one thread inside a page, fixed for the whole kernel; the page pointer and the tile's first token
@@ -61,16 +62,35 @@ __device__ __forceinline__ LaneOffs lane_offs(int tid, int h) {
   const uint32_t pair = tid >> 4, dw = tid & 15;
   (void)h;
   return LaneOffs{(uint32_t)tid * 4u, kPageVc + pair * 128u + dw * 4u, kPageVs + (dw >> 2) * (kPageTok * 2u) + pair * 4u,
-                  kPageKs + (uint32_t)tid * 2u};
+                  kPageKs + ((uint32_t)tid & 127u) * 2u};
+}
+// The tile loads are written as instructions: they stay in flight across two loop steps, and the counter wait the
+// compiler would place at the loop header (it merges the header's predecessors conservatively) drains all of them.
+// Every load here is "wave-uniform base in scalar registers + 32-bit lane offset"; wait_raw<N> ties the six registers
+// of a tile to a wait that leaves the N younger loads in flight.  Loads return in order and nothing stores in the loop.
+template <int IMM>
+__device__ __forceinline__ uint32_t gload32(const uint8_t* base, uint32_t off) {
+  uint32_t v;
+  asm volatile("global_load_dword %0, %1, %2 offset:%3" : "=v"(v) : "v"(off), "s"(base), "n"(IMM));
+  return v;
+}
+__device__ __forceinline__ uint32_t gload16(const uint8_t* base, uint32_t off) {
+  uint32_t v;
+  asm volatile("global_load_ushort %0, %1, %2" : "=v"(v) : "v"(off), "s"(base));
+  return v;
 }
 __device__ __forceinline__ void load_raw(const uint8_t* pg, int tp, const LaneOffs& L, Raw& R) {
   const uint8_t* kt = pg + (uint32_t)tp * 64u;            // K and V code rows of the tile start here (+ plane offset)
-  R.kw[0] = *reinterpret_cast<const uint32_t*>(kt + L.k);
-  R.kw[1] = *reinterpret_cast<const uint32_t*>(kt + L.k + NT * 4);
-  R.vw[0] = *reinterpret_cast<const uint32_t*>(kt + L.v);
-  R.vw[1] = *reinterpret_cast<const uint32_t*>(kt + L.v + 64);
-  R.vs = *reinterpret_cast<const uint32_t*>(pg + (uint32_t)tp * 2u + L.vs);
-  if (L.k < 128 * 4) R.ks = *reinterpret_cast<const uint16_t*>(pg + (uint32_t)tp * 8u + L.ks);   // waves 0 and 1 only
+  R.kw[0] = gload32<0>(kt, L.k);
+  R.kw[1] = gload32<NT * 4>(kt, L.k);
+  R.vw[0] = gload32<0>(kt, L.v);
+  R.vw[1] = gload32<64>(kt, L.v);
+  R.vs = gload32<0>(pg + (uint32_t)tp * 2u, L.vs);
+  R.ks = gload16(pg + (uint32_t)tp * 8u, L.ks);
+}
+template <int N>
+__device__ __forceinline__ void wait_raw(Raw& R) {
+  asm volatile("s_waitcnt vmcnt(%6)" : "+v"(R.kw[0]), "+v"(R.kw[1]), "+v"(R.vw[0]), "+v"(R.vw[1]), "+v"(R.vs), "+v"(R.ks) : "n"(N));
 }
 
 // (w & mask) | magic as one bit-field insert: `magic` (0x64006400, no bit inside either nibble mask) is kept opaque to
@@ -90,9 +110,9 @@ __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw&
     o.w = as_u32(as_h2(nib(t, 0x00f000f0u, magic)) - c1152);
     *reinterpret_cast<uint4*>(buf + kLdsK + key * kKPitch + (4 * (p & 3) + (p >> 2)) * 16) = o;
   }
-  if (tid < 128) {                                                   // K group scales as fp32, [group][a][h][b] for key 8a+4h+b
-    const int key = tid >> 2, m = tid & 3;
-    reinterpret_cast<float*>(buf + kLdsS)[m * 32 + (key >> 3) * 8 + (key & 7)] = (float)__builtin_bit_cast(_Float16, (uint16_t)R.ks);
+  {                                                                  // K group scales as fp32, [group][a][h][b] for key 8a+4h+b;
+    const int key = (tid & 127) >> 2, m = tid & 3;                   // waves 2 and 3 repeat waves 0 and 1 (no divergent branch)
+    reinterpret_cast<float*>(buf + kLdsS)[m * 32 + (key >> 3) * 8 + (key & 7)] = (float)as_h2(R.ks)[0];
   }
   {
     const int pair = tid >> 4, dw = tid & 15;
@@ -116,8 +136,7 @@ __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw&
 
 }  // namespace
 
-// grid (S, n_kv, ceil(6M / rows_per_block)), block 256; wave w owns rows [32 RT w, 32 RT (w+1)) of the block
-template <int RT>
+// grid (S, n_kv, ceil(6M / rows_per_block)), block 256; wave w owns rows [32 w, 32 (w+1)) of the block
 __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
   __shared__ __align__(16) uint8_t lds[2][kLdsBuf];
   const int split = blockIdx.x, kvh = blockIdx.y, rb = blockIdx.z;
@@ -125,30 +144,28 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
   const int pos = *A.d_pos;
   const int nrows = kG * A.M;
 
-  // rows of this wave: R = rb*128*RT + wave*32*RT + rt*32 + j  ->  token R/6 of the slice, head kvh*6 + R%6
+  // row of this lane: R = rb*rows_per_block + wave*32 + j  ->  token R/6 of the slice, head kvh*6 + R%6
   const int RPB = A.rows_per_block;
-  const int row0 = rb * RPB + wave * 32 * RT;
-  int len[RT]; bool vrow[RT]; size_t pidx[RT];
-  h8 qf[RT][8];
-#pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    const int R = row0 + rt * 32 + j;
-    vrow[rt] = R < nrows && R < (rb + 1) * RPB;
-    const int tl = R / kG, head = kvh * kG + R % kG;
-    len[rt] = 0;
-    if (vrow[rt]) { const int tg = A.tok0 + tl; len[rt] = min(pos + (A.depth ? (int)A.depth[tg] : tg) + 1, A.kv.max_ctx); }
-    pidx[rt] = ((size_t)tl * A.S + split) * A.n_heads + head;
-    // B operand of S^T = K Q^T, k-step ks: lane (row j, half h) holds chunk 2ks+h = (group ks/2, sub-chunk 2(ks&1)+h)
+  const int row0 = rb * RPB + wave * 32;
+  const int R = row0 + j;
+  const bool vrow = R < nrows && R < (rb + 1) * RPB;
+  const int tl = R / kG, head = kvh * kG + R % kG;
+  int len = 0;
+  if (vrow) { const int tg = A.tok0 + tl; len = min(pos + (A.depth ? (int)A.depth[tg] : tg) + 1, A.kv.max_ctx); }
+  const size_t pidx = ((size_t)tl * A.S + split) * A.n_heads + head;
+  // B operand of S^T = K Q^T, k-step ks: lane (row j, half h) holds chunk 2ks+h = (group ks/2, sub-chunk 2(ks&1)+h)
+  h8 qf[8];
+  {
     const uint16_t* qrow = A.q16 + ((size_t)tl * A.n_heads + head) * kD;
     const _Float16 sx = (_Float16)0.0625f;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      uint4 u = vrow[rt] ? *reinterpret_cast<const uint4*>(qrow + 32 * (ks >> 1) + 8 * (2 * (ks & 1) + h)) : make_uint4(0, 0, 0, 0);
+      uint4 u = vrow ? *reinterpret_cast<const uint4*>(qrow + 32 * (ks >> 1) + 8 * (2 * (ks & 1) + h)) : make_uint4(0, 0, 0, 0);
       const h8 c = __builtin_bit_cast(h8, u);
-      qf[rt][ks] = h8{c[0], c[4], c[1] * sx, c[5] * sx, c[2], c[6], c[3] * sx, c[7] * sx};
+      qf[ks] = h8{c[0], c[4], c[1] * sx, c[5] * sx, c[2], c[6], c[3] * sx, c[7] * sx};
     }
   }
-  const int nrt = min(RT, max(0, (min(nrows, (rb + 1) * RPB) - row0 + 31) / 32));         // row tiles of this wave that hold rows (wave uniform)
+  const bool has_rows = row0 < min(nrows, (rb + 1) * RPB);             // wave uniform
 
   // key range of the workgroup: its splits cut [0, maxlen) of the block's longest row into 32-key tiles
   const int tok_lo = (rb * RPB) / kG, tok_hi = min(A.M, (rb * RPB + RPB + kG - 1) / kG);
@@ -159,173 +176,160 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
   const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
 
   const float sc_log2 = kLog2e / sqrtf((float)kD);
-  float m_run[RT], l_run[RT];                  // m_run in log2 units, shared by the two lanes of a row
-  f16v o[RT][4];
+  float m_run = -1e30f, l_run = 0.f;           // m_run in log2 units, shared by the two lanes of a row
+  f16v o[4];
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    m_run[rt] = -1e30f; l_run[rt] = 0.f;
+  for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o[rt][dt][r] = 0.f;
-  }
+    for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
 
-  Raw raw0, raw1;                              // raw codes of the next two tiles: loads run two tiles ahead of their use
+  Raw raw0{}, raw1{};                          // raw codes of the next two tiles: loads run two tiles ahead of their use
   const LaneOffs offs = lane_offs(tid, h);
   uint32_t magic = kMagic;
   asm volatile("" : "+v"(magic));
-  auto load_tile_raw = [&](int T, Raw& r) { load_raw(kv_page_uniform(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, r); };
+  auto load_tile_raw = [&](int T, Raw& r) __attribute__((always_inline)) { load_raw(kv_page_uniform(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, r); };
   if (tile0 < tile1) {
     load_tile_raw(tile0, raw0);
+    wait_raw<0>(raw0);
     dequant_to_lds(lds[0], tid, raw0, magic);
-    if (tile0 + 1 < tile1) load_tile_raw(tile0 + 1, raw1);
-    if (tile0 + 2 < tile1) load_tile_raw(tile0 + 2, raw0);
+    load_tile_raw(min(tile0 + 1, tile1 - 1), raw1);
+    load_tile_raw(min(tile0 + 2, tile1 - 1), raw0);
   }
   __syncthreads();
-  // One tile: `rs` holds the raw codes of tile T+1, which are dequantized into the other LDS buffer and replaced by the
-  // request for tile T+3; cb (the LDS buffer of tile T) is a literal at both call sites.
-  auto tile_step = [&](const int T, const int cb, Raw& rs) {
-    // all K fragments of tile T are requested before anything else, so that their LDS latency runs under the
-    // dequantization of tile T+1
+
+  // The loop is software pipelined inside the wave: the probabilities and the V fragments of a tile stay in registers
+  // across the barrier, and their eight MFMAs are issued at the start of the NEXT step, next to the dequantization of
+  // the tile after that - matrix and vector work with no dependence on each other in one basic block.  The first step
+  // multiplies zeros; the product of the last tile is issued after the loop.
+  h8 pf[2], vfr[8];
+#pragma unroll
+  for (int c = 0; c < 8; ++c)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) { vfr[c][e] = (_Float16)0.f; pf[c & 1][e] = (_Float16)0.f; }
+  auto pv = [&]() __attribute__((always_inline)) {                            // O^T += V^T P^T : d-tile dt (32 rows of the V image), k-step u (16 tokens)
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vfr[2 * dt + u], pf[u], o[dt], 0, 0, 0);
+  };
+  // One tile: `rs` holds the raw codes of tile T+1, which are dequantized into the other LDS buffer (unconditionally:
+  // after the last tile that buffer is read by nobody) and replaced by the request for tile T+3; cb, the LDS buffer of
+  // tile T, is a literal at both call sites.  kCompute is false for a wave whose rows all lie past the window.
+  auto tile_step = [&](auto compute_tag, const int T, const int cb, Raw& rs) __attribute__((always_inline)) {
+    constexpr bool kCompute = decltype(compute_tag)::value;
+    const uint8_t* buf = lds[cb];
     h8 kfr[8];
-    if (nrt > 0) {
+    if constexpr (kCompute) {
 #pragma unroll
       for (int c = 0; c < 8; ++c)
-        kfr[c] = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(lds[cb] + kLdsK + j * kKPitch + (4 * (c >> 1) + 2 * (c & 1) + h) * 16));
+        kfr[c] = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsK + j * kKPitch + (4 * (c >> 1) + 2 * (c & 1) + h) * 16));
+      pv();
     }
-    if (T + 1 < tile1) {
-      dequant_to_lds(lds[cb ^ 1], tid, rs, magic);
-      if (T + 3 < tile1) load_tile_raw(T + 3, rs);
-    }
-    const uint8_t* buf = lds[cb];
-    const int t0 = T << 5;
-    const bool need_mask = t0 + 32 > minlen;
-    if (nrt > 0) {
-      h8 pf[RT][2];
-      // ---- scores: per scale group two chained MFMAs (32 channels), then the fp32 sum times the group scale; one
-      //      K fragment read feeds every row tile of the wave ----
-      float s[RT][16];
+    wait_raw<6>(rs);                           // the six loads of the other register set stay in flight
+    dequant_to_lds(lds[cb ^ 1], tid, rs, magic);
+    load_tile_raw(min(T + 3, tile1 - 1), rs);  // always issued (past the end: the last tile again), so that the count of loads in flight is static
+    if constexpr (kCompute) {
+      const int t0 = T << 5;
+      // ---- scores: per scale group two chained MFMAs (32 channels), then the fp32 sum times the group scale ----
+      float s[16];
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
-        const h8 k0 = kfr[2 * m], k1 = kfr[2 * m + 1];
         float4 sc4[4];                         // fp32 scales of group m for the lane's 16 keys, the same for all 32 lanes of a half
 #pragma unroll
         for (int a = 0; a < 4; ++a) sc4[a] = *reinterpret_cast<const float4*>(buf + kLdsS + ((m * 4 + a) * 2 + h) * 16);
+        f16v part;
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) {
-          {                                    // row tiles past the wave's last row run on zero queries; nothing of them is stored
-            f16v part;
+        for (int r = 0; r < 16; ++r) part[r] = 0.f;
+        part = __builtin_amdgcn_mfma_f32_32x32x16_f16(kfr[2 * m], qf[2 * m], part, 0, 0, 0);
+        part = __builtin_amdgcn_mfma_f32_32x32x16_f16(kfr[2 * m + 1], qf[2 * m + 1], part, 0, 0, 0);
+        // part[r]: key 8(r/4) + 4h + r%4 of the tile against row j
 #pragma unroll
-            for (int r = 0; r < 16; ++r) part[r] = 0.f;
-            part = __builtin_amdgcn_mfma_f32_32x32x16_f16(k0, qf[rt][2 * m], part, 0, 0, 0);
-            part = __builtin_amdgcn_mfma_f32_32x32x16_f16(k1, qf[rt][2 * m + 1], part, 0, 0, 0);
-            // part[r]: key 8(r/4) + 4h + r%4 of the tile against row j
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const float sh = (&sc4[r >> 2].x)[r & 3];
-              s[rt][r] = m == 0 ? part[r] * sh : __builtin_fmaf(part[r], sh, s[rt][r]);
-            }
-          }
+        for (int r = 0; r < 16; ++r) {
+          const float sh = (&sc4[r >> 2].x)[r & 3];
+          s[r] = m == 0 ? part[r] * sh : __builtin_fmaf(part[r], sh, s[r]);
         }
       }
-      // all V fragments are requested here: their LDS latency runs under the softmax arithmetic
-      h8 vfr[8];
+      // the V fragments are requested here and used after the barrier: their LDS latency runs under the softmax arithmetic
 #pragma unroll
       for (int c = 0; c < 8; ++c)
         vfr[c] = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsV + (32 * (c >> 1) + j) * kVPitch + (16 * (c & 1) + 8 * h) * 2));
+      // ---- online softmax with a lazily raised maximum.  s stays in raw units; the factor log2(e)/sqrt(d) is
+      //      folded into the exponent's fused multiply-add: p = 2^(s * sc_log2 - m_run) ----
+      if (t0 + 32 > minlen) {
 #pragma unroll
-      for (int rt = 0; rt < RT; ++rt) {
-        {
-          // ---- online softmax with a lazily raised maximum.  s stays in raw units; the factor log2(e)/sqrt(d) is
-          //      folded into the exponent's fused multiply-add: p = 2^(s * sc_log2 - m_run) ----
-          float tmax = -INFINITY;
-          if (need_mask) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int key = t0 + 8 * (r >> 2) + 4 * h + (r & 3);
-              s[rt][r] = key < len[rt] ? s[rt][r] : -INFINITY;
-            }
-          }
-#pragma unroll
-          for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[rt][r]);
-          tmax *= sc_log2;
-          if (__any(tmax > m_run[rt] + kRaise)) {
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-            const float m_new = fmaxf(m_run[rt], tmax);
-            const float alpha = __builtin_amdgcn_exp2f(m_run[rt] - m_new);
-            m_run[rt] = m_new; l_run[rt] *= alpha;
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-              for (int r = 0; r < 16; ++r) o[rt][dt][r] *= alpha;
-          }
-          float lsum = 0.f;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[rt][r], sc_log2, -m_run[rt]));
-            lsum += p; pf[rt][r >> 3][r & 7] = (_Float16)p;
-          }
-          l_run[rt] += lsum;
+        for (int r = 0; r < 16; ++r) {
+          const int key = t0 + 8 * (r >> 2) + 4 * h + (r & 3);
+          s[r] = key < len ? s[r] : -INFINITY;
         }
       }
-      // ---- O^T += V^T P^T : d-tile dt (32 rows of the V image), k-step u (16 tokens) ----
+      float tmax = -INFINITY;
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
+      for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[r]);
+      tmax *= sc_log2;
+      if (__any(tmax > m_run + kRaise)) {
+        tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+        const float m_new = fmaxf(m_run, tmax);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        m_run = m_new; l_run *= alpha;
 #pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          const h8 vf = vfr[2 * dt + u];
+        for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-          for (int rt = 0; rt < RT; ++rt)
-            o[rt][dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf, pf[rt][u], o[rt][dt], 0, 0, 0);
-        }
+          for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+      }
+      float lsum = 0.f;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], sc_log2, -m_run));
+        lsum += p; pf[r >> 3][r & 7] = (_Float16)p;
+      }
+      l_run += lsum;
     }
     __syncthreads();
   };
-  for (int T = tile0; T < tile1; T += 2) {
-    tile_step(T, 0, raw1);
-    if (T + 1 < tile1) tile_step(T + 1, 1, raw0);
-  }
+  auto run = [&](auto compute_tag) __attribute__((always_inline)) {
+    for (int T = tile0; T < tile1; T += 2) {
+      tile_step(compute_tag, T, 0, raw1);
+      if (T + 1 < tile1) tile_step(compute_tag, T + 1, 1, raw0);
+    }
+  };
+  if (has_rows) { run(std::true_type{}); pv(); } else run(std::false_type{});
+  if (!has_rows) return;                       // no barrier follows
   // ---- partials: normalised fp16.  o[dt][4a+b] of lane (row j, half h) is V-image row 32dt + 8a + 4h + b, i.e.
   //      channel 64(a&1) + 32h + 8b + 4(a>>1) + dt: for each (a&1, b) the lane owns 8 consecutive channels.
   //      Rows go through LDS (the tile buffers are free after the last barrier) so that every store instruction
   //      writes whole 256-byte rows: 16 lanes per row instead of 64 scattered 16-byte pieces. ----
   constexpr int kOPitch = 2 * kD + 16;                       // bytes per staged row
-  uint8_t* stage = &lds[0][0] + wave * 32 * kOPitch;         // 4 waves x 8704 bytes, reused for every row tile
+  uint8_t* stage = &lds[0][0] + wave * 32 * kOPitch;         // 4 waves x 8704 bytes
+  float l = l_run;
+  l += __shfl_xor(l, 32, 64);
+  if (vrow && h == 0) { A.pm[pidx] = m_run; A.pl[pidx] = l; }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt) {
-    if (rt >= nrt) break;
-    float l = l_run[rt];
-    l += __shfl_xor(l, 32, 64);
-    if (vrow[rt] && h == 0) { A.pm[pidx[rt]] = m_run[rt]; A.pl[pidx[rt]] = l; }
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+  for (int a0 = 0; a0 < 2; ++a0)
 #pragma unroll
-    for (int a0 = 0; a0 < 2; ++a0)
+    for (int b = 0; b < 4; ++b) {
+      h8 v;
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        h8 v;
-#pragma unroll
-        for (int c = 0; c < 8; ++c) v[c] = (_Float16)(o[rt][c & 3][4 * (2 * (c >> 2) + a0) + b] * inv);
-        *reinterpret_cast<uint4*>(stage + j * kOPitch + (64 * a0 + 32 * h + 8 * b) * 2) = __builtin_bit_cast(uint4, v);
-      }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // the wave reads back what its own lanes wrote
-    const int chunk = lane & 15;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      const int jr = 4 * k + (lane >> 4);
-      const int R = row0 + rt * 32 + jr;
-      if (R < nrows && R < (rb + 1) * RPB) {
-        const size_t p = ((size_t)(R / kG) * A.S + split) * A.n_heads + kvh * kG + R % kG;
-        const uint4 v = *reinterpret_cast<const uint4*>(stage + jr * kOPitch + chunk * 16);
-        *reinterpret_cast<uint4*>(A.pacc16 + p * kD + chunk * 8) = v;
-      }
+      for (int c = 0; c < 8; ++c) v[c] = (_Float16)(o[c & 3][4 * (2 * (c >> 2) + a0) + b] * inv);
+      *reinterpret_cast<uint4*>(stage + j * kOPitch + (64 * a0 + 32 * h + 8 * b) * 2) = __builtin_bit_cast(uint4, v);
     }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");   // reads done before the next row tile overwrites the stage
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");     // the wave reads back what its own lanes wrote
+  const int chunk = lane & 15;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int jr = 4 * k + (lane >> 4);
+    const int Rr = row0 + jr;
+    if (Rr < nrows && Rr < (rb + 1) * RPB) {
+      const size_t p = ((size_t)(Rr / kG) * A.S + split) * A.n_heads + kvh * kG + Rr % kG;
+      const uint4 v = *reinterpret_cast<const uint4*>(stage + jr * kOPitch + chunk * 16);
+      *reinterpret_cast<uint4*>(A.pacc16 + p * kD + chunk * 8) = v;
+    }
   }
 }
 
 void launch_attend_wide(const AttnArgs& A, hipStream_t st) {
   const int rows = kG * A.M, rb = (rows + A.rows_per_block - 1) / A.rows_per_block;
-  hipLaunchKernelGGL(attend_wide_kernel<1>, dim3(A.S, A.kv.n_kv, rb), dim3(NT), 0, st, A);
+  hipLaunchKernelGGL(attend_wide_kernel, dim3(A.S, A.kv.n_kv, rb), dim3(NT), 0, st, A);
 }
 
 }  // namespace yka
