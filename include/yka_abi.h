@@ -58,7 +58,11 @@ YKA_API const char* yka_build_info(void);
  * key 3: 1 forces the narrow kernel for every width (cross-check of the wide kernel), 0 = automatic;
  * key 4: 1 = attention outputs get the inverse signed Hadamard rotation before they are rounded to fp16 (for caches
  *        filled by yka_attn_post or yka_append256_f32 with rotate = 1; the reference un-rotates in its output step,
- *        q35_kernels.cu:1421). */
+ *        q35_kernels.cu:1421);
+ * key 5: context length (tokens) the caller expects, used only to size the decode grid (the reference picks its split
+ *        count from the length known on the host, engine35.hpp:434-439); 0 = the max_ctx of the handle.  Any actual
+ *        position stays correct: positions are read on the device and the kernel uses as many of the launched
+ *        splits as the length it finds there justifies. */
 YKA_API int yka_set_opt(yka_kv* kv, int key, int value);
 
 /* Paged mode: logical page p of `layer` (-1 = every layer) lives in physical page h_table[p]; n_pages = max_ctx/256

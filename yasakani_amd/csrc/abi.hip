@@ -30,7 +30,7 @@ struct yka_kv {
   size_t ws_rows = 0;              // capacity of the partial workspace in (token, split) pairs
   int* d_pos = nullptr;            // position used by the host-pointer hooks
   hipStream_t stream = nullptr;    // stream of the host-pointer hooks
-  int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0, opt_unrot = 0;
+  int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0, opt_unrot = 0, opt_ctx_hint = 0;
   bool r256() const { return cfg.head_dim == 256; }   // the reference's own rows (attend256.hip); otherwise the 128-channel format
   int D() const { return cfg.head_dim; }
   KvView view(int layer) const {
@@ -57,11 +57,15 @@ void on_device(const yka_kv* kv) {
 constexpr int kMaxSplits = 256;
 constexpr size_t kWsPairs = 4096;  // (token, split) pairs the partial workspace holds: 4096 * 24 * (256 + 8) bytes = 26 MB
 
-// splits for the narrow kernel: enough workgroups (n_kv * S * ceil(M/2)) to put 4 waves on every SIMD of 256 CUs
+// splits for the narrow kernel: enough workgroups (n_kv * S * ceil(M/2)) to put 2 waves on every SIMD of 256 CUs (the
+// kernel itself uses fewer of them on short contexts)
 int narrow_splits(const yka_kv* kv, int M) {
   if (kv->opt_splits_narrow > 0) return std::min(kv->opt_splits_narrow, (int)(kWsPairs / (size_t)M));
   const int tiles = (M + 1) / 2;
-  int S = 1024 / (kv->cfg.n_kv_heads * tiles);
+  // launching a split costs more than letting it exit: the grid is sized for the context the caller expects (option
+  // key 5; by default the capacity of the handle), two 32-key tiles per workgroup at least
+  const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
+  int S = std::min(512 / (kv->cfg.n_kv_heads * tiles), ((ctx + 31) / 32) / 2);
   S = std::max(2, std::min(kMaxSplits, S));
   return std::min(S, (int)(kWsPairs / (size_t)M));
 }
@@ -220,6 +224,7 @@ int yka_set_opt(yka_kv* kv, int key, int value) {
     case 2: if (value < 0 || value > kMaxSplits) throw std::runtime_error("splits must be in [0, 256]"); kv->opt_splits_wide = value; break;
     case 3: kv->opt_force_narrow = value != 0; break;
     case 4: kv->opt_unrot = value != 0; break;
+    case 5: if (value < 0) throw std::runtime_error("context hint must be >= 0"); kv->opt_ctx_hint = value; break;
     default: throw std::runtime_error("unknown option key");
   }
   YKA_CATCH_INT

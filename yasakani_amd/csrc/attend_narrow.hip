@@ -131,7 +131,20 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
 #pragma unroll
   for (int o = 1; o < 16; o <<= 1) { maxlen = max(maxlen, __shfl_xor(maxlen, o, 64)); minlen = min(minlen, __shfl_xor(minlen, o, 64)); }
   maxlen = __builtin_amdgcn_readfirstlane(maxlen); minlen = __builtin_amdgcn_readfirstlane(minlen);
-  const int ntiles = (maxlen + 31) >> 5, tps = (ntiles + A.S - 1) / A.S;
+  // The grid is sized for long contexts; how many of its splits a row tile uses follows from the length it finds on the
+  // device: at least two 32-key tiles per workgroup.  The other workgroups leave the "no keys" marker and exit, and
+  // the combiner does not read their rows.
+  const int ntiles = (maxlen + 31) >> 5;
+  const int s_used = min(A.S, max(1, ntiles >> 1));
+  if (split >= s_used) {
+    const int j = threadIdx.x, tj = TPT * rt + j / kG;
+    if (j < TPT * kG && tj < A.M) {
+      const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
+      A.pm[p] = -1e30f; A.pl[p] = 0.f;
+    }
+    return;
+  }
+  const int tps = (ntiles + s_used - 1) / s_used;
   const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
 
   // ---- fused quantize-on-append (decode, M <= 2, one row tile): a row of this pass is written by the one workgroup
@@ -317,7 +330,8 @@ __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
     for (int k = 0; k < kInFlight; ++k) {
       const int sp = s0 + 16 * k;
       w[k] = sp < A.S ? s_w[sp] : 0.f;
-      u[k] = sp < A.S ? *reinterpret_cast<const uint4*>(src + (size_t)sp * stride) : make_uint4(0, 0, 0, 0);
+      // rows of weight 0 are not read: a split that was not used leaves its row unwritten
+      u[k] = (sp < A.S && w[k] != 0.f) ? *reinterpret_cast<const uint4*>(src + (size_t)sp * stride) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int k = 0; k < kInFlight; ++k) {
