@@ -75,7 +75,10 @@ int narrow_splits(const yka_kv* kv, int M) {
 int wide_rows_per_block(int) { return 128; }
 int wide_splits(const yka_kv* kv, int M) {
   const int rows = kG * M, rpb = wide_rows_per_block(M), rb = (rows + rpb - 1) / rpb;
-  int S = kv->opt_splits_wide > 0 ? kv->opt_splits_wide : 512 / (kv->cfg.n_kv_heads * rb);
+  // about two workgroups per CU, and (sized like the decode grid, by the expected context) at least 2 * rb 32-key
+  // tiles per workgroup: measured best at 4k context for 16 and 64 rows, no change at 32k
+  const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
+  int S = kv->opt_splits_wide > 0 ? kv->opt_splits_wide : std::min(512 / (kv->cfg.n_kv_heads * rb), ((ctx + 31) / 32) / (2 * rb));
   S = std::max(1, std::min(kMaxSplits, S));
   return std::min(S, std::max(1, (int)kWsPairs / M));
 }
