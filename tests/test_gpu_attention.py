@@ -41,7 +41,8 @@ def test_window_matches_oracle(native, oracle, M):
         assert_attn_close(out, ref32, f"window M={M}")
         # appended rows are in the cache, bit-exact
         got = kv.export_rows(0, ctx, M)
-        assert (got[0] == oc.kc[:, ctx:ctx + M]).all() and (got[3] == oc.vs[:, ctx:ctx + M]).all()
+        assert (got[0] == oc.kc[:, ctx:ctx + M]).all() and (got[1] == oc.ks[:, ctx:ctx + M]).all()
+        assert (got[2] == oc.vc[:, ctx:ctx + M]).all() and (got[3] == oc.vs[:, ctx:ctx + M]).all()
 
 
 def test_window_equals_single_row_calls(native, oracle):
@@ -133,6 +134,10 @@ def test_wide_pass_is_cut_into_slices(native, oracle):
         out = kv.layer_call(0, q, kn, vn, ctx)
         oc.append(kn, vn, ctx)
         assert_attn_close(out, oc.attend_f32(q, ctx, threads=8, want_f32=True)[1], "150-row pass")
+        # every slice stored its own rows (quantize-on-append rides in the attention launches), bit-exact
+        got = kv.export_rows(0, ctx, M)
+        for a, b in zip(got, (oc.kc, oc.ks, oc.vc, oc.vs)):
+            assert (a == b[:, ctx:ctx + M]).all()
 
 
 def test_errors_are_reported_not_thrown(native):

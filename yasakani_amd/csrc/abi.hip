@@ -116,7 +116,10 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
     }
     return;
   }
-  const bool fuse_append = k16 && M <= 2;
+  // quantize-on-append rides in the attention launch: in the decode kernel for rows of at most 2 tokens, in the wide
+  // kernel for every 64-row slice (each slice stores its own rows); only a wide pass forced through the narrow kernel
+  // launches the append kernel first
+  const bool fuse_append = k16 && (M <= 2 || !kv->opt_force_narrow);
   if (k16 && !fuse_append) do_append(kv, layer, k16, v16, M, d_pos, st);
   for (int s0 = 0; s0 < M; s0 += kMaxSlice) {   // 64-row slices, as attn_block cuts wide passes (engine35.cpp:935-947)
     const int Ms = std::min(kMaxSlice, M - s0);

@@ -154,11 +154,11 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
   if (!MS && A.k16) {
     bool mine = false;
     for (int t = 0; t < A.M; ++t) {
-      const int r = pos + t;
+      const int r = pos + A.tok0 + t;              // k16/v16 point at row 0 of the pass, this slice starts at row tok0
       if (r < 0 || r >= A.kv.max_ctx || (r >> 5) < tile0 || (r >> 5) >= tile1) continue;
       mine = true;
       const bool isv = threadIdx.x >= 128;
-      const uint16_t* src = (isv ? A.v16 : A.k16) + ((size_t)t * A.kv.n_kv + kvh) * kD;
+      const uint16_t* src = (isv ? A.v16 : A.k16) + ((size_t)(A.tok0 + t) * A.kv.n_kv + kvh) * kD;
       quant_store_row(A.kv, kvh, r, isv, src, threadIdx.x & 127);
     }
     if (mine) {                      // uniform over the workgroup

@@ -26,7 +26,7 @@
 //                          the same for all 32 lanes of a wave half; converted to fp32 once per workgroup, each lane reads
 //                          four of them per instruction (a broadcast read) and multiplies with a plain fp32 FMA
 // Partial results leave through the same LDS after the last tile so that every store writes whole 256-byte rows.
-#include "yka_internal.h"
+#include "codec_device.h"
 #include <hip/hip_fp16.h>
 #include <type_traits>
 
@@ -172,8 +172,41 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
   int maxdep = 0, mindep = 0x7fffffff;
   for (int t = tok_lo; t < tok_hi; ++t) { const int tg = A.tok0 + t; const int dp = A.depth ? (int)A.depth[tg] : tg; maxdep = max(maxdep, dp); mindep = min(mindep, dp); }
   const int maxlen = min(pos + maxdep + 1, A.kv.max_ctx), minlen = min(pos + mindep + 1, A.kv.max_ctx);
-  const int ntiles = (maxlen + 31) >> 5, tps = (ntiles + A.S - 1) / A.S;
-  const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
+  // The last split owns the tiles that hold rows of this slice (from tile Tw on), the other splits share the cached
+  // context before them evenly: the rows a pass appends are then read by the workgroups of one split only, which
+  // is what lets them be quantized and stored by those workgroups themselves (below) instead of by a launch of
+  // their own.  The window split has a handful of tiles, so the quantization is off the critical path.
+  const int ntiles = (maxlen + 31) >> 5;
+  const int Tw = min(ntiles, max(0, pos + A.tok0) >> 5);
+  int tile0, tile1;
+  if (A.S == 1) { tile0 = 0; tile1 = ntiles; }
+  else if (split == A.S - 1) { tile0 = Tw; tile1 = ntiles; }
+  else { const int tps = (Tw + A.S - 2) / (A.S - 1); tile0 = split * tps; tile1 = min(Tw, tile0 + tps); }
+  // ---- fused quantize-on-append: every workgroup of the window split stores the slice's rows up to its own last
+  //      token (the row blocks of one kv head write identical bytes) and reads them back after a workgroup barrier:
+  //      writer and readers are waves of one CU and one write-through L1 ----
+  if (A.k16 && split == A.S - 1) {
+    // 16 lanes per 128-channel row, 16 rows (K and V of 8 tokens) per step; all loads of the slice (at most 64 tokens)
+    // are requested before the first row is quantized
+    static_assert(kMaxSlice <= 64, "8 steps of 16 rows cover K and V of a slice");
+    const int c = tid & 15, slot = tid >> 4;
+    uint4 rawv[8];
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int hh = it * 16 + slot, t = hh >> 1;
+      const uint16_t* src = ((hh & 1) ? A.v16 : A.k16) + ((size_t)(A.tok0 + t) * A.kv.n_kv + kvh) * kD + 8 * c;
+      rawv[it] = t < tok_hi ? *reinterpret_cast<const uint4*>(src) : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int it = 0; it < 8; ++it) {
+      const int hh = it * 16 + slot, t = hh >> 1, r = pos + A.tok0 + t;
+      if (t < tok_hi && r >= 0 && r < A.kv.max_ctx) quant_store_chunk8(A.kv, kvh, r, hh & 1, rawv[it], c);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    asm volatile("" ::: "memory");             // the tile loads below are instructions the compiler does not see as loads
+  }
 
   const float sc_log2 = kLog2e / sqrtf((float)kD);
   float m_run = -1e30f, l_run = 0.f;           // m_run in log2 units, shared by the two lanes of a row

@@ -52,4 +52,38 @@ __device__ __forceinline__ void quant_store_value(const KvView& kv, int kvh, int
   }
 }
 
+// The same quantizer with 16 lanes per row: lane c (0..15, four consecutive lanes = one scale group) owns channels
+// 8c .. 8c+7, given as 8 fp16 in `raw`.  Bit-identical to quant_store_value: the group maximum is exact in any order,
+// everything after it is the same sequence of IEEE operations per channel.  Must be called by all 16 lanes of a row.
+__device__ __forceinline__ void quant_store_chunk8(const KvView& kv, int kvh, int pos, bool isv, uint4 raw, int c) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  float x[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) x[e] = h2f_bits((uint16_t)(w[e >> 1] >> (16 * (e & 1))));
+  float am = fabsf(x[0]);
+#pragma unroll
+  for (int e = 1; e < 8; ++e) am = fmaxf(am, fabsf(x[e]));
+  am = fmaxf(am, __shfl_xor(am, 1, 64));
+  am = fmaxf(am, __shfl_xor(am, 2, 64));
+  const float s32 = __fdiv_rn(am, 7.0f);
+  uint16_t s16 = __half_as_ushort(__float2half_rn(s32));
+  if ((s16 & 0x7fffu) == 0) s16 = 0x3c00u;
+  const float sd = h2f_bits(s16);
+  uint32_t word = 0;                           // channel 8c+e in bits [4e, 4e+4): even channel = low nibble of its byte
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float q = rintf(__fdiv_rn(x[e], sd));
+    q = fminf(fmaxf(q, -7.f), 7.f);
+    word |= (uint32_t)((int)q + 8) << (4 * e);
+  }
+  uint8_t* pg = kv_page(kv, kvh, pos);
+  const int tp = pos % kPageTok, g = c >> 2;
+  if (isv) *reinterpret_cast<uint32_t*>(pg + kPageVc + tp * 64 + 4 * c) = word;
+  else *reinterpret_cast<uint32_t*>(pg + kPageKc + tp * 64 + 4 * k_phys_dword(c)) = word;
+  if ((c & 3) == 0) {
+    if (isv) reinterpret_cast<uint16_t*>(pg + kPageVs)[g * kPageTok + tp] = s16;
+    else reinterpret_cast<uint16_t*>(pg + kPageKs)[tp * kNG + g] = s16;
+  }
+}
+
 }  // namespace yka

@@ -60,8 +60,9 @@ struct AttnArgs {
   int S;        // splits
   int rows_per_block;  // wide kernel: query rows one workgroup owns (multiple of 32)
   float* pm; float* pl; uint16_t* pacc16;
-  // narrow kernel only.  k16/v16 != nullptr (M <= 2): the workgroup whose tiles hold a new row quantizes and stores it
-  // before reading it (fused quantize-on-append).
+  // k16/v16 != nullptr: fused quantize-on-append - the workgroups whose tiles hold the new rows quantize and store them
+  // before reading them.  Narrow kernel (M <= 2): rows [0, M) of the pass; wide kernel: k16/v16 point at row 0 of the
+  // pass and the slice stores its own rows tok0 .. tok0 + M - 1.
   const uint16_t* k16; const uint16_t* v16;
   RowMap rows;  // narrow kernel only: multi-stream pass, one token per workgroup column, no depth table, no fused append
 };
