@@ -102,7 +102,7 @@ __device__ __forceinline__ void load_tile(const uint8_t* pg, int tp, const LaneO
 template <bool MS>
 __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
   __shared__ float s_m[4][16], s_l[4][16];
-  __shared__ float s_acc[4][16][kD + 4];
+  __shared__ __align__(16) float s_acc[4][16][kD + 4];
   constexpr int TPT = MS ? 1 : 2;
   const int split = blockIdx.x, kvh = blockIdx.y, rt = blockIdx.z;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // a scalar: tile indices and page pointers are wave uniform
@@ -275,18 +275,29 @@ __global__ void __launch_bounds__(256, 4) attend_narrow_kernel(AttnArgs A) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) s_acc[wave][i][8 * (4 * g + r) + b] = o[b][r];
   __syncthreads();
-  for (int idx = threadIdx.x; idx < TPT * kG * kD; idx += 256) {
-    const int j = idx >> 7, d = idx & (kD - 1);
+  // 16 lanes per row, 8 channels each: one 16-byte store per lane
+  if (threadIdx.x < TPT * kG * 16) {
+    const int j = threadIdx.x >> 4, c8 = (threadIdx.x & 15) * 8;
     const int tj = TPT * rt + j / kG;
-    if (tj >= A.M) continue;
-    const float m0 = s_m[0][j], m1 = s_m[1][j], m2 = s_m[2][j], m3 = s_m[3][j];
-    const float M2 = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
-    const float w0 = exp2f(m0 - M2), w1 = exp2f(m1 - M2), w2 = exp2f(m2 - M2), w3 = exp2f(m3 - M2);
-    const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
-    const float L = w0 * s_l[0][j] + w1 * s_l[1][j] + w2 * s_l[2][j] + w3 * s_l[3][j];
-    const float acc = w0 * s_acc[0][j][d] + w1 * s_acc[1][j][d] + w2 * s_acc[2][j][d] + w3 * s_acc[3][j][d];
-    A.pacc16[p * kD + d] = __half_as_ushort(__float2half_rn(L > 0.f ? acc / L : 0.f));
-    if (d == 0) { A.pm[p] = M2; A.pl[p] = L; }
+    if (tj < A.M) {
+      const float m0 = s_m[0][j], m1 = s_m[1][j], m2 = s_m[2][j], m3 = s_m[3][j];
+      const float M2 = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
+      const float w[4] = {exp2f(m0 - M2), exp2f(m1 - M2), exp2f(m2 - M2), exp2f(m3 - M2)};
+      const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
+      const float L = w[0] * s_l[0][j] + w[1] * s_l[1][j] + w[2] * s_l[2][j] + w[3] * s_l[3][j];
+      float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int wv = 0; wv < 4; ++wv) {
+        const float4 a0 = *reinterpret_cast<const float4*>(&s_acc[wv][j][c8]), a1 = *reinterpret_cast<const float4*>(&s_acc[wv][j][c8 + 4]);
+        acc[0] += w[wv] * a0.x; acc[1] += w[wv] * a0.y; acc[2] += w[wv] * a0.z; acc[3] += w[wv] * a0.w;
+        acc[4] += w[wv] * a1.x; acc[5] += w[wv] * a1.y; acc[6] += w[wv] * a1.z; acc[7] += w[wv] * a1.w;
+      }
+      h8 v;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) v[e] = (_Float16)(L > 0.f ? acc[e] / L : 0.f);
+      *reinterpret_cast<uint4*>(A.pacc16 + p * kD + c8) = __builtin_bit_cast(uint4, v);
+      if (c8 == 0) { A.pm[p] = M2; A.pl[p] = L; }
+    }
   }
 }
 
