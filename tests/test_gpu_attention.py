@@ -168,3 +168,79 @@ def test_bench_hook_runs_and_agrees_with_single_call(native, oracle):
             ms, out = kv.bench(q, kn, vn, ctx, mode=0, use_graph=graph, reps=3)
             assert (ms > 0).all()
             assert (out.view(np.uint16) == one.view(np.uint16)).all()
+
+
+def _rows_equal(kv, oc, ctx, M):
+    got = kv.export_rows(0, ctx, M)
+    for a, b in zip(got, (oc.kc, oc.ks, oc.vc, oc.vs)):
+        assert (a == b[:, ctx:ctx + M]).all()
+
+
+@pytest.mark.parametrize("ctx,M", [(0, 64), (0, 3), (5, 33), (31, 64), (32, 16), (250, 64), (4000, 64)])
+def test_wide_window_on_short_contexts_stores_its_rows(native, oracle, ctx, M):
+    # the window's rows are quantized inside the attention launch by the split that owns their tiles; with few or no
+    # cached tokens that split is the only one with keys
+    kv, oc, q, kn, vn = _fill(native, oracle, 600 + ctx + M, ctx, M)
+    with kv:
+        out = kv.layer_call(0, q, kn, vn, ctx)
+        oc.append(kn, vn, ctx)
+        assert_attn_close(out, oc.attend_f32(q, ctx, threads=8, want_f32=True)[1], f"ctx={ctx} M={M}")
+        _rows_equal(kv, oc, ctx, M)
+
+
+def test_fused_append_equals_separate_append(native, oracle):
+    # yka_append + yka_attend against yka_append_attend: same cache rows, same outputs bit for bit (one split geometry)
+    ctx, M = 1234, 40
+    q, k, v, kn, vn, ch = oracle.make_inputs(610, ctx, M)
+    oc = oracle.Cache(1536); oc.append(k, v, 0)
+    outs = []
+    for fused in (True, False):
+        with native.KvCache(max_ctx=1536) as kv:
+            kv.import_rows(0, 0, oc.kc[:, :ctx], oc.ks[:, :ctx], oc.vc[:, :ctx], oc.vs[:, :ctx])
+            if fused:
+                outs.append(kv.layer_call(0, q, kn, vn, ctx))
+            else:
+                kv.append_host(0, kn, vn, ctx)
+                outs.append(kv.layer_call(0, q, None, None, ctx))
+            rows = kv.export_rows(0, ctx, M)
+            outs.append(rows)
+    assert (outs[0].view(np.uint16) == outs[2].view(np.uint16)).all()
+    for a, b in zip(outs[1], outs[3]):
+        assert (a == b).all()
+
+
+def test_window_across_a_page_boundary_in_shuffled_pages(native, oracle):
+    ctx, M = 2 * 256 - 20, 64                    # rows 492..555: the window starts in page 1 and ends in page 2
+    q, k, v, kn, vn, ch = oracle.make_inputs(611, ctx, M)
+    oc = oracle.Cache(1024); oc.append(k, v, 0)
+    with native.KvCache(max_ctx=1024, paged=True) as kv:
+        kv.set_page_table(np.array([2, 0, 3, 1], np.int32))
+        kv.import_rows(0, 0, oc.kc[:, :ctx], oc.ks[:, :ctx], oc.vc[:, :ctx], oc.vs[:, :ctx])
+        out = kv.layer_call(0, q, kn, vn, ctx)
+        oc.append(kn, vn, ctx)
+        assert_attn_close(out, oc.attend_f32(q, ctx, threads=8, want_f32=True)[1], "paged window")
+        _rows_equal(kv, oc, ctx, M)
+
+
+def test_depth_table_on_a_wide_window(native, oracle):
+    ctx, M = 900, 24
+    kv, oc, q, kn, vn = _fill(native, oracle, 612, ctx, M)
+    depth = np.minimum(np.arange(M) // 2, 9).astype(np.uint8)     # a tree: rows see fewer keys than their index
+    with kv:
+        out = kv.layer_call(0, q, kn, vn, ctx, depth=depth)
+        oc.append(kn, vn, ctx)
+        assert_attn_close(out, oc.attend_f32(q, ctx, depth, threads=8, want_f32=True)[1], "depth table, wide")
+        _rows_equal(kv, oc, ctx, M)
+
+
+@pytest.mark.parametrize("hint", [64, 100000])
+def test_context_hint_only_sizes_the_grid(native, oracle, hint):
+    # option key 5 names the context the caller expects; any actual position stays correct
+    for ctx, M in ((3000, 1), (3000, 64), (40, 2)):
+        kv, oc, q, kn, vn = _fill(native, oracle, 620 + M, ctx, M, max_ctx=4096)
+        with kv:
+            kv.set_opt(5, hint)
+            out = kv.layer_call(0, q, kn, vn, ctx)
+            oc.append(kn, vn, ctx)
+            assert_attn_close(out, oc.attend_f32(q, ctx, threads=8, want_f32=True)[1], f"hint={hint} ctx={ctx} M={M}")
+            _rows_equal(kv, oc, ctx, M)
