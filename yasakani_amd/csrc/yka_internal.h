@@ -86,7 +86,8 @@ void launch_attn_post(const PostArgs&, hipStream_t);
 // the reference's own rows, head_dim 256 (attend256.hip): same argument structs, 67584-byte pages
 void launch_append256(const AppendArgs&, hipStream_t);
 void launch_rotate_q256(const float* x32, int rows, uint16_t* q16, hipStream_t);   // rotated query rows, rounded to fp16
-void launch_attend256(const AttnArgs&, hipStream_t);       // row tiles of 2 tokens x 6 heads for every width
+void launch_attend256(const AttnArgs&, hipStream_t);       // row tiles of 2 tokens x 6 heads (decode; any width)
+void launch_attend256_wide(const AttnArgs&, hipStream_t);  // 3..64 rows: 128 query rows per workgroup, tiles dequantized once into LDS
 void launch_combine256(const CombineArgs&, hipStream_t);
 void launch_export_rows256(const KvView&, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs, hipStream_t);
 void launch_import_rows256(const KvView&, int pos0, int n, const uint32_t* kw, const float* ks, const uint32_t* vw, const float* vs, hipStream_t);
