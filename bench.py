@@ -111,7 +111,7 @@ def small_decode(native, ctx=4096, L=128):
 
 def r256_figures(native, ctx=32768, L=16):
     """The reference's own rows (head_dim 256, one fp32 scale per row): 1,056 B per token per layer, 16 containers of
-    34.6 MB.  One layer call = append + attention (row tiles of 2 tokens) + combine."""
+    34.6 MB.  One layer call = append + attention (decode: row tiles of 2 tokens; windows: 128-row workgroups) + combine."""
     rng = np.random.default_rng(256)
     D2 = 256
     k = rng.standard_normal((4096 + 64, KVH, D2)).astype(np.float16)
