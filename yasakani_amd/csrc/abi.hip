@@ -111,7 +111,7 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
     for (int s0 = 0; s0 < M; s0 += kMaxSlice) {
       const int Ms = std::min(kMaxSlice, M - s0), tiles = (Ms + 1) / 2, rb = (kG * Ms + 127) / 128;
       const bool narrow = Ms <= 2 || kv->opt_force_narrow;
-      int S = narrow ? (kv->opt_splits_narrow > 0 ? kv->opt_splits_narrow : 512 / (kv->cfg.n_kv_heads * tiles))
+      int S = narrow ? (kv->opt_splits_narrow > 0 ? kv->opt_splits_narrow : std::min(512 / (kv->cfg.n_kv_heads * tiles), ((ctx + 31) / 32) / 2))
                      : (kv->opt_splits_wide > 0 ? kv->opt_splits_wide : std::min(256 / (kv->cfg.n_kv_heads * rb), ((ctx + 31) / 32) / (2 * rb)));
       S = std::min(std::max(narrow ? 2 : 1, std::min(kMaxSplits, S)), (int)(kWsPairs / (size_t)Ms));
       AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * 256, d_pos, depth, Ms, s0, NH, S, 0, kv->pm, kv->pl, kv->pacc16, nullptr, nullptr};

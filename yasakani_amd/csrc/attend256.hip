@@ -139,7 +139,19 @@ __global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
 #pragma unroll
   for (int o = 1; o < 16; o <<= 1) { maxlen = max(maxlen, __shfl_xor(maxlen, o, 64)); minlen = min(minlen, __shfl_xor(minlen, o, 64)); }
   maxlen = __builtin_amdgcn_readfirstlane(maxlen); minlen = __builtin_amdgcn_readfirstlane(minlen);
-  const int ntiles = (maxlen + 31) >> 5, tps = (ntiles + A.S - 1) / A.S;
+  // as many of the launched splits as the length found on the device justifies (two 32-key tiles per workgroup at
+  // least); the others leave the "no keys" marker, whose rows the combiner does not read
+  const int ntiles = (maxlen + 31) >> 5;
+  const int s_used = min(A.S, max(1, ntiles >> 1));
+  if (split >= s_used) {
+    const int j = threadIdx.x, tj = 2 * rt + j / kG;
+    if (j < 2 * kG && tj < A.M) {
+      const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
+      A.pm[p] = -1e30f; A.pl[p] = 0.f;
+    }
+    return;
+  }
+  const int tps = (ntiles + s_used - 1) / s_used;
   const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
 
   // Q fragments: k-step t of 8, lane (row i, group g), element e <-> channel 64g + 8t + [7,3,6,2,5,1,4,0][e]
@@ -258,7 +270,10 @@ __global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
 }
 
 // combiner (src/attention_kv4q.cu:325-332) for 256-channel rows: grid (n_heads, M), block 256 = 8 split lanes x 32 channel
-// lanes of 8 channels; the split lanes run in parallel (4 loads in flight each) and are summed through LDS.  S <= 256.
+// lanes of 8 channels; the split lanes run in parallel and are summed through LDS.  S <= 256.  kInFlight = partial rows a
+// split lane requests before it uses any: 16 covers 128 splits in one memory round trip (decode: few, long workgroups),
+// 4 keeps the register count low where thousands of workgroups run (wide windows).  Rows of weight 0 are not read.
+template <int kInFlight>
 __global__ void __launch_bounds__(256) combine256_kernel(CombineArgs A) {
   __shared__ float s_w[256];
   __shared__ float s_o[8][kD2 + 4];
@@ -281,16 +296,16 @@ __global__ void __launch_bounds__(256) combine256_kernel(CombineArgs A) {
   float wsum = 0.f;
   const uint16_t* src = A.pacc16 + p0 * kD2 + c8;
   const size_t stride = (size_t)A.n_heads * kD2;
-  for (int s0 = sl; s0 < A.S; s0 += 32) {
-    uint4 u[4]; float w[4];
+  for (int s0 = sl; s0 < A.S; s0 += 8 * kInFlight) {
+    uint4 u[kInFlight]; float w[kInFlight];
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < kInFlight; ++k) {
       const int sp = s0 + 8 * k;
       w[k] = sp < A.S ? s_w[sp] : 0.f;
-      u[k] = sp < A.S ? *reinterpret_cast<const uint4*>(src + (size_t)sp * stride) : make_uint4(0, 0, 0, 0);
+      u[k] = (sp < A.S && w[k] != 0.f) ? *reinterpret_cast<const uint4*>(src + (size_t)sp * stride) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < kInFlight; ++k) {
       const h8 v = __builtin_bit_cast(h8, u[k]);
 #pragma unroll
       for (int c = 0; c < 8; ++c) acc[c] += w[k] * (float)v[c];
@@ -319,7 +334,8 @@ void launch_attend256(const AttnArgs& A, hipStream_t st) {
   hipLaunchKernelGGL(attend256_kernel, dim3(A.S, A.kv.n_kv, (A.M + 1) / 2), dim3(256), 0, st, A);
 }
 void launch_combine256(const CombineArgs& A, hipStream_t st) {
-  hipLaunchKernelGGL(combine256_kernel, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
+  if (A.S > 32) hipLaunchKernelGGL(combine256_kernel<16>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
+  else hipLaunchKernelGGL(combine256_kernel<4>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
 }
 void launch_export_rows256(const KvView& kv, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs, hipStream_t st) {
   hipLaunchKernelGGL(xfer256_kernel<false>, dim3(n, kv.n_kv), dim3(64), 0, st, kv, pos0, n, kw, ks, vw, vs);
