@@ -106,7 +106,8 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
   if (kv->r256()) {
     // 256-channel rows: append first; rows of at most 2 tokens (or option key 3) run on row tiles of 2 tokens x 6 heads,
     // two workgroups per CU; wider slices on 128-row workgroups of 8 waves, one per CU
-    if (k16) do_append(kv, layer, k16, v16, M, d_pos, st);
+    const bool fuse256 = k16 && M <= 2;         // the decode kernel stores its own rows; wider passes launch the append first
+    if (k16 && !fuse256) do_append(kv, layer, k16, v16, M, d_pos, st);
     const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
     for (int s0 = 0; s0 < M; s0 += kMaxSlice) {
       const int Ms = std::min(kMaxSlice, M - s0), tiles = (Ms + 1) / 2, rb = (kG * Ms + 127) / 128;
@@ -114,7 +115,8 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
       int S = narrow ? (kv->opt_splits_narrow > 0 ? kv->opt_splits_narrow : std::min(512 / (kv->cfg.n_kv_heads * tiles), ((ctx + 31) / 32) / 2))
                      : (kv->opt_splits_wide > 0 ? kv->opt_splits_wide : std::min(256 / (kv->cfg.n_kv_heads * rb), ((ctx + 31) / 32) / (2 * rb)));
       S = std::min(std::max(narrow ? 2 : 1, std::min(kMaxSplits, S)), (int)(kWsPairs / (size_t)Ms));
-      AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * 256, d_pos, depth, Ms, s0, NH, S, 0, kv->pm, kv->pl, kv->pacc16, nullptr, nullptr};
+      AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * 256, d_pos, depth, Ms, s0, NH, S, 0, kv->pm, kv->pl, kv->pacc16,
+                 fuse256 ? k16 : nullptr, fuse256 ? v16 : nullptr};
       if (narrow) launch_attend256(A, st); else launch_attend256_wide(A, st);
       if (mode != 2) launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, kv->opt_unrot}, st);
     }

@@ -40,6 +40,33 @@ __device__ __forceinline__ uint8_t* page256(const KvView& kv, int kvh, int t) {
   return kv.base + (size_t)(pp * kv.n_kv + kvh) * kPage256Bytes;
 }
 
+// One row of 256 values (thread d holds channel d) -> 32 words + one fp32 scale at token `pos` of kv head `kvh`.  Called by
+// all 256 threads of a workgroup (three barriers inside); red[4] and fld[256] are its LDS scratch.
+__device__ __forceinline__ void quant_store_row256(const KvView& kv, int kvh, int pos, bool isv, float x, int d, float* red, uint8_t* fld) {
+  float am = fabsf(x);
+#pragma unroll
+  for (int o = 32; o; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, 64));
+  __syncthreads();                               // the scratch of a previous row is no longer read
+  if ((d & 63) == 0) red[d >> 6] = am;
+  __syncthreads();
+  am = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  float s7 = __fdiv_rn(am, 7.f);
+  if (s7 == 0.f) s7 = 1.f;
+  float q = rintf(__fdiv_rn(x, s7));
+  q = fminf(fmaxf(q, -7.f), 7.f);
+  fld[d] = (uint8_t)((int)q + 8);
+  __syncthreads();
+  uint8_t* pg = page256(kv, kvh, pos);
+  const int tp = pos % kPageTok;
+  if (d < 32) {                                  // word d = fields 8d .. 8d+7, the first in the top nibble
+    uint32_t w = 0u;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) w |= (uint32_t)fld[8 * d + k] << (28 - 4 * k);
+    reinterpret_cast<uint32_t*>(pg + (isv ? kP2Vw : kP2Kw))[tp * 32 + d] = w;
+  }
+  if (d == 0) reinterpret_cast<float*>(pg + (isv ? kP2Vs : kP2Ks))[tp] = s7;
+}
+
 // ---- quantize-on-append: grid (M, n_kv * 2), block 256 = one row, thread = channel ----
 __global__ void __launch_bounds__(256) append256_kernel(AppendArgs A) {
   __shared__ float red[4];
@@ -51,27 +78,7 @@ __global__ void __launch_bounds__(256) append256_kernel(AppendArgs A) {
   const size_t e = ((size_t)tok * A.kv.n_kv + kvh) * kD2 + d;
   float x = A.k32 ? (isv ? A.v32 : A.k32)[e] : __half2float(__ushort_as_half((isv ? A.v16 : A.k16)[e]));
   if (A.rot) x = rotate256(x, buf, false);
-  float am = fabsf(x);
-#pragma unroll
-  for (int o = 32; o; o >>= 1) am = fmaxf(am, __shfl_xor(am, o, 64));
-  if ((d & 63) == 0) red[d >> 6] = am;
-  __syncthreads();
-  am = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-  float s7 = __fdiv_rn(am, 7.f);
-  if (s7 == 0.f) s7 = 1.f;
-  float q = rintf(__fdiv_rn(x, s7));
-  q = fminf(fmaxf(q, -7.f), 7.f);
-  fld[d] = (uint8_t)((int)q + 8);
-  __syncthreads();
-  uint8_t* pg = page256(A.kv, kvh, pos);
-  const int tp = pos % kPageTok;
-  if (d < 32) {                                  // word d = fields 8d .. 8d+7, the first in the top nibble
-    uint32_t w = 0u;
-#pragma unroll
-    for (int k = 0; k < 8; ++k) w |= (uint32_t)fld[8 * d + k] << (28 - 4 * k);
-    reinterpret_cast<uint32_t*>(pg + (isv ? kP2Vw : kP2Kw))[tp * 32 + d] = w;
-  }
-  if (d == 0) reinterpret_cast<float*>(pg + (isv ? kP2Vs : kP2Ks))[tp] = s7;
+  quant_store_row256(A.kv, kvh, pos, isv, x, d, red, fld);
 }
 
 // ---- canonical image <-> pages: grid (n, n_kv), block 64: lanes 0..31 move K words, 32..63 V words ----
@@ -153,6 +160,28 @@ __global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
   }
   const int tps = (ntiles + s_used - 1) / s_used;
   const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
+
+  // ---- fused quantize-on-append (rows of at most 2 tokens, one row tile): a row of this pass is written by the one
+  //      workgroup whose tile range holds it - the only workgroup of this kv head that reads it in this launch; writer
+  //      and readers are waves of one CU and one write-through L1, so workgroup-scope fences order the stores ----
+  if (A.k16) {
+    __shared__ float a_red[4];
+    __shared__ uint8_t a_fld[256];
+    bool mine = false;
+    for (int t = 0; t < A.M; ++t) {
+      const int r = pos + A.tok0 + t;
+      if (r < 0 || r >= A.kv.max_ctx || (r >> 5) < tile0 || (r >> 5) >= tile1) continue;    // uniform over the workgroup
+      mine = true;
+      const size_t e = ((size_t)(A.tok0 + t) * A.kv.n_kv + kvh) * kD2 + threadIdx.x;
+      quant_store_row256(A.kv, kvh, r, false, __half2float(__ushort_as_half(A.k16[e])), threadIdx.x, a_red, a_fld);
+      quant_store_row256(A.kv, kvh, r, true, __half2float(__ushort_as_half(A.v16[e])), threadIdx.x, a_red, a_fld);
+    }
+    if (mine) {
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __syncthreads();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    }
+  }
 
   // Q fragments: k-step t of 8, lane (row i, group g), element e <-> channel 64g + 8t + [7,3,6,2,5,1,4,0][e]
   h8 qf[8];
