@@ -84,9 +84,11 @@ YKA_API int yka_append(yka_kv* kv, int layer, const uint16_t* d_k16, const uint1
 YKA_API int yka_attend(yka_kv* kv, int layer, const uint16_t* d_q16, int M, const int* d_pos,
                        const uint8_t* d_depth, uint16_t* d_out16, void* hip_stream);
 
-/* One layer call = yka_append then yka_attend on the same stream: the sequence of Engine35::attn_block
- * (engine35.cpp:911-934).  M may be as large as max_rows; passes wider than 64 rows are cut into 64-row slices
- * inside, as attn_block does (engine35.cpp:935-947). */
+/* One layer call = the effect of yka_append followed by yka_attend on the same stream: the sequence of
+ * Engine35::attn_block (engine35.cpp:911-934).  The rows are quantized inside the attention launches (each 64-row
+ * slice stores its own rows before it reads them; bit-identical to yka_append), so a layer call is two launches:
+ * attention and the split combiner.  M may be as large as max_rows; passes wider than 64 rows are cut into 64-row
+ * slices inside, as attn_block does (engine35.cpp:935-947). */
 YKA_API int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16_t* d_k16,
                               const uint16_t* d_v16, int M, const int* d_pos, const uint8_t* d_depth,
                               uint16_t* d_out16, void* hip_stream);
