@@ -318,7 +318,20 @@ __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
   __shared__ float s_wsum[16];
   const int head = blockIdx.x, tok = blockIdx.y, tid = threadIdx.x;
   const size_t p0 = (size_t)tok * A.S * A.n_heads + head;      // split s lives at p0 + s * n_heads
-  // weights: every thread of the first two waves looks at one split
+  // 16 split lanes; each takes splits sl, sl+16, ... (at most kInFlight of them: the launcher picks kInFlight so that
+  // 16 * kInFlight >= S).  Their partial rows are requested first, together with the (m, l) pairs the weights come
+  // from: one memory round trip instead of two.  A row of weight 0 may be one that no workgroup wrote: it is zeroed
+  // before use.
+  const int sl = tid >> 4, c8 = (tid & 15) * 8;
+  const uint16_t* src = A.pacc16 + p0 * kD + c8;
+  const size_t stride = (size_t)A.n_heads * kD;
+  uint4 u[kInFlight];
+#pragma unroll
+  for (int k = 0; k < kInFlight; ++k) {
+    const int sp = sl + 16 * k;
+    u[k] = sp < A.S ? *reinterpret_cast<const uint4*>(src + (size_t)sp * stride) : make_uint4(0, 0, 0, 0);
+  }
+  // weights: every thread looks at one split
   float pmv = -1e30f, plv = 0.f;
   if (tid < A.S) { pmv = A.pm[p0 + (size_t)tid * A.n_heads]; plv = A.pl[p0 + (size_t)tid * A.n_heads]; }
   float M2 = pmv;
@@ -329,28 +342,17 @@ __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
   M2 = fmaxf(fmaxf(s_wsum[0], s_wsum[1]), fmaxf(s_wsum[2], s_wsum[3]));
   s_w[tid] = (tid < A.S && pmv > -1e29f) ? exp2f(pmv - M2) * plv : 0.f;
   __syncthreads();
-  const int sl = tid >> 4, c8 = (tid & 15) * 8;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float wsum = 0.f;
-  // 16 split lanes; each takes splits sl, sl+16, ...; loads are issued 4 at a time so that their latencies overlap
-  const uint16_t* src = A.pacc16 + p0 * kD + c8;
-  const size_t stride = (size_t)A.n_heads * kD;
-  for (int s0 = sl; s0 < A.S; s0 += 16 * kInFlight) {
-    uint4 u[kInFlight]; float w[kInFlight];
 #pragma unroll
-    for (int k = 0; k < kInFlight; ++k) {
-      const int sp = s0 + 16 * k;
-      w[k] = sp < A.S ? s_w[sp] : 0.f;
-      // rows of weight 0 are not read: a split that was not used leaves its row unwritten
-      u[k] = (sp < A.S && w[k] != 0.f) ? *reinterpret_cast<const uint4*>(src + (size_t)sp * stride) : make_uint4(0, 0, 0, 0);
-    }
+  for (int k = 0; k < kInFlight; ++k) {
+    const int sp = sl + 16 * k;
+    const float w = sp < A.S ? s_w[sp] : 0.f;
+    const uint4 r = w != 0.f ? u[k] : make_uint4(0, 0, 0, 0);
+    const h8 v = __builtin_bit_cast(h8, r);
 #pragma unroll
-    for (int k = 0; k < kInFlight; ++k) {
-      const h8 v = __builtin_bit_cast(h8, u[k]);
-#pragma unroll
-      for (int c = 0; c < 8; ++c) acc[c] += w[k] * (float)v[c];
-      wsum += w[k];
-    }
+    for (int c = 0; c < 8; ++c) acc[c] += w * (float)v[c];
+    wsum += w;
   }
 #pragma unroll
   for (int c = 0; c < 8; ++c) s_o[sl][c8 + c] = acc[c];
@@ -384,7 +386,7 @@ __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
   if (tid < kD) A.out16[((size_t)tok * A.n_heads + head) * kD + tid] = __half_as_ushort(__float2half_rn(y));
 }
 void launch_combine(const CombineArgs& A, hipStream_t st) {
-  if (A.S > 64) hipLaunchKernelGGL(combine_kernel<16>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
+  if (A.S > 64) hipLaunchKernelGGL(combine_kernel<16>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);    // S <= 256
   else hipLaunchKernelGGL(combine_kernel<4>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
 }
 
