@@ -7,14 +7,22 @@
 //     Each 32-key tile is dequantized ONCE per workgroup into LDS - K as exact integer codes in fp16 (n-8, odd nibbles
 //     16(n-8)), V scaled and transposed (channel-major, the operand shape of the token-contracting MFMA) - and every
 //     wave reads its MFMA fragments from there;
-//   * a wave owns one tile of 32 rows (MFMA 32x32x16, the shape that sustains the full matrix rate on this chip) and
-//     stays under 256 registers, so two waves share a SIMD: one runs MFMAs while the other runs the softmax VALU work,
-//     and all MFMA results live in ordinary VGPRs (no accumulator-file copies);
+//   * a wave owns one tile of 32 rows (MFMA 32x32x16: one K or V fragment read from LDS serves 32 rows) and stays
+//     under 256 registers, so two waves share a SIMD and all MFMA results live in ordinary VGPRs (no accumulator-file
+//     copies).  Matrix and vector instructions share the SIMD's issue port and overlap little on this chip: the loop
+//     runs at about the sum of its MFMA time and its vector time;
 //   * the group scales of K are applied to the fp32 partial sum of each 32-channel group (two chained MFMAs per
 //     group), so K is never rounded; V carries one fp16 rounding;
 //   * the running maximum of a row is only raised when a score exceeds it by more than 2^8: accumulators stay in
 //     their registers untouched on almost every tile;
-//   * LDS is double buffered: tile n+1 is dequantized while tile n is consumed; one barrier per tile.
+//   * LDS is double buffered: tile n+1 is dequantized while tile n is consumed; one barrier per tile.  The PV product of
+//     a tile is issued one step later, next to that dequantization; the raw tile loads run two tiles ahead as explicit
+//     load instructions with their own counter waits;
+//   * the last split owns the tiles that hold the rows this pass appends and quantizes them itself before reading
+//     them (quantize-on-append without a launch of its own).
+// The values the instruction-form loads produce must reach their wait in the registers they were loaded into: the
+// generated code is checked for copies or spills of those registers whenever this file changes (none; they are loop
+// carried in fixed registers), and every parity test would fail on one.
 // LDS image of one tile (19456 bytes):
 //   K  [32 keys][272 B]   chunk 4m+g of a key = channels 32m+8g..+7 in the order n0,n4,n1,n5,n2,n6,n3,n7; the 272-byte
 //                          pitch makes the lanes of a fragment read hit distinct banks
