@@ -132,13 +132,17 @@ YKA_API int yka_attn_out256(const uint16_t* d_y16, const uint16_t* d_gate16, con
  * Q rows are written to d_q16 [M][n_heads][128] fp16; K and V rows are rounded to fp16 and quantized into rows
  * *d_pos .. *d_pos+M-1 of `layer` exactly as yka_append would store them.  d_xq [M][n_heads][128], d_xk, d_xv
  * [M][n_kv_heads][128] are the projection's fp32 outputs (the reference's split-K recombination and per-column factors,
- * q35_kernels.cu:1027-1032, happen before this call).  Allocates nothing, synchronises nothing. */
+ * q35_kernels.cu:1027-1032, happen before this call).  Allocates nothing, synchronises nothing.
+ * On a handle opened with head_dim 256 (the reference's own head size) the same call works on 256-channel rows: the
+ * normalisation divides by 256, the rotation is the 256-point kvx_rotate (x 1/16 for Q, K and V), Q rows leave as fp16
+ * [M][n_heads][256], and K / V rows go through the flat row quantizer (kvq_fast.cuh:194-198) as fp32 values, i.e. what
+ * yka_append256_f32 stores for them. */
 typedef struct yka_post_params {
-  const uint16_t* d_qn_w16;  /* [128] fp16 norm weights of Q heads, applied as (1 + w) (q35_kernels.cu:1057) */
-  const uint16_t* d_kn_w16;  /* [128] the same for K heads */
+  const uint16_t* d_qn_w16;  /* [head_dim] fp16 norm weights of Q heads, applied as (1 + w) (q35_kernels.cu:1057) */
+  const uint16_t* d_kn_w16;  /* [head_dim] the same for K heads */
   float eps;
   const float* d_rope;       /* [rope_rows][rope_dims/2][2] fp32 (cos, sin) by position (q35_kernels.cu:1101-1107) */
-  int32_t rope_dims;         /* even, 0..128; 0 = no rotary step (the reference rotates 64 of 256 channels, q35.hpp:13) */
+  int32_t rope_dims;         /* even, 0..head_dim; 0 = no rotary step (the reference rotates 64 of 256 channels, q35.hpp:13) */
   int32_t rope_rows;         /* rows whose position is not below rope_rows are dropped */
   int32_t rotate;            /* 0 / 1 */
 } yka_post_params;

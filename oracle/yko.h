@@ -36,6 +36,8 @@
  *                            q.k invariance
  *   yko_attn_post            pinned: numpy fp64 RMS normalisation and complex-multiplication rotary form within the
  *                            fp16 roundings, position 0 = no rotary change, pair-norm preservation, V rows pass through
+ *   yko_attn_post256         pinned the same way on 256 channels; its rotation is yko_kvx_rotate256 (pinned above), so the
+ *                            rotated rows are checked against the un-rotated ones through scipy's Sylvester matrix
  *
  * The reference holds no golden vectors or known-answer tests for this path, so
  * none are replayed here; the checks above are what the mathematics fixes.
@@ -87,6 +89,12 @@ void yko_attn_post(const float* xq, const float* xk, const float* xv, int M, int
                    const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope, int rd, int pos,
                    int rot, uint16_t* q16, uint16_t* k16, uint16_t* v16);
 void yko_unrotate_out(const float* y32, int rows, uint16_t* out16);
+/* the same step for 256-channel heads (src/q35_kernels.cu:1037-1065): Q rows as fp16, K / V rows as the fp32 rows the
+ * row quantizer takes */
+void yko_post256_qk_row(const float* y, const uint16_t* w16, float eps, const float* cs, int rd, int rot, float* o32);
+void yko_attn_post256(const float* xq, const float* xk, const float* xv, int M, int n_heads, int n_kv,
+                      const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope, int rd, int pos,
+                      int rot, uint16_t* q16, float* k32, float* v32);
 
 /* ---- canonical cache image used by the oracle and by the export/import hooks of the product ----
  * One layer: kc/vc [kvh][max_ctx][dim/2] bytes, ks/vs [kvh][max_ctx][dim/32] fp16 bit patterns. */

@@ -63,6 +63,7 @@ def lib():
         L.yko_rotate128.argtypes = [vp, vp, C.c_int, C.c_float]
         L.yko_attn_post.argtypes = [vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, C.c_float, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp]
         L.yko_unrotate_out.argtypes = [vp, C.c_int, vp]
+        L.yko_attn_post256.argtypes = [vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, C.c_float, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp]
         _lib = L
     return _lib
 
@@ -286,6 +287,23 @@ def attn_post(xq, xk, xv, qn_w16, kn_w16, eps, rope, rd, pos, rot):
     lib().yko_attn_post(_p(xq), _p(xk), _p(xv), M, H, KVH, _p(qw), _p(kw), float(eps), _p(rope), int(rd), int(pos), int(rot),
                         _p(q16), _p(k16), _p(v16))
     return q16, k16, v16
+
+
+def attn_post256(xq, xk, xv, qn_w16, kn_w16, eps, rope, rd, pos, rot):
+    """256-channel heads: fp32 projection rows -> (q16 fp16 bit patterns [M,H,256], k32, v32 fp32 [M,KVH,256]: the rows
+    the row quantizer takes)"""
+    xq = np.ascontiguousarray(xq, np.float32); xk = np.ascontiguousarray(xk, np.float32); xv = np.ascontiguousarray(xv, np.float32)
+    M, H, _ = xq.shape; KVH = xk.shape[1]
+    q16 = np.empty((M, H, 256), np.uint16); k32 = np.empty((M, KVH, 256), np.float32); v32 = np.empty((M, KVH, 256), np.float32)
+    qw = _as_u16(qn_w16); kw = _as_u16(kn_w16)
+    if rd > 0:
+        rope = np.ascontiguousarray(rope, np.float32)
+        assert rope.shape[0] >= pos + M and rope.shape[1] == rd // 2
+    else:
+        rope = np.zeros(1, np.float32)
+    lib().yko_attn_post256(_p(xq), _p(xk), _p(xv), M, H, KVH, _p(qw), _p(kw), float(eps), _p(rope), int(rd), int(pos), int(rot),
+                           _p(q16), _p(k32), _p(v32))
+    return q16, k32, v32
 
 
 def unrotate_out(y32):

@@ -103,3 +103,59 @@ void yko_unrotate_out(const float* y32, int rows, uint16_t* out16) {
     for (int d = 0; d < 128; ++d) out16[(size_t)r * 128 + d] = yko_f2h(o[d]);
   }
 }
+
+/* ---- the same step for 256-channel heads (the reference's own head size, src/q35_kernels.cu:1037-1065) ----
+ * Q and K: ss = sum y^2 - inside each quarter of 64 channels the butterfly a[i] += a[i ^ o], o = 32 .. 1, then
+ * ((q0 + q1) + q2) + q3; r = 1 / sqrt(ss / 256 + eps); xn = f16(y * r * (1 + w[d])); rotary on the first rd channels as
+ * above; then [the 256-point signed rotation x 1/16, yko_kvx_rotate256].  Q rows leave as fp16.  K rows (and V rows,
+ * which skip normalisation and the rotary step) leave as the fp32 values the row quantizer (yko_flat4_encode256) takes:
+ * fp16-valued when the rotation is off, the rotation's fp32 result when it is on. */
+static float sumsq256(const float* y) {
+  float q[4];
+  for (int w = 0; w < 4; ++w) {
+    float a[64], b[64];
+    for (int i = 0; i < 64; ++i) a[i] = y[64 * w + i] * y[64 * w + i];
+    for (int o = 32; o; o >>= 1) {
+      for (int i = 0; i < 64; ++i) b[i] = a[i] + a[i ^ o];
+      memcpy(a, b, sizeof a);
+    }
+    q[w] = a[0];
+  }
+  return ((q[0] + q[1]) + q[2]) + q[3];
+}
+
+/* one Q or K head row: y[256] -> o32[256] (before the final rounding of Q rows / the row quantizer of K rows) */
+void yko_post256_qk_row(const float* y, const uint16_t* w16, float eps, const float* cs, int rd, int rot, float* o32) {
+  const float tot = sumsq256(y);
+  const float r = 1.f / sqrtf(tot / 256.f + eps);
+  float xn[256], o[256];
+  for (int d = 0; d < 256; ++d) xn[d] = f16r((y[d] * r) * (1.f + yko_h2f(w16[d])));
+  const int hr = rd / 2;
+  for (int d = 0; d < 256; ++d) {
+    if (d < hr) o[d] = f16r(f16r(xn[d] * cs[2 * d]) + f16r(-xn[d + hr] * cs[2 * d + 1]));
+    else if (d < rd) o[d] = f16r(f16r(xn[d] * cs[2 * (d - hr)]) + f16r(xn[d - hr] * cs[2 * (d - hr) + 1]));
+    else o[d] = xn[d];
+  }
+  if (rot) yko_kvx_rotate256(o, o32, 0); else memcpy(o32, o, sizeof o);
+}
+
+/* xq [M][n_heads][256], xk, xv [M][n_kv][256] fp32; rope [rows][rd/2][2]; row t sits at position pos + t.
+ * q16 [M][n_heads][256] fp16; k32, v32 [M][n_kv][256]: the rows handed to the row quantizer. */
+void yko_attn_post256(const float* xq, const float* xk, const float* xv, int M, int n_heads, int n_kv,
+                      const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope, int rd, int pos,
+                      int rot, uint16_t* q16, float* k32, float* v32) {
+  for (int t = 0; t < M; ++t) {
+    const float* cs = rope + (size_t)(pos + t) * rd;
+    for (int h = 0; h < n_heads; ++h) {
+      float o[256];
+      yko_post256_qk_row(xq + ((size_t)t * n_heads + h) * 256, qn_w16, eps, cs, rd, rot, o);
+      for (int d = 0; d < 256; ++d) q16[((size_t)t * n_heads + h) * 256 + d] = yko_f2h(o[d]);
+    }
+    for (int h = 0; h < n_kv; ++h) {
+      yko_post256_qk_row(xk + ((size_t)t * n_kv + h) * 256, kn_w16, eps, cs, rd, rot, k32 + ((size_t)t * n_kv + h) * 256);
+      const float* y = xv + ((size_t)t * n_kv + h) * 256;
+      float* o = v32 + ((size_t)t * n_kv + h) * 256;
+      if (rot) yko_kvx_rotate256(y, o, 0); else memcpy(o, y, 256 * sizeof(float));
+    }
+  }
+}

@@ -6,7 +6,7 @@ comes from the reference: the fixtures freeze the oracle's outputs on small seed
 has been pinned by tests/test_oracle_*.py), so that (i) a later change of the oracle is noticed and (ii) the GPU
 tests can compare against committed data.
 
-    python tests/golden/make_golden.py        # rewrites codec_v1.npz, attention_v1.npz, row256_v1.npz and post_v1.npz
+    python tests/golden/make_golden.py        # rewrites codec_v1.npz, attention_v1.npz, row256_v1.npz, post_v1.npz and post256_v1.npz
 """
 import os
 import sys
@@ -100,10 +100,35 @@ def post_fixture():
     np.savez_compressed(os.path.join(HERE, "post_v1.npz"), **out)
 
 
+def post256_fixture():
+    """The same step for 256-channel heads: fp32 rows in, fp16 Q rows and the words / fp32 scales of the cache rows out."""
+    rng = np.random.default_rng(20261128)
+    M, rd, pos, ctx = 4, 64, 252, 512
+    xq = (rng.standard_normal((M, 24, 256)) * 2).astype(np.float32)
+    xk = (rng.standard_normal((M, 4, 256)) * 0.7).astype(np.float32)
+    xk[:, :, [5, 77, 130, 201]] *= 8
+    xv = rng.standard_normal((M, 4, 256)).astype(np.float32)
+    xq[1] = 0; xk[1] = 0; xv[1] = 0
+    qw = (rng.standard_normal(256) * 0.1).astype(np.float16).view(np.uint16)
+    kw = (rng.standard_normal(256) * 0.1).astype(np.float16).view(np.uint16)
+    rope = yko.rope_table(ctx, rd)
+    out = {"xq": xq, "xk": xk, "xv": xv, "qw": qw, "kw": kw, "rope": rope, "rd": np.int32(rd), "pos": np.int32(pos),
+           "eps": np.float32(1e-6), "ctx": np.int32(ctx)}
+    for rot in (0, 1):
+        q16, k32, v32 = yko.attn_post256(xq, xk, xv, qw, kw, 1e-6, rope, rd, pos, rot)
+        kw_ = np.empty((4, M, 32), np.uint32); vw_ = np.empty_like(kw_); ks_ = np.empty((4, M), np.float32); vs_ = np.empty_like(ks_)
+        for h in range(4):
+            kw_[h], ks_[h], _ = yko.flat4_encode256(k32[:, h])
+            vw_[h], vs_[h], _ = yko.flat4_encode256(v32[:, h])
+        out.update({f"r{rot}.q16": q16, f"r{rot}.kw": kw_, f"r{rot}.ks": ks_, f"r{rot}.vw": vw_, f"r{rot}.vs": vs_})
+    np.savez_compressed(os.path.join(HERE, "post256_v1.npz"), **out)
+
+
 if __name__ == "__main__":
     codec_fixture()
     attention_fixture()
     row256_fixture()
     post_fixture()
-    for f in ("codec_v1.npz", "attention_v1.npz", "row256_v1.npz", "post_v1.npz"):
+    post256_fixture()
+    for f in ("codec_v1.npz", "attention_v1.npz", "row256_v1.npz", "post_v1.npz", "post256_v1.npz"):
         print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

@@ -112,3 +112,29 @@ def test_gpu_reproduces_post_fixture(native):
         assert (q16.view(np.uint16) == g[f"r{rot}.q16"]).all()
         for arr, name in zip(got, ("kc", "ks", "vc", "vs")):
             assert (arr == g[f"r{rot}.{name}"]).all(), name
+
+
+def test_oracle_reproduces_post256_fixture(oracle):
+    g = _load("post256_v1.npz")
+    pos = int(g["pos"])
+    for rot in (0, 1):
+        q16, k32, v32 = oracle.attn_post256(g["xq"], g["xk"], g["xv"], g["qw"], g["kw"], float(g["eps"]), g["rope"], int(g["rd"]), pos, rot)
+        assert (q16 == g[f"r{rot}.q16"]).all()
+        for h in range(4):
+            w, s, _ = oracle.flat4_encode256(k32[:, h])
+            assert (w == g[f"r{rot}.kw"][h]).all() and (s.view(np.uint32) == g[f"r{rot}.ks"][h].view(np.uint32)).all()
+            w, s, _ = oracle.flat4_encode256(v32[:, h])
+            assert (w == g[f"r{rot}.vw"][h]).all() and (s.view(np.uint32) == g[f"r{rot}.vs"][h].view(np.uint32)).all()
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_post256_fixture(native):
+    g = _load("post256_v1.npz")
+    M, pos, ctx = g["xq"].shape[0], int(g["pos"]), int(g["ctx"])
+    for rot in (0, 1):
+        with native.KvCache(head_dim=256, max_ctx=ctx) as kv:
+            q16 = kv.attn_post_host(0, g["xq"], g["xk"], g["xv"], pos, g["qw"], g["kw"], float(g["eps"]), g["rope"], int(g["rd"]), rotate=bool(rot))
+            kw, ks, vw, vs = kv.export_rows(0, pos, M)
+        assert (q16.view(np.uint16) == g[f"r{rot}.q16"]).all()
+        assert (kw == g[f"r{rot}.kw"]).all() and (vw == g[f"r{rot}.vw"]).all()
+        assert (ks.view(np.uint32) == g[f"r{rot}.ks"].view(np.uint32)).all() and (vs.view(np.uint32) == g[f"r{rot}.vs"].view(np.uint32)).all()

@@ -91,3 +91,61 @@ def test_post_rejects_bad_arguments(native, oracle):
             kv.attn_post_host(0, xq, xk, xv, 0, qw, kw, 1e-6, oracle.rope_table(1, 32), 32)   # table shorter than pos + M
         with pytest.raises(native.YkaError):
             kv.attn_post_host(0, xq, xk, xv, 0, qw, kw, 1e-6, oracle.rope_table(8, 6)[:, :1], 3)   # odd rope_dims
+
+
+# ---- the same step for 256-channel heads (handles opened with head_dim = 256) ----
+
+def _inputs256(seed, M):
+    rng = np.random.default_rng(seed)
+    xq = (rng.standard_normal((M, 24, 256)) * 2.0).astype(np.float32)
+    xk = (rng.standard_normal((M, 4, 256)) * 0.7).astype(np.float32)
+    xk[:, :, [5, 77, 130, 201]] *= 8.0
+    xv = rng.standard_normal((M, 4, 256)).astype(np.float32)
+    qw = (rng.standard_normal(256) * 0.1).astype(np.float16)
+    kw = (rng.standard_normal(256) * 0.1).astype(np.float16)
+    return xq, xk, xv, qw, kw
+
+
+@pytest.mark.parametrize("paged", [False, True])
+@pytest.mark.parametrize("rot", [0, 1])
+@pytest.mark.parametrize("rd", [0, 64, 256])
+def test_post256_rows_bit_exact(native, oracle, paged, rot, rd):
+    M, pos, ctx = 11, 250, 512                             # the rows straddle a 256-token page
+    xq, xk, xv, qw, kw = _inputs256(40 + rd + rot, M)
+    xq[2] = 0.0; xk[2] = 0.0; xv[2] = 0.0                  # an all-zero token: eps keeps the norm finite, scales become 1
+    rope = oracle.rope_table(ctx, rd) if rd else None
+    rq, rk32, rv32 = oracle.attn_post256(xq, xk, xv, qw, kw, 1e-6, rope, rd, pos, rot)
+    with native.KvCache(head_dim=256, max_ctx=ctx, paged=paged) as kv:
+        if paged:
+            kv.set_page_table(np.array([1, 0], np.int32))
+        q16 = kv.attn_post_host(0, xq, xk, xv, pos, qw, kw, 1e-6, rope, rd, rotate=bool(rot))
+        kw_, ks_, vw_, vs_ = kv.export_rows(0, pos, M)
+    assert np.array_equal(q16.view(np.uint16), rq)
+    for h in range(4):
+        words, scale, _ = oracle.flat4_encode256(rk32[:, h])
+        assert np.array_equal(kw_[h], words) and np.array_equal(ks_[h].view(np.uint32), scale.view(np.uint32))
+        words, scale, _ = oracle.flat4_encode256(rv32[:, h])
+        assert np.array_equal(vw_[h], words) and np.array_equal(vs_[h].view(np.uint32), scale.view(np.uint32))
+
+
+def test_attention_over_rows_the_post256_step_stored(native, oracle):
+    # projection rows -> post step with rotation -> cache; Q rows of the pass attend to them; outputs rotated back
+    ctx, M, rd = 300, 4, 64
+    xq, xk, xv, qw, kw = _inputs256(50, ctx + M)
+    rope = oracle.rope_table(512, rd)
+    ref = oracle.Cache(512, 24, 4, 256)
+    with native.KvCache(head_dim=256, max_ctx=512, max_rows=64) as kv:
+        qs = []
+        for p in range(0, ctx + M, 64):
+            m = min(64, ctx + M - p)
+            qs.append(kv.attn_post_host(0, xq[p:p + m], xk[p:p + m], xv[p:p + m], p, qw, kw, 1e-6, rope, rd, rotate=True))
+            _, rk32, rv32 = oracle.attn_post256(xq[p:p + m], xk[p:p + m], xv[p:p + m], qw, kw, 1e-6, rope, rd, p, 1)
+            for h in range(4):
+                ref.kc[h, p:p + m], ref.ks[h, p:p + m], _ = oracle.flat4_encode256(rk32[:, h])
+                ref.vc[h, p:p + m], ref.vs[h, p:p + m], _ = oracle.flat4_encode256(rv32[:, h])
+        q16 = np.concatenate(qs)[ctx:]
+        kv.set_opt(4, 1)
+        out = kv.layer_call(0, q16, None, None, ctx)
+    _, o32 = ref.attend_f32(q16, ctx, want_f32=True)
+    expect = oracle.kvx_rotate256(o32.reshape(-1, 256), inverse=True).astype(np.float16).reshape(M, 24, 256)
+    assert_attn_close(out, expect, "attention over post256 rows, outputs un-rotated")

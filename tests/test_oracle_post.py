@@ -115,3 +115,63 @@ def test_unrotate_out_inverts_v_rotation():
     rv = yko.rotate128(v, False, 0.125)
     out = yko.unrotate_out(rv)
     assert np.abs(_h(out) - v).max() < 2e-3
+
+
+# ---- the same step for 256-channel heads ----
+
+def _post_numpy_d(y, w16, eps, cs, rd):
+    return _post_numpy(y, w16, eps, cs, rd)       # the fp64 form does not depend on the row length
+
+
+def test_post256_rows_match_fp64_forms_and_rotation():
+    rng = np.random.default_rng(13)
+    M, H, KVH, rd, pos = 3, 24, 4, 64, 21
+    xq = (rng.standard_normal((M, H, 256)) * 3).astype(np.float32)
+    xk = (rng.standard_normal((M, KVH, 256)) * 0.5).astype(np.float32)
+    xv = rng.standard_normal((M, KVH, 256)).astype(np.float32)
+    qw = (rng.standard_normal(256) * 0.1).astype(np.float16).view(np.uint16)
+    kw = (rng.standard_normal(256) * 0.1).astype(np.float16).view(np.uint16)
+    rope = yko.rope_table(32, rd)
+    q16, k32, v32 = yko.attn_post256(xq, xk, xv, qw, kw, 1e-6, rope, rd, pos, rot=0)
+    for t in range(M):
+        cs = rope[pos + t].astype(np.float64)
+        for h in range(H):
+            ref = _post_numpy_d(xq[t, h], qw, 1e-6, cs, rd)
+            assert np.abs(_h(q16[t, h]) - ref).max() <= 2.5e-3 * max(1.0, np.abs(ref).max())
+        for h in range(KVH):
+            ref = _post_numpy_d(xk[t, h], kw, 1e-6, cs, rd)
+            assert np.abs(k32[t, h] - ref).max() <= 2.5e-3 * max(1.0, np.abs(ref).max())
+    # K rows without rotation are fp16 valued; V rows pass through untouched
+    assert np.array_equal(k32, k32.astype(np.float16).astype(np.float32))
+    assert np.array_equal(v32, xv)
+    # channels past rd carry no rotary change: one rounding only
+    ref = _post_numpy_d(xq[0, 0], qw, 1e-6, rope[pos].astype(np.float64), rd)
+    assert np.array_equal(q16[0, 0, rd:], ref[rd:].astype(np.float16).view(np.uint16))
+    # with the rotation on: exactly the pinned 256-point rotation of the un-rotated rows (Q rounded to fp16 after it)
+    q16r, k32r, v32r = yko.attn_post256(xq, xk, xv, qw, kw, 1e-6, rope, rd, pos, rot=1)
+    qf = q16.view(np.float16).astype(np.float32).reshape(-1, 256)
+    assert np.array_equal(q16r.reshape(-1, 256), yko.kvx_rotate256(qf).astype(np.float16).view(np.uint16))
+    assert np.array_equal(k32r.reshape(-1, 256), yko.kvx_rotate256(k32.reshape(-1, 256)))
+    assert np.array_equal(v32r.reshape(-1, 256), yko.kvx_rotate256(xv.reshape(-1, 256)))
+
+
+def test_post256_structure():
+    rng = np.random.default_rng(14)
+    rd = 64
+    x = rng.standard_normal((1, 1, 256)).astype(np.float32)
+    zero_w = np.zeros(256, np.uint16)
+    rope = yko.rope_table(16, rd)
+    q16, _, _ = yko.attn_post256(x, x[:, :1], x[:, :1], zero_w, zero_w, 0.0, rope, rd, 0, 0)
+    assert abs(np.sqrt((_h(q16) ** 2).mean()) - 1.0) < 1e-3                 # unit RMS; position 0 turns nothing
+    qb, _, _ = yko.attn_post256(x, x[:, :1], x[:, :1], zero_w, zero_w, 0.0, rope, rd, 7, 0)
+    a, b = _h(q16)[0, 0], _h(qb)[0, 0]
+    hr = rd // 2
+    assert np.allclose(a[:hr] ** 2 + a[hr:rd] ** 2, b[:hr] ** 2 + b[hr:rd] ** 2, atol=2e-2)
+    assert np.array_equal(a[rd:], b[rd:]) and not np.array_equal(a[:rd], b[:rd])
+    qc, _, _ = yko.attn_post256(x * 4, x[:, :1], x[:, :1], zero_w, zero_w, 0.0, rope, rd, 7, 0)
+    assert np.array_equal(qb, qc)                                            # power-of-two scale invariance: exact
+    # the sum of squares is exact on small integers whatever the order: r = 1 / sqrt(ss / 256)
+    xi = rng.integers(-3, 4, size=(1, 1, 256)).astype(np.float32)
+    qi, _, _ = yko.attn_post256(xi, xi[:, :1], xi[:, :1], zero_w, zero_w, 0.0, rope, 0, 0, 0)
+    r = np.float32(1.0) / np.sqrt(np.float32((xi.astype(np.float64) ** 2).sum() / 256.0))
+    assert np.array_equal(qi[0, 0], (xi[0, 0] * r).astype(np.float16).view(np.uint16))

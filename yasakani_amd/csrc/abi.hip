@@ -337,18 +337,18 @@ int yka_codec_probe(const uint16_t* x16, int rows, uint8_t* codes, uint16_t* sca
 static void check_post(const yka_kv* kv, const yka_post_params* P) {
   if (!P) throw std::runtime_error("null parameter block");
   if (!P->d_qn_w16 || !P->d_kn_w16) throw std::runtime_error("null norm weights");
-  if (P->rope_dims < 0 || P->rope_dims > kD || (P->rope_dims & 1)) throw std::runtime_error("rope_dims must be even and in [0, 128]");
+  if (P->rope_dims < 0 || P->rope_dims > kv->D() || (P->rope_dims & 1)) throw std::runtime_error("rope_dims must be even and in [0, head_dim]");
   if (P->rope_dims > 0 && (!P->d_rope || P->rope_rows < 1)) throw std::runtime_error("rotary table missing");
-  (void)kv;
 }
 
 int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float* d_xk, const float* d_xv, int M, const int* d_pos,
                   const yka_post_params* P, uint16_t* d_q16, void* hip_stream) {
   YKA_TRY
-  on_device(kv); need_128(kv); check_layer(kv, layer); check_rows(kv, M); check_post(kv, P);
+  on_device(kv); check_layer(kv, layer); check_rows(kv, M); check_post(kv, P);
   if (!d_xq || !d_xk || !d_xv || !d_pos || !d_q16) throw std::runtime_error("null pointer");
-  launch_attn_post(PostArgs{kv->view(layer), d_xq, d_xk, d_xv, M, kv->cfg.n_heads, d_pos, P->d_qn_w16, P->d_kn_w16, P->eps,
-                            P->d_rope, P->rope_dims, P->rope_rows, P->rotate != 0, d_q16}, (hipStream_t)hip_stream);
+  const PostArgs A{kv->view(layer), d_xq, d_xk, d_xv, M, kv->cfg.n_heads, d_pos, P->d_qn_w16, P->d_kn_w16, P->eps,
+                   P->d_rope, P->rope_dims, P->rope_rows, P->rotate != 0, d_q16};
+  if (kv->r256()) launch_attn_post256(A, (hipStream_t)hip_stream); else launch_attn_post(A, (hipStream_t)hip_stream);
   HIPCHK(hipGetLastError());
   YKA_CATCH_INT
 }
@@ -357,14 +357,15 @@ int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, 
                        const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope, int rope_dims,
                        int rope_rows, int rotate, uint16_t* q16) {
   YKA_TRY
-  on_device(kv); need_128(kv); check_layer(kv, layer); check_rows(kv, M);
+  on_device(kv); check_layer(kv, layer); check_rows(kv, M);
   if (!xq || !xk || !xv || !qn_w16 || !kn_w16 || !q16) throw std::runtime_error("null pointer");
   if (pos < 0 || (long long)pos + M > kv->cfg.max_ctx) throw std::runtime_error("rows outside the container");
-  if (rope_dims < 0 || rope_dims > kD || (rope_dims & 1)) throw std::runtime_error("rope_dims must be even and in [0, 128]");
+  const int kD = kv->D();                          // 128 or 256 channels per head
+  if (rope_dims < 0 || rope_dims > kD || (rope_dims & 1)) throw std::runtime_error("rope_dims must be even and in [0, head_dim]");
   if (rope_dims > 0 && (!rope || rope_rows < pos + M)) throw std::runtime_error("rotary table shorter than pos + M");
   const size_t nq = (size_t)M * kv->cfg.n_heads * kD, nk = (size_t)M * kv->cfg.n_kv_heads * kD;
   const size_t nr = rope_dims > 0 ? (size_t)rope_rows * rope_dims : 1;
-  DevBuf dq(nq * 4), dk(nk * 4), dv(nk * 4), dqw(kD * 2), dkw(kD * 2), dr(nr * 4), dq16(nq * 2);
+  DevBuf dq(nq * 4), dk(nk * 4), dv(nk * 4), dqw((size_t)kD * 2), dkw((size_t)kD * 2), dr(nr * 4), dq16(nq * 2);
   HIPCHK(hipMemcpy(dq.p, xq, nq * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dk.p, xk, nk * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dv.p, xv, nk * 4, hipMemcpyHostToDevice));
@@ -374,8 +375,9 @@ int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, 
   yka_post_params P{dqw.as<uint16_t>(), dkw.as<uint16_t>(), eps, dr.as<float>(), rope_dims, rope_rows, rotate};
   check_post(kv, &P);
   launch_set_int(kv->d_pos, pos, kv->stream);
-  launch_attn_post(PostArgs{kv->view(layer), dq.as<float>(), dk.as<float>(), dv.as<float>(), M, kv->cfg.n_heads, kv->d_pos,
-                            P.d_qn_w16, P.d_kn_w16, eps, P.d_rope, rope_dims, rope_rows, rotate != 0, dq16.as<uint16_t>()}, kv->stream);
+  const PostArgs A{kv->view(layer), dq.as<float>(), dk.as<float>(), dv.as<float>(), M, kv->cfg.n_heads, kv->d_pos,
+                   P.d_qn_w16, P.d_kn_w16, eps, P.d_rope, rope_dims, rope_rows, rotate != 0, dq16.as<uint16_t>()};
+  if (kv->r256()) launch_attn_post256(A, kv->stream); else launch_attn_post(A, kv->stream);
   HIPCHK(hipGetLastError());
   HIPCHK(hipStreamSynchronize(kv->stream));
   HIPCHK(hipMemcpy(q16, dq16.p, nq * 2, hipMemcpyDeviceToHost));

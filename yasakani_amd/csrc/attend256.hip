@@ -81,6 +81,61 @@ __global__ void __launch_bounds__(256) append256_kernel(AppendArgs A) {
   quant_store_row256(A.kv, kvh, pos, isv, x, d, red, fld);
 }
 
+// ---- the step between the QKV projection and the cache for 256-channel heads, fused with quantize-on-append
+//      (src/q35_kernels.cu:1037-1065 with fp16 in the place of the reference's bf16 roundings): per-head RMS normalisation
+//      (sum of squares: butterfly inside each wave, then ((w0 + w1) + w2) + w3), partial rotary embedding with the
+//      rotate-half pairing, optional 256-point signed rotation; Q rows leave as fp16, K and V rows go through the row
+//      quantizer as fp32 values.  grid (n_heads + 2 n_kv, M), block 256 = one head row. ----
+__device__ __forceinline__ float f16r256(float x) { asm volatile("" : "+v"(x)); return __half2float(__float2half_rn(x)); }
+__global__ void __launch_bounds__(256) attn_post256_kernel(PostArgs A) {
+  __shared__ float buf[256];
+  __shared__ float red[4];
+  __shared__ uint8_t fld[256];
+  const int blk = blockIdx.x, tok = blockIdx.y, d = threadIdx.x;
+  const int NH = A.n_heads, KVH = A.kv.n_kv;
+  const int pos = *A.d_pos + tok;
+  if (pos < 0 || pos >= A.kv.max_ctx || (A.rd > 0 && pos >= A.rope_rows)) return;   // rows outside the container are dropped
+  const bool isq = blk < NH, isk = !isq && blk < NH + KVH;
+  const int head = isq ? blk : (isk ? blk - NH : blk - NH - KVH);
+  const float* src = isq ? A.xq + ((size_t)tok * NH + head) * kD2
+                         : (isk ? A.xk : A.xv) + ((size_t)tok * KVH + head) * kD2;
+  const float y = src[d];
+  float out;
+  if (isq || isk) {
+    float ss = __fmul_rn(y, y);
+#pragma unroll
+    for (int o = 32; o; o >>= 1) ss = __fadd_rn(ss, __shfl_xor(ss, o, 64));
+    if ((d & 63) == 0) red[d >> 6] = ss;
+    __syncthreads();
+    const float tot = __fadd_rn(__fadd_rn(__fadd_rn(red[0], red[1]), red[2]), red[3]);
+    // sqrtf, not __fsqrt_rn: only the former is correctly rounded on this target
+    const float r = __fdiv_rn(1.f, sqrtf(__fadd_rn(__fdiv_rn(tot, 256.f), A.eps)));
+    const float w = __half2float(__ushort_as_half((isq ? A.qn_w16 : A.kn_w16)[d]));
+    const float xn = f16r256(__fmul_rn(__fmul_rn(y, r), __fadd_rn(1.f, w)));
+    out = xn;
+    const int hr = A.rd >> 1;
+    if (hr > 0) {
+      buf[d] = xn;
+      __syncthreads();
+      if (d < A.rd) {
+        const int i = d < hr ? d : d - hr;
+        const float2 cs = reinterpret_cast<const float2*>(A.rope)[(size_t)pos * hr + i];
+        const float partner = d < hr ? -buf[d + hr] : buf[d - hr];
+        out = f16r256(__fadd_rn(f16r256(__fmul_rn(xn, cs.x)), f16r256(__fmul_rn(partner, cs.y))));
+      }
+    }
+    if (A.rot) out = rotate256(out, buf, false);
+  } else {
+    out = A.rot ? rotate256(y, buf, false) : y;
+  }
+  if (isq) {
+    asm volatile("" : "+v"(out));                  // the rotation's last multiply is rounded to fp32 before the fp16 rounding
+    A.q16[((size_t)tok * NH + head) * kD2 + d] = __half_as_ushort(__float2half_rn(out));
+  } else {
+    quant_store_row256(A.kv, head, pos, !isk, out, d, red, fld);
+  }
+}
+
 // ---- canonical image <-> pages: grid (n, n_kv), block 64: lanes 0..31 move K words, 32..63 V words ----
 // rotated query rows: grid rows, block 256
 __global__ void __launch_bounds__(256) rotate_q256_kernel(const float* x32, uint16_t* q16) {
@@ -353,6 +408,9 @@ __global__ void __launch_bounds__(256) combine256_kernel(CombineArgs A) {
   A.out16[((size_t)tok * A.n_heads + head) * kD2 + tid] = __half_as_ushort(__float2half_rn(y));
 }
 
+void launch_attn_post256(const PostArgs& A, hipStream_t st) {
+  hipLaunchKernelGGL(attn_post256_kernel, dim3(A.n_heads + 2 * A.kv.n_kv, A.M), dim3(256), 0, st, A);
+}
 void launch_append256(const AppendArgs& A, hipStream_t st) {
   hipLaunchKernelGGL(append256_kernel, dim3(A.M, A.kv.n_kv * 2), dim3(256), 0, st, A);
 }

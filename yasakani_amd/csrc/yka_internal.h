@@ -83,6 +83,7 @@ void launch_attend_narrow(const AttnArgs&, hipStream_t);   // 16-row tiles: 2 to
 void launch_attend_wide(const AttnArgs&, hipStream_t);     // 3..64 tokens
 void launch_combine(const CombineArgs&, hipStream_t);
 void launch_attn_post(const PostArgs&, hipStream_t);
+void launch_attn_post256(const PostArgs&, hipStream_t);    // the same step for 256-channel heads (attend256.hip)
 // the reference's own rows, head_dim 256 (attend256.hip): same argument structs, 67584-byte pages
 void launch_append256(const AppendArgs&, hipStream_t);
 void launch_rotate_q256(const float* x32, int rows, uint16_t* q16, hipStream_t);   // rotated query rows, rounded to fp16

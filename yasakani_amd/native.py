@@ -311,9 +311,10 @@ class KvCache:
         _chk(lib().yka_append_host(self._h, layer, _ptr(k), _ptr(v), M, pos))
 
     def attn_post_host(self, layer, xq, xk, xv, pos, qn_w16, kn_w16, eps, rope, rope_dims, rotate=False):
-        """Projection outputs (fp32; xq [M,n_heads,128], xk/xv [M,n_kv_heads,128]) -> RMS norm, rotary, optional
-        rotation; K/V rows are quantized into rows pos..pos+M-1, the Q rows come back as fp16 [M,n_heads,128]."""
+        """Projection outputs (fp32; xq [M,n_heads,head_dim], xk/xv [M,n_kv_heads,head_dim]) -> RMS norm, rotary,
+        optional rotation; K/V rows are quantized into rows pos..pos+M-1, the Q rows come back as fp16."""
         M = xq.shape[0]
+        D = self.cfg.head_dim
         xq = np.ascontiguousarray(xq, np.float32).reshape(M, self.cfg.n_heads, D)
         xk = np.ascontiguousarray(xk, np.float32).reshape(M, self.cfg.n_kv_heads, D)
         xv = np.ascontiguousarray(xv, np.float32).reshape(M, self.cfg.n_kv_heads, D)
