@@ -273,6 +273,8 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary decode / verify-16 / verify-32 lines")
     ap.add_argument("--batched-only", action="store_true",
                     help="run only the multi-stream (batched decode) passes and print their figures (for profiling that kernel)")
+    ap.add_argument("--r256-only", action="store_true",
+                    help="run only the passes over the reference's 256-channel rows and print their figures (for profiling those kernels)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three device-to-device copies of 256 MiB (a kernel of known traffic, for scaling FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -284,6 +286,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
 
+    if args.r256_only:
+        print(json.dumps({"reference_rows_head_dim_256": r256_figures(native, args.ctx)}))
+        return
     ctx, M, L = args.ctx, args.rows, args.layers
     max_ctx = ((ctx + 64 + 255) // 256) * 256
     q, k, v = synth(2026, ctx, 64)

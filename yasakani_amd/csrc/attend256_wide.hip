@@ -10,9 +10,9 @@
 //     fragments take 32 registers), so that two waves fit a SIMD;
 //   * LDS is double buffered: tile n+1 is dequantized while tile n is consumed; one barrier per tile; the tile loads are
 //     explicit instructions two tiles ahead with their own waits.
-// LDS image of one tile (37632 bytes):
-//   K  [32 keys][528 B]    chunk c (16 bytes) of a key = word c of its row = channels 8c + [7,3,6,2,5,1,4,0]
-//   V  [256 channels][80 B] key 16kb + 4g + r sits at slot 8g + 4kb + r: the 8 keys whose probabilities an MFMA lane of
+// LDS image of one tile (42240 bytes):
+//   K  [32 keys][544 B]    chunk c (16 bytes) of a key = word c of its row = channels 8c + [7,3,6,2,5,1,4,0]
+//   V  [256 channels][96 B] key 16kb + 4g + r sits at slot 8g + 4kb + r: the 8 keys whose probabilities an MFMA lane of
 //                           group g holds are 16 contiguous bytes
 //   SC [2][32] fp32        K scales, V scales of the tile's keys
 #include "yka_internal.h"
@@ -37,8 +37,13 @@ constexpr int kP2Kw = 0, kP2Vw = 32768, kP2Ks = 65536, kP2Vs = 66560;
 constexpr uint32_t kMagic = 0x64006400u;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int NT = 512;                        // threads per workgroup (8 waves x 16 rows)
-constexpr int kKPitch = 528, kVPitch = 80;
-constexpr int kLdsK = 0, kLdsV = 32 * kKPitch, kLdsS = kLdsV + kD2 * kVPitch, kLdsBuf = kLdsS + 256;   // 37632
+// Row pitches: a 128-bit LDS read of a wave is served 16 lanes at a time, and the 16 are lanes {0-7, 24-31}, {8-15, 16-23}
+// (and the same in the upper half) - measured.  With lane = row i + 16 * group g, i.e. (i 0-7, g) together with
+// (i 8-15, g+1), the 16 lanes of a pass fall into 16 different 4-bank groups iff the pitch is 2 * odd chunks of 16 bytes:
+// 34 chunks for K rows, 6 for V rows.  (33 and 5 chunks, free of conflicts for 16 consecutive lanes, measure a 2-way
+// conflict on every fragment read.)
+constexpr int kKPitch = 544, kVPitch = 96;
+constexpr int kLdsK = 0, kLdsV = 32 * kKPitch, kLdsS = kLdsV + kD2 * kVPitch, kLdsBuf = kLdsS + 256;   // 42240
 constexpr float kRaise = 8.f;                  // log2 slack before a running maximum is raised
 
 __device__ __forceinline__ uint8_t* page256w(const KvView& kv, int kvh, int t) {
@@ -256,7 +261,7 @@ __global__ void __launch_bounds__(NT, 1) attend256_wide_kernel(AttnArgs A) {
   // ---- partials: normalised fp16.  o[b][r] of lane (row i, group g) is channel 16b + 4g + r.  Rows go through LDS (the
   //      tile buffers are free after the last barrier) so that every store instruction writes whole 512-byte rows ----
   constexpr int kOPitch = 2 * kD2 + 16;                      // bytes per staged row
-  uint8_t* stage = &lds[0][0] + wave * 16 * kOPitch;         // 8 waves x 8448 bytes
+  uint8_t* stage = &lds[0][0] + wave * 16 * kOPitch;         // 8 waves x 8448 bytes of the 84480
   float l = l_run;
   l += __shfl_xor(l, 16, 64);
   l += __shfl_xor(l, 32, 64);
