@@ -100,7 +100,8 @@ YKA_API int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, cons
  * consecutive positions (a stream's last token and its draft tokens).  A row whose slot or position is out of range is
  * dropped and yields zeros.  Replaces launch_q35_attn_post_ms / launch_tb_requant_ms, launch_q35_atx_pk_ms and
  * launch_q35_combine_ms (q35.hpp:28-35,109-112,157; q35_atxpk.hpp:18-20; kernel src/q35_atxpk_ms.cu).  The reference caps
- * such a pass at 16 rows (Q35_SST, q35.hpp:20); here M may be up to max_rows.  Allocates nothing, synchronises nothing. */
+ * such a pass at 16 rows (Q35_SST, q35.hpp:20); here M may be up to max_rows.  Works on both row formats (head_dim 128
+ * and 256: the reference's multi-stream kernel runs on its 256-channel rows).  Allocates nothing, synchronises nothing. */
 YKA_API int yka_append_attend_ms(yka_kv* kv, const uint16_t* d_q16, const uint16_t* d_k16, const uint16_t* d_v16, int M,
                                  const int* d_row_pos, const int* d_row_slot, uint16_t* d_out16, void* hip_stream);
 

@@ -93,8 +93,6 @@ def test_entry_points_of_the_other_format_refuse(native):
     with native.KvCache(head_dim=D, max_ctx=256) as kv:
         with pytest.raises(native.YkaError, match="128"):
             kv.dequant_rows(0, 0, 1)
-        with pytest.raises(native.YkaError, match="128"):
-            kv.ms_call(np.zeros((1, NH, 128), np.float16), None, None, [0], [0])
     with native.KvCache(max_ctx=256) as kv:
         with pytest.raises(native.YkaError, match="256"):
             native._chk(native.lib().yka_kv_export_rows256(kv._h, 0, 0, 1, None, None, None, None))

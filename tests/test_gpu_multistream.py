@@ -94,3 +94,71 @@ def test_rejected_rows_yield_zeros_and_touch_nothing(native, oracle):
             assert np.array_equal(a, b)
         with pytest.raises(native.YkaError):
             kv.ms_call(q, k, None, pos, slots)
+
+
+# ---- the same passes over the reference's own 256-channel rows (handles opened with head_dim = 256) ----
+
+def _streams256(native, oracle, paged, seed=5):
+    rng = np.random.default_rng(seed)
+    kv = native.KvCache(n_layers=len(LENS), head_dim=256, max_ctx=CTX, max_rows=64, paged=paged)
+    if paged:
+        for s in range(len(LENS)):
+            kv.set_page_table(rng.permutation(CTX // 256).astype(np.int32), layer=s)
+    refs = []
+    for s, n in enumerate(LENS):
+        ref = oracle.Cache(CTX, 24, 4, 256)
+        if n:
+            k = rng.standard_normal((n, 4, 256)).astype(np.float16)
+            k[:, :, [5, 77, 130, 201]] *= 8
+            v = rng.standard_normal((n, 4, 256)).astype(np.float16)
+            for p in range(0, n, 64):
+                kv.append_host(s, k[p:p + 64], v[p:p + 64], p)
+            ref.append(k, v, 0)
+        refs.append(ref)
+    return kv, refs, rng
+
+
+def _rows256(rng, M):
+    return tuple(rng.standard_normal((M, h, 256)).astype(np.float16) for h in (24, 4, 4))
+
+
+@pytest.mark.parametrize("paged", [False, True])
+def test_one_row_per_stream_256(native, oracle, paged):
+    kv, refs, rng = _streams256(native, oracle, paged)
+    with kv:
+        slots = np.array([2, 0, 4, 1, 3], np.int32)
+        pos = np.array([LENS[s] for s in slots], np.int32)
+        q, k, v = _rows256(rng, len(slots))
+        out = kv.ms_call(q, k, v, pos, slots)
+        for t, s in enumerate(slots):
+            refs[s].append(k[t:t + 1], v[t:t + 1], int(pos[t]))
+            assert_attn_close(out[t:t + 1], refs[s].attend_f32(q[t:t + 1], int(pos[t])), f"row {t} stream {s}")
+            got = kv.export_rows(int(s), int(pos[t]), 1)
+            assert np.array_equal(got[0], refs[s].kc[:, pos[t]:pos[t] + 1]) and np.array_equal(got[2], refs[s].vc[:, pos[t]:pos[t] + 1])
+            assert np.array_equal(got[1].view(np.uint32), refs[s].ks[:, pos[t]:pos[t] + 1].view(np.uint32))
+            assert np.array_equal(got[3].view(np.uint32), refs[s].vs[:, pos[t]:pos[t] + 1].view(np.uint32))
+
+
+def test_rows_of_one_stream_and_bad_rows_256(native, oracle):
+    kv, refs, rng = _streams256(native, oracle, False)
+    with kv:
+        # stream 0: its last token and two draft tokens (they see each other's keys); stream 2: one row; a row whose slot
+        # does not exist and one whose position lies outside its container yield zeros and write nothing
+        slots = np.array([0, 0, 0, 2, 9, 1], np.int32)
+        pos = np.array([300, 301, 302, 900, 5, CTX], np.int32)
+        q, k, v = _rows256(rng, 6)
+        out = kv.ms_call(q, k, v, pos, slots)
+        refs[0].append(k[0:3], v[0:3], 300)
+        assert_attn_close(out[0:3], refs[0].attend_f32(q[0:3], 300), "stream 0 window")
+        refs[2].append(k[3:4], v[3:4], 900)
+        assert_attn_close(out[3:4], refs[2].attend_f32(q[3:4], 900), "stream 2")
+        assert not out[4:6].view(np.uint16).any()
+        # attend only, more rows than the reference's 16-row cap
+        M = 20
+        slots = np.array([s % 4 for s in range(M)], np.int32)
+        pos = np.array([max(0, LENS[s] - 1 - t) for t, s in enumerate(slots)], np.int32)
+        q = rng.standard_normal((M, 24, 256)).astype(np.float16)
+        out = kv.ms_call(q, None, None, pos, slots)
+        for t, s in enumerate(slots):
+            if LENS[s] + (3 if s == 0 else 1 if s == 2 else 0) > pos[t]:
+                assert_attn_close(out[t:t + 1], refs[s].attend_f32(q[t:t + 1], int(pos[t])), f"attend-only row {t}")

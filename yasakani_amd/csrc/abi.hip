@@ -142,17 +142,19 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
 // keys), then every row attends to keys [0, pos[t]] of its own container.  One token per workgroup column.
 void do_attend_ms(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, const int* row_pos,
                   const int* row_slot, uint16_t* out16, hipStream_t st) {
-  const int NH = kv->cfg.n_heads;
+  const int NH = kv->cfg.n_heads, D = kv->D();
+  const bool r256 = kv->r256();
   const RowMap R{row_pos, row_slot, kv->cfg.n_layers, kv->layer_bytes, kv->n_pages};
-  if (k16) launch_append(AppendArgs{kv->view(0), k16, v16, nullptr, M, R}, st);
+  if (k16) { const AppendArgs P{kv->view(0), k16, v16, nullptr, M, R}; if (r256) launch_append256(P, st); else launch_append(P, st); }
   for (int s0 = 0; s0 < M; s0 += kMaxSlice) {
     const int Ms = std::min(kMaxSlice, M - s0);
-    int S = kv->opt_splits_narrow > 0 ? kv->opt_splits_narrow : 1024 / (kv->cfg.n_kv_heads * Ms);
+    int S = kv->opt_splits_narrow > 0 ? kv->opt_splits_narrow : (r256 ? 512 : 1024) / (kv->cfg.n_kv_heads * Ms);   // 2 / 4 waves per SIMD
     S = std::min(std::max(2, std::min(kMaxSplits, S)), (int)(kWsPairs / (size_t)Ms));
     RowMap Rs = R; Rs.pos += s0; Rs.slot += s0;
-    AttnArgs A{kv->view(0), q16 + (size_t)s0 * NH * kD, nullptr, nullptr, Ms, s0, NH, S, 128, kv->pm, kv->pl, kv->pacc16, nullptr, nullptr, Rs};
-    launch_attend_narrow(A, st);
-    launch_combine(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD, kv->opt_unrot}, st);
+    AttnArgs A{kv->view(0), q16 + (size_t)s0 * NH * D, nullptr, nullptr, Ms, s0, NH, S, 128, kv->pm, kv->pl, kv->pacc16, nullptr, nullptr, Rs};
+    const CombineArgs C{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * D, kv->opt_unrot};
+    if (r256) { launch_attend256(A, st); launch_combine256(C, st); }
+    else { launch_attend_narrow(A, st); launch_combine(C, st); }
   }
 }
 
@@ -291,7 +293,7 @@ int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16
 int yka_append_attend_ms(yka_kv* kv, const uint16_t* d_q16, const uint16_t* d_k16, const uint16_t* d_v16, int M,
                          const int* d_row_pos, const int* d_row_slot, uint16_t* d_out16, void* hip_stream) {
   YKA_TRY
-  on_device(kv); need_128(kv); check_rows(kv, M);
+  on_device(kv); check_rows(kv, M);
   if (!d_q16 || !d_row_pos || !d_row_slot || !d_out16) throw std::runtime_error("null pointer");
   if ((d_k16 == nullptr) != (d_v16 == nullptr)) throw std::runtime_error("new K and V rows come together or not at all");
   do_attend_ms(kv, d_q16, d_k16, d_v16, M, d_row_pos, d_row_slot, d_out16, (hipStream_t)hip_stream);
@@ -302,10 +304,10 @@ int yka_append_attend_ms(yka_kv* kv, const uint16_t* d_q16, const uint16_t* d_k1
 int yka_ms_call_host(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, const int32_t* row_pos,
                      const int32_t* row_slot, uint16_t* out16) {
   YKA_TRY
-  on_device(kv); need_128(kv); check_rows(kv, M);
+  on_device(kv); check_rows(kv, M);
   if (!q16 || !row_pos || !row_slot || !out16) throw std::runtime_error("null pointer");
   if ((k16 == nullptr) != (v16 == nullptr)) throw std::runtime_error("new K and V rows come together or not at all");
-  const size_t nq = (size_t)M * kv->cfg.n_heads * kD, nk = (size_t)M * kv->cfg.n_kv_heads * kD;
+  const size_t nq = (size_t)M * kv->cfg.n_heads * kv->D(), nk = (size_t)M * kv->cfg.n_kv_heads * kv->D();
   DevBuf dq(nq * 2), dk(nk * 2), dv(nk * 2), dout(nq * 2), dp((size_t)M * 4), dsl((size_t)M * 4);
   HIPCHK(hipMemcpy(dq.p, q16, nq * 2, hipMemcpyHostToDevice));
   if (k16) { HIPCHK(hipMemcpy(dk.p, k16, nk * 2, hipMemcpyHostToDevice)); HIPCHK(hipMemcpy(dv.p, v16, nk * 2, hipMemcpyHostToDevice)); }

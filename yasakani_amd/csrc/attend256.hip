@@ -73,8 +73,16 @@ __global__ void __launch_bounds__(256) append256_kernel(AppendArgs A) {
   __shared__ float buf[256];
   __shared__ uint8_t fld[256];
   const int tok = blockIdx.x, kvh = blockIdx.y >> 1, isv = blockIdx.y & 1, d = threadIdx.x;
-  const int pos = *A.d_pos + tok;
-  if (pos < 0 || pos >= A.kv.max_ctx) return;
+  int pos;
+  if (A.rows.pos) {                                // multi-stream pass: the row's own container and position
+    pos = A.rows.pos[tok];
+    const int slot = A.rows.slot[tok];
+    if (pos < 0 || pos >= A.kv.max_ctx || slot < 0 || slot >= A.rows.n_slots) return;
+    A.kv = slot_view(A.kv, A.rows, slot);
+  } else {
+    pos = *A.d_pos + tok;
+    if (pos < 0 || pos >= A.kv.max_ctx) return;
+  }
   const size_t e = ((size_t)tok * A.kv.n_kv + kvh) * kD2 + d;
   float x = A.k32 ? (isv ? A.v32 : A.k32)[e] : __half2float(__ushort_as_half((isv ? A.v16 : A.k16)[e]));
   if (A.rot) x = rotate256(x, buf, false);
@@ -184,19 +192,35 @@ __device__ __forceinline__ void load_tile256(const uint8_t* pg, int tp, const Of
 
 }  // namespace
 
-// grid (S, n_kv, ceil(M/2)), block 256 (4 waves, 2 waves per SIMD).  Workgroup = (split, kv head, 2 tokens x 6 heads).
+// grid (S, n_kv, ceil(M/TPT)), block 256 (4 waves, 2 waves per SIMD).  Workgroup = (split, kv head, TPT tokens x 6 heads):
+// TPT = 2 for a single-stream pass; MS (multi-stream pass, reference: src/q35_atxpk_ms.cu:13-33): one token per row
+// tile, which reads the container and the position its row map names.
+template <bool MS>
 __global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
+  constexpr int TPT = MS ? 1 : 2;
   __shared__ float s_m[4][16], s_l[4][16];
   __shared__ float s_acc[4][16][kD2 + 4];
   const int split = blockIdx.x, kvh = blockIdx.y, rt = blockIdx.z;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
-  const int pos = *A.d_pos;
-  const int tl = 2 * rt + i / kG;
-  const bool vrow = i < 2 * kG && tl < A.M;
+  int pos; bool row_ok = true;
+  if (MS) {
+    pos = A.rows.pos[rt];
+    const int slot = A.rows.slot[rt];
+    row_ok = pos >= 0 && pos < A.kv.max_ctx && slot >= 0 && slot < A.rows.n_slots;   // a bad row reads nothing and yields zeros
+    A.kv = slot_view(A.kv, A.rows, row_ok ? slot : 0);
+  } else {
+    pos = *A.d_pos;
+  }
+  const int tl = TPT * rt + i / kG;
+  const bool vrow = i < TPT * kG && tl < A.M && row_ok;
   const int head = kvh * kG + i % kG;
   int len = 0;
-  if (vrow) { const int tg = A.tok0 + tl; len = min(pos + (A.depth ? (int)A.depth[tg] : tg) + 1, A.kv.max_ctx); }
+  if (vrow) {
+    if (MS) len = pos + 1;
+    else { const int tg = A.tok0 + tl; len = pos + (A.depth ? (int)A.depth[tg] : tg) + 1; }
+    len = min(len, A.kv.max_ctx);
+  }
   int maxlen = len, minlen = vrow ? len : 0x7fffffff;
 #pragma unroll
   for (int o = 1; o < 16; o <<= 1) { maxlen = max(maxlen, __shfl_xor(maxlen, o, 64)); minlen = min(minlen, __shfl_xor(minlen, o, 64)); }
@@ -206,8 +230,8 @@ __global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
   const int ntiles = (maxlen + 31) >> 5;
   const int s_used = min(A.S, max(1, ntiles >> 1));
   if (split >= s_used) {
-    const int j = threadIdx.x, tj = 2 * rt + j / kG;
-    if (j < 2 * kG && tj < A.M) {
+    const int j = threadIdx.x, tj = TPT * rt + j / kG;
+    if (j < TPT * kG && tj < A.M) {
       const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
       A.pm[p] = -1e30f; A.pl[p] = 0.f;
     }
@@ -219,7 +243,7 @@ __global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
   // ---- fused quantize-on-append (rows of at most 2 tokens, one row tile): a row of this pass is written by the one
   //      workgroup whose tile range holds it - the only workgroup of this kv head that reads it in this launch; writer
   //      and readers are waves of one CU and one write-through L1, so workgroup-scope fences order the stores ----
-  if (A.k16) {
+  if (!MS && A.k16) {
     __shared__ float a_red[4];
     __shared__ uint8_t a_fld[256];
     bool mine = false;
@@ -338,9 +362,9 @@ __global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) s_acc[wave][i][8 * (4 * g + r + 16 * hh) + el] = o[hh * 8 + el][r];
   __syncthreads();
-  for (int idx = threadIdx.x; idx < 2 * kG * kD2; idx += 256) {
+  for (int idx = threadIdx.x; idx < TPT * kG * kD2; idx += 256) {
     const int j = idx >> 8, d = idx & (kD2 - 1);
-    const int tj = 2 * rt + j / kG;
+    const int tj = TPT * rt + j / kG;
     if (tj >= A.M) continue;
     const float m0 = s_m[0][j], m1 = s_m[1][j], m2 = s_m[2][j], m3 = s_m[3][j];
     const float M2 = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
@@ -418,7 +442,8 @@ void launch_rotate_q256(const float* x32, int rows, uint16_t* q16, hipStream_t s
   hipLaunchKernelGGL(rotate_q256_kernel, dim3(rows), dim3(256), 0, st, x32, q16);
 }
 void launch_attend256(const AttnArgs& A, hipStream_t st) {
-  hipLaunchKernelGGL(attend256_kernel, dim3(A.S, A.kv.n_kv, (A.M + 1) / 2), dim3(256), 0, st, A);
+  if (A.rows.pos) hipLaunchKernelGGL(attend256_kernel<true>, dim3(A.S, A.kv.n_kv, A.M), dim3(256), 0, st, A);
+  else hipLaunchKernelGGL(attend256_kernel<false>, dim3(A.S, A.kv.n_kv, (A.M + 1) / 2), dim3(256), 0, st, A);
 }
 void launch_combine256(const CombineArgs& A, hipStream_t st) {
   if (A.S > 32) hipLaunchKernelGGL(combine256_kernel<16>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);

@@ -233,8 +233,9 @@ class KvCache:
         _chk(lib().yka_append_attend_ms(self._h, d_q16, d_k16, d_v16, M, d_row_pos, d_row_slot, d_out16, stream))
 
     def ms_call(self, q16, k16, v16, row_pos, row_slot):
-        """Multi-stream pass with host arrays: q16 [M,n_heads,128], k16/v16 [M,n_kv_heads,128] (or None), row_pos/row_slot [M]."""
+        """Multi-stream pass with host arrays: q16 [M,n_heads,head_dim], k16/v16 [M,n_kv_heads,head_dim] (or None), row_pos/row_slot [M]."""
         M = q16.shape[0]
+        D = self.cfg.head_dim
         q = _u16(q16, (M, self.cfg.n_heads, D))
         k = None if k16 is None else _u16(k16, (M, self.cfg.n_kv_heads, D))
         v = None if v16 is None else _u16(v16, (M, self.cfg.n_kv_heads, D))
