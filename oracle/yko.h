@@ -38,6 +38,14 @@
  *                            fp16 roundings, position 0 = no rotary change, pair-norm preservation, V rows pass through
  *   yko_attn_post256         pinned the same way on 256 channels; its rotation is yko_kvx_rotate256 (pinned above), so the
  *                            rotated rows are checked against the un-rotated ones through scipy's Sylvester matrix
+ *   yko_tb_viterbi           pinned: exhaustive search over all paths on short chunks (minimum cost, and among equal
+ *                            costs the path the tie rules name, on tables with repeated values)
+ *   yko_tb_pack /            pinned: numpy.unpackbits on the big-endian byte image of the words; the sliding 8-bit
+ *   yko_tb_decode_row        window against the state recursion; decode(encode(y)) == the encoder's own x, bit for bit
+ *   yko_tb_encode_row        pinned as an algorithm: projections / rms against numpy fp64 within fp32 rounding, the kept
+ *                            multiplier against a direct error evaluation of every multiplier, flat mode against
+ *                            yko_flat4_encode256.  PARITY UNPINNED against real profiles: the reference's tables live
+ *                            in a profile blob (kvq_u5.bin) that is not in its repository; tests use synthetic blobs
  *
  * The reference holds no golden vectors or known-answer tests for this path, so
  * none are replayed here; the checks above are what the mathematics fixes.
@@ -95,6 +103,17 @@ void yko_post256_qk_row(const float* y, const uint16_t* w16, float eps, const fl
 void yko_attn_post256(const float* xq, const float* xk, const float* xv, int M, int n_heads, int n_kv,
                       const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope, int rd, int pos,
                       int rot, uint16_t* q16, float* k32, float* v32);
+
+/* ---- trellis-coded rows (src/kvq_gpu.cuh:51-147, src/kvq_fast.cuh:63-233, decode src/kvq_attn.cuh:46-75) ---- */
+int yko_tb_check_blob(const uint8_t* blob, size_t n);                 /* 0 if a KVQP v1 blob this codec can use */
+int yko_tb_group(const uint8_t* blob, int g, int* fields6);           /* mode, kk, table, guard, m, has_mu */
+int yko_tb_viterbi(const int* xi, int T, const int16_t* ci, int kk, uint8_t* states);
+int yko_tb_encode_row(const uint8_t* blob, int g, int pos, const float* y, float* x, uint8_t* fields, float* scale,
+                      uint32_t* pc, int* best_mi);
+void yko_tb_pack(const uint8_t* fields, int kb, uint32_t* words);
+int yko_tb_decode_row(const uint8_t* blob, int g, const uint32_t* words, float scale, uint32_t pc, float* y);
+void yko_tb_encode_rows(const uint8_t* blob, const int* grp, const int* pos, int n, const float* y, float* x, uint32_t* words,
+                        int stride_words, float* scale, uint32_t* pc, int* best_mi, int* coded);
 
 /* ---- canonical cache image used by the oracle and by the export/import hooks of the product ----
  * One layer: kc/vc [kvh][max_ctx][dim/2] bytes, ks/vs [kvh][max_ctx][dim/32] fp16 bit patterns. */

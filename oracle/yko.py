@@ -64,6 +64,12 @@ def lib():
         L.yko_attn_post.argtypes = [vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, C.c_float, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp]
         L.yko_unrotate_out.argtypes = [vp, C.c_int, vp]
         L.yko_attn_post256.argtypes = [vp, vp, vp, C.c_int, C.c_int, C.c_int, vp, vp, C.c_float, vp, C.c_int, C.c_int, C.c_int, vp, vp, vp]
+        L.yko_tb_check_blob.argtypes = [vp, C.c_size_t]
+        L.yko_tb_group.argtypes = [vp, C.c_int, vp]
+        L.yko_tb_viterbi.argtypes = [vp, C.c_int, vp, C.c_int, vp]
+        L.yko_tb_pack.argtypes = [vp, C.c_int, vp]
+        L.yko_tb_decode_row.argtypes = [vp, C.c_int, vp, C.c_float, C.c_uint32, vp]
+        L.yko_tb_encode_rows.argtypes = [vp, vp, vp, C.c_int, vp, vp, vp, C.c_int, vp, vp, vp, vp]
         _lib = L
     return _lib
 
@@ -322,3 +328,52 @@ def attn_out256(y16, gate16, signs):
     qx = np.empty((M, H * 256), np.int8); alpha = np.empty((M, H * 256 // 512), np.float32)
     lib().yko_attn_out256(_p(y), _p(g), _p(sg), M, H, _p(qx), _p(alpha))
     return qx, alpha
+
+
+# ---- trellis-coded rows ----
+def tb_check_blob(blob):
+    b = np.frombuffer(bytes(blob), np.uint8)
+    return lib().yko_tb_check_blob(_p(b), b.size)
+
+
+def tb_group(blob, g):
+    b = np.frombuffer(bytes(blob), np.uint8); f = np.zeros(6, np.int32)
+    if lib().yko_tb_group(_p(b), int(g), _p(f)) != 0:
+        raise IndexError(g)
+    return dict(zip(("mode", "kk", "table", "guard", "m", "has_mu"), (int(v) for v in f)))
+
+
+def tb_viterbi(xi, ci, kk):
+    """one chunk: integer targets xi [T <= 64], table ci [256] int16 -> (states [T] uint8, path cost)"""
+    xi = np.ascontiguousarray(xi, np.int32); ci = np.ascontiguousarray(ci, np.int16)
+    st = np.zeros(xi.size, np.uint8)
+    cost = lib().yko_tb_viterbi(_p(xi), int(xi.size), _p(ci), int(kk), _p(st))
+    return st, cost
+
+
+def tb_pack(fields, kb):
+    fields = np.ascontiguousarray(fields, np.uint8); w = np.zeros(8 * kb, np.uint32)
+    lib().yko_tb_pack(_p(fields), int(kb), _p(w))
+    return w
+
+
+def tb_encode_rows(blob, grp, pos, y, stride_words=40):
+    """rows y [n, 256] fp32 of groups grp [n] at positions pos [n] -> dict(x, words [n, stride_words], scale, pc, best_mi, coded)"""
+    b = np.frombuffer(bytes(blob), np.uint8)
+    y = np.ascontiguousarray(y, np.float32); n = y.shape[0]
+    grp = np.ascontiguousarray(grp, np.int32); pos = np.ascontiguousarray(pos, np.int32)
+    out = dict(x=np.empty((n, 256), np.float32), words=np.zeros((n, stride_words), np.uint32), scale=np.empty(n, np.float32),
+               pc=np.empty(n, np.uint32), best_mi=np.empty(n, np.int32), coded=np.empty(n, np.int32))
+    lib().yko_tb_encode_rows(_p(b), _p(grp), _p(pos), n, _p(y), _p(out["x"]), _p(out["words"]), int(stride_words), _p(out["scale"]),
+                             _p(out["pc"]), _p(out["best_mi"]), _p(out["coded"]))
+    return out
+
+
+def tb_decode_rows(blob, grp, words, scale, pc):
+    b = np.frombuffer(bytes(blob), np.uint8)
+    words = np.ascontiguousarray(words, np.uint32); n = words.shape[0]
+    y = np.empty((n, 256), np.float32)
+    for i in range(n):
+        if lib().yko_tb_decode_row(_p(b), int(grp[i]), _p(words[i]), float(scale[i]), int(pc[i]), _p(y[i])) != 0:
+            raise IndexError(int(grp[i]))
+    return y
