@@ -180,6 +180,18 @@ YKA_API int yka_codec_probe(const uint16_t* x16, int rows, uint8_t* codes, uint1
  * may be NULL.  Results are bit-identical to the reference's arithmetic. */
 YKA_API int yka_kvx256_probe(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, float* y);
 
+/* Trellis-coded rows (the reference's KV4 / KV5 row formats): encode, pack, unpack.  Replaces yskn_tbp_pack_unpack
+ * (kvx_probe.cu:123-188; kernels launch_tb_fast, kvq_fast.cuh:63-233, and tba_unpack_kernel, kvq_attn.cuh:46-75).
+ * blob: a "KVQP" v1 profile (host memory); x [rows][256] fp32; grp / pos [rows]: the group ((layer * kv heads + kv head)
+ * * 2 + K|V) and the position of every row; stride: bytes between payload rows (>= 160).  Outputs, all host memory:
+ * y_fq [rows][256] = what each row decodes to according to the encoder; pay [rows][stride]: 8 * kb MSB-first words per
+ * coded row (kb = the group's bits per element, 4 for flat groups), zero otherwise; side [rows][2]: the row's fp32 scale
+ * and two fp16 projection coefficients; y_dec [rows][256] = the decoder's result from pay and side (x for rows that stay
+ * uncoded: position below the group's guard, or no such group).  Bit-identical to the reference's arithmetic for the
+ * same blob.  Synchronous; allocates. */
+YKA_API int yka_tb_pack_unpack(const uint8_t* blob, size_t blob_len, const float* x, const int* grp, const int* pos, int rows,
+                               int stride, float* y_fq, uint8_t* pay, uint32_t* side, float* y_dec);
+
 /* Canonical image of rows [pos0, pos0+n) of one layer, independent of the physical layout:
  * kc/vc [n_kv_heads][n][64], ks/vs [n_kv_heads][n][4].  export = device -> host, import = host -> device.
  * (The reference reads its containers back only inside its hooks, e.g. kvx_probe.cu:369.) Synchronous. */

@@ -405,6 +405,72 @@ int yka_kvx256_probe(const float* x, int rows, int mode, int rot, int8_t* q8, ui
   YKA_CATCH_INT
 }
 
+// ---- trellis-coded rows ----
+}  // extern "C"
+namespace {
+struct TbInfo { int nm = 0, ngrp = 0, layers = 0, kv_heads = 0; bool has_trellis = false; };
+// the checks of the reference's loaders (src/engine35.cpp:48-52, src/kvq_fast.hpp:52-76) plus bounds on every record
+TbInfo tb_check_blob(const uint8_t* b, size_t n) {
+  auto u16 = [&](size_t o) { return (unsigned)b[o] | ((unsigned)b[o + 1] << 8); };
+  auto u32 = [&](size_t o) { return u16(o) | (u16(o + 2) << 16); };
+  if (!b || n < 100 || std::memcmp(b, "KVQP", 4) != 0 || u16(4) != 1 || u32(8) != n) throw std::runtime_error("not a KVQP v1 profile blob");
+  if (u16(16) != 256) throw std::runtime_error("profile blob: rows must have 256 elements");
+  TbInfo I; I.layers = (int)u16(18); I.kv_heads = (int)u16(20); I.nm = (int)u16(24); I.ngrp = (int)u32(28);
+  const unsigned nt = u16(22);
+  const size_t off_m = u32(32), off_t = u32(36), off_g = u32(40);
+  if (I.nm < 1 || I.nm > 16) throw std::runtime_error("profile blob: bad scale-multiplier count");
+  if (off_m + 4 * (size_t)I.nm > n || off_t + 4 * (size_t)nt > n || off_g + 4 * (size_t)I.ngrp > n) throw std::runtime_error("profile blob: offsets outside the blob");
+  for (unsigned t = 0; t < nt; ++t) {
+    const size_t to = u32(off_t + 4 * t);
+    if (to + 12 + 512 > n || b[to] != 8 || b[to + 2] != 64 || b[to + 3] != 8) throw std::runtime_error("profile blob: tables must have 8 state bits, chunks of 64");
+    for (int s = 0; s < 256; ++s) { const int c = (int)(short)u16(to + 12 + 2 * (size_t)s); if (c > 1100 || c < -1100) throw std::runtime_error("profile blob: table value out of range"); }
+  }
+  for (int g = 0; g < I.ngrp; ++g) {
+    const size_t go = u32(off_g + 4 * (size_t)g);
+    if (go + 8 > n) throw std::runtime_error("profile blob: group record outside the blob");
+    const int mode = b[go], kk = b[go + 1], tix = b[go + 2], m = b[go + 4], has_mu = b[go + 5];
+    if (mode > 1 || m > 2 || go + 8 + (has_mu ? 512 : 0) + 512 * (size_t)m > n) throw std::runtime_error("profile blob: bad group record");
+    if (mode == 0) { if (kk < 3 || kk > 5 || (unsigned)tix >= nt) throw std::runtime_error("profile blob: trellis groups need 3..5 bits and a table"); I.has_trellis = true; }
+  }
+  return I;
+}
+}  // namespace
+extern "C" {
+
+int yka_tb_pack_unpack(const uint8_t* blob, size_t blob_len, const float* x, const int* grp, const int* pos, int rows, int stride,
+                       float* y_fq, uint8_t* pay, uint32_t* side, float* y_dec) {
+  YKA_TRY
+  if (!x || !grp || !pos || rows < 1 || !y_fq || !pay || !side || !y_dec) throw std::runtime_error("bad argument");
+  if (stride < 160 || stride > 1024 || stride % 4) throw std::runtime_error("stride must be a multiple of 4 in [160, 1024]");
+  const TbInfo I = tb_check_blob(blob, blob_len);
+  constexpr int kTile = 1024;                        // rows per launch
+  const size_t nx = (size_t)rows * 256, w_ofs = (size_t)kTile * I.nm * 256;
+  DevBuf db(blob_len), dx(nx * 4), dg((size_t)rows * 4), dp((size_t)rows * 4), dy(nx * 4), dpay((size_t)rows * stride), dside((size_t)rows * 8),
+         dd(nx * 4), scr(w_ofs + (size_t)kTile * I.nm * 32);
+  HIPCHK(hipMemcpy(db.p, blob, blob_len, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dx.p, x, nx * 4, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dg.p, grp, (size_t)rows * 4, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dp.p, pos, (size_t)rows * 4, hipMemcpyHostToDevice));
+  for (int r0 = 0; r0 < rows; r0 += kTile) {
+    TbEncArgs A{};
+    A.blob = db.as<uint8_t>(); A.nm = I.nm; A.has_trellis = I.has_trellis;
+    A.yin = dx.as<float>(); A.grp = dg.as<int>(); A.pos = dp.as<int>(); A.row0 = r0; A.nrow = std::min(kTile, rows - r0);
+    A.yout = dy.as<float>(); A.side = dside.as<uint32_t>(); A.scr = scr.as<uint8_t>(); A.scr_w_ofs = w_ofs;
+    A.pay0 = dpay.as<uint8_t>(); A.stride = stride;
+    launch_tb_encode(A, nullptr);
+    HIPCHK(hipGetLastError());
+    HIPCHK(hipDeviceSynchronize());                  // the scratch block is reused by the next tile
+  }
+  launch_tb_unpack(db.as<uint8_t>(), dg.as<int>(), dp.as<int>(), dpay.as<uint8_t>(), dside.as<uint32_t>(), stride, dx.as<float>(), dd.as<float>(), rows, nullptr);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipDeviceSynchronize());
+  HIPCHK(hipMemcpy(y_fq, dy.p, nx * 4, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(pay, dpay.p, (size_t)rows * stride, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(side, dside.p, (size_t)rows * 8, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(y_dec, dd.p, nx * 4, hipMemcpyDeviceToHost));
+  YKA_CATCH_INT
+}
+
 static void check_range(const yka_kv* kv, int pos0, int n) {
   if (pos0 < 0 || n < 1 || (long long)pos0 + n > kv->cfg.max_ctx) throw std::runtime_error("row range outside the container");
 }

@@ -77,6 +77,23 @@ struct PostArgs {
   int rot; uint16_t* q16;
 };
 
+// Trellis-coded rows (trellis.hip; reference TbFastArgs, src/kvq_fast.hpp:16-37).  Probe form (yin != nullptr): rows
+// row0 .. row0 + nrow - 1 of yin with their own group and position; results indexed by row.  Cache form: row rj of the
+// launch is (token rj / (2 n_kv), K | V, kv head) of the pass, read from k32 / v32 [M][n_kv][256]; its payload goes to
+// pay0 (K) / pay1 (V) + (kvh * max_ctx + pos) * stride and its scale to scl0 / scl1 [kvh * max_ctx + pos].
+struct TbEncArgs {
+  const uint8_t* blob; int nm; int has_trellis;
+  const float* k32; const float* v32; const int* d_pos; int layer, tok0, n_kv, max_ctx, rot;
+  const float* yin; const int* grp; const int* pos; int row0;
+  float* yout; uint32_t* side; int* coded;
+  int nrow;
+  uint8_t* scr; size_t scr_w_ofs;     // scratch: states [nrow * nm][256] bytes, then at scr_w_ofs error sums [nrow * nm][8] fp32
+  uint8_t* pay0; uint8_t* pay1; float* scl0; float* scl1; int stride;
+};
+void launch_tb_encode(const TbEncArgs&, hipStream_t);
+void launch_tb_unpack(const uint8_t* blob, const int* grp, const int* pos, const uint8_t* pay, const uint32_t* side, int stride, const float* yin,
+                      float* y, int rows, hipStream_t);
+
 // launchers (each checks nothing: the C layer validates shapes first)
 void launch_append(const AppendArgs&, hipStream_t);
 void launch_attend_narrow(const AttnArgs&, hipStream_t);   // 16-row tiles: 2 tokens x 6 heads per workgroup column

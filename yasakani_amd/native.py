@@ -53,6 +53,7 @@ def _load():
         "yka_codec_probe": (i32, [vp, i32, vp, vp, vp]),
         "yka_kvx256_probe": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_attn_post": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
+        "yka_tb_pack_unpack": (i32, [vp, C.c_size_t, vp, vp, vp, i32, i32, vp, vp, vp, vp]),
         "yka_kv_export_rows256": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_append256_f32": (i32, [vp, i32, vp, vp, i32, vp, i32, vp]),
         "yka_attn_out256": (i32, [vp, vp, vp, i32, i32, vp, vp, vp]),
@@ -82,7 +83,7 @@ def _load():
 
 
 EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "yka_set_opt", "yka_kv_set_page_table",
-           "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kvx256_probe", "yka_attn_post", "yka_append_attend_ms", "yka_ms_call_host",
+           "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kvx256_probe", "yka_tb_pack_unpack", "yka_attn_post", "yka_append_attend_ms", "yka_ms_call_host",
            "yka_attn_post_host", "yka_kv_export_rows", "yka_kv_export_rows256", "yka_kv_import_rows256",
            "yka_attn_out256", "yka_attn_out256_host", "yka_append256_f32", "yka_rotate_q256", "yka_append256_f32_host", "yka_rotate_q256_host",
            "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
@@ -168,6 +169,20 @@ def kvx256_probe(x, mode, rot):
     _chk(lib().yka_kvx256_probe(_ptr(x), rows, int(mode), int(rot), _ptr(q8) if q8 is not None else None,
                                 _ptr(words) if words is not None else None, _ptr(scales), _ptr(y)))
     return q8, words, scales, y
+
+
+def tb_pack_unpack(blob, x, grp, pos, stride=160):
+    """Trellis row codec round trip (kvx_probe.cu:123-188): x [rows,256] f32 with a group and a position per row ->
+    dict(x = the encoder's reconstruction, words [rows, stride/4] u32, scale [rows] f32, pc [rows] u32, dec = the decoder's rows)."""
+    b = np.frombuffer(bytes(blob), np.uint8)
+    x = np.ascontiguousarray(x, np.float32).reshape(-1, 256)
+    rows = x.shape[0]
+    grp = np.ascontiguousarray(grp, np.int32); pos = np.ascontiguousarray(pos, np.int32)
+    assert grp.shape == (rows,) and pos.shape == (rows,)
+    y = np.empty((rows, 256), np.float32); dec = np.empty((rows, 256), np.float32)
+    pay = np.empty((rows, stride), np.uint8); side = np.empty((rows, 2), np.uint32)
+    _chk(lib().yka_tb_pack_unpack(_ptr(b), b.size, _ptr(x), _ptr(grp), _ptr(pos), rows, int(stride), _ptr(y), _ptr(pay), _ptr(side), _ptr(dec)))
+    return dict(x=y, words=pay.view(np.uint32), scale=side[:, 0].copy().view(np.float32), pc=side[:, 1].copy(), dec=dec)
 
 
 class KvCache:
