@@ -192,6 +192,23 @@ YKA_API int yka_kvx256_probe(const float* x, int rows, int mode, int rot, int8_t
 YKA_API int yka_tb_pack_unpack(const uint8_t* blob, size_t blob_len, const float* x, const int* grp, const int* pos, int rows,
                                int stride, float* y_fq, uint8_t* pay, uint32_t* side, float* y_dec);
 
+/* Switches a handle opened with head_dim 256 (not paged) to trellis-coded rows under the given "KVQP" v1 profile (host
+ * memory; copied).  Replaces the profile loading of the engine (YSKN_TB_PROFILE, engine35.cpp:38-66) and its packed KV
+ * streams (kp / vp / kps / vps of Q35PkArgs, q35_atxpk.hpp:14).  As the reference asks before it keeps packed rows for a
+ * layer (kvqaxpk_packable, kvq_atxpk.hpp:61-72) every group of the handle's layers must be trellis-coded with the same 4
+ * or 5 bits per element, guard position 0 and no projected directions; mean rows are allowed.  Rows are then laid out as
+ * the reference lays them out: payload (kv head * max_ctx + pos) * 32 * bits bytes, one fp32 scale per row in a parallel
+ * array (q35_atxpk3.cuh:196-200).  From then on yka_append / yka_append256_f32 / yka_append_attend encode rows with the
+ * trellis encoder (launch_tb_requant -> launch_tb_fast, q35_kernels.cu:1084-1092) and yka_attend / yka_append_attend
+ * read them (launch_q35_atx_pk); yka_attn_post, the multi-stream pass and the flat-row export / import refuse.
+ * Synchronous; allocates (the only call of the trellis path that does). */
+YKA_API int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len);
+/* bits per element of the handle's trellis-coded rows, 0 if it has no profile */
+YKA_API int yka_kv_profile_bits(const yka_kv* kv);
+/* rows [pos0, pos0 + n) of one layer of a handle with a profile: kw / vw [n_kv_heads][n][8 * bits] payload words,
+ * ks / vs [n_kv_heads][n] scales (host memory).  Test hook; synchronous. */
+YKA_API int yka_kv_export_rows_tb(yka_kv* kv, int layer, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs);
+
 /* Canonical image of rows [pos0, pos0+n) of one layer, independent of the physical layout:
  * kc/vc [n_kv_heads][n][64], ks/vs [n_kv_heads][n][4].  export = device -> host, import = host -> device.
  * (The reference reads its containers back only inside its hooks, e.g. kvx_probe.cu:369.) Synchronous. */

@@ -377,3 +377,20 @@ def tb_decode_rows(blob, grp, words, scale, pc):
         if lib().yko_tb_decode_row(_p(b), int(grp[i]), _p(words[i]), float(scale[i]), int(pc[i]), _p(y[i])) != 0:
             raise IndexError(int(grp[i]))
     return y
+
+
+def tb_attend_f64(k, v, q16, pos, depth=None):
+    """textbook attention in fp64 over decoded rows: k, v [n_kv, rows, 256] fp32 (what tb_decode_rows returns per kv head),
+    q16 [M, n_heads, 256] fp16; row t sees keys [0, pos + depth(t) + 1).  Returns [M, n_heads, 256] fp64."""
+    q = np.asarray(q16, np.float16).astype(np.float64) if np.asarray(q16).dtype != np.uint16 else np.asarray(q16).view(np.float16).astype(np.float64)
+    M, H, Dh = q.shape
+    n_kv = k.shape[0]; G = H // n_kv
+    out = np.zeros((M, H, Dh))
+    for t in range(M):
+        n = pos + (int(depth[t]) if depth is not None else t) + 1
+        for h in range(H):
+            kh = k[h // G, :n].astype(np.float64); vh = v[h // G, :n].astype(np.float64)
+            s = kh @ q[t, h] / np.sqrt(Dh)
+            p = np.exp(s - s.max()); p /= p.sum()
+            out[t, h] = p @ vh
+    return out

@@ -72,3 +72,96 @@ def test_bad_blobs_are_refused(native):
         native.tb_pack_unpack(blob[:-4], y, [0], [0])
     with pytest.raises(native.YkaError, match="stride"):
         native.tb_pack_unpack(blob, y, [0], [0], stride=128)
+
+
+# ---- the cache: trellis-coded rows behind the ordinary entry points ----
+NH, KVH = 24, 4
+
+
+def _kv_rows(seed, n):
+    rng = np.random.default_rng(seed)
+    k = rng.standard_normal((n, KVH, 256)).astype(np.float32)
+    k[:, :, [5, 77, 130, 201]] *= 4
+    v = rng.standard_normal((n, KVH, 256)).astype(np.float32)
+    return k, v
+
+
+def _oracle_rows(oracle, blob, layer, k, v):
+    """rows [n, KVH, 256] -> per kv head: coded rows of K and V as the oracle codes them"""
+    n = k.shape[0]
+    enc = {}
+    for kind, x in ((0, k), (1, v)):
+        for h in range(KVH):
+            g = (layer * KVH + h) * 2 + kind
+            enc[kind, h] = oracle.tb_encode_rows(blob, np.full(n, g, np.int32), np.arange(n, dtype=np.int32), x[:, h])
+            assert enc[kind, h]["coded"].all()
+    return enc
+
+
+@pytest.mark.parametrize("kk,mu", [(5, False), (4, False), (5, True), (4, True)])
+@pytest.mark.parametrize("ctx,M", [(0, 1), (70, 2), (300, 5), (1000, 1), (1500, 16)])
+def test_cache_rows_bit_exact_and_attention_within_the_bars(native, oracle, kk, mu, ctx, M):
+    from tolerances import assert_attn_close
+    layer = 1
+    blob = kvqp.synthetic(layers=2, kk=kk, seed=3 + kk, mu=mu)
+    n = ctx + M
+    k, v = _kv_rows(ctx * 7 + M + kk, n)
+    k16, v16 = k[ctx:].astype(np.float16), v[ctx:].astype(np.float16)
+    k[ctx:] = k16; v[ctx:] = v16                                   # the pass's own rows arrive as fp16
+    q = np.random.default_rng(n).standard_normal((M, NH, 256)).astype(np.float16)
+    max_ctx = ((n + 255) // 256) * 256
+    with native.KvCache(n_layers=2, head_dim=256, max_ctx=max_ctx) as kv:
+        kv.set_profile(blob)
+        assert kv.profile_bits == kk
+        for p in range(0, ctx, 64):
+            m = min(64, ctx - p)
+            kv.append256_f32_host(layer, k[p:p + m], v[p:p + m], p, rotate=False)
+        out = kv.layer_call(layer, q, k16, v16, ctx)
+        kw, ks, vw, vs = kv.export_rows(layer, 0, n)
+    enc = _oracle_rows(oracle, blob, layer, k, v)
+    kd = np.empty((KVH, n, 256), np.float32); vd = np.empty_like(kd)
+    for h in range(KVH):
+        assert np.array_equal(kw[h], enc[0, h]["words"][:, :8 * kk]) and np.array_equal(vw[h], enc[1, h]["words"][:, :8 * kk]), h
+        assert _same(ks[h], enc[0, h]["scale"]) and _same(vs[h], enc[1, h]["scale"])
+        kd[h] = enc[0, h]["x"]; vd[h] = enc[1, h]["x"]
+    assert_attn_close(out, oracle.tb_attend_f64(kd, vd, q, ctx), f"kk={kk} mu={mu} ctx={ctx} M={M}")
+
+
+def test_depth_table_and_split_counts(native, oracle):
+    from tolerances import assert_attn_close
+    blob = kvqp.synthetic(layers=1, kk=5, seed=11)
+    ctx, M = 700, 6
+    k, v = _kv_rows(5, ctx + M)
+    q = np.random.default_rng(6).standard_normal((M, NH, 256)).astype(np.float16)
+    depth = np.array([0, 1, 1, 2, 2, 3], np.uint8)
+    with native.KvCache(head_dim=256, max_ctx=1024) as kv:
+        kv.set_profile(blob)
+        for p in range(0, ctx + M, 64):
+            m = min(64, ctx + M - p)
+            kv.append256_f32_host(0, k[p:p + m], v[p:p + m], p, rotate=False)
+        outs = []
+        for S in (0, 3, 97):
+            kv.set_opt(1, S)
+            outs.append(kv.layer_call(0, q, None, None, ctx, depth=depth))
+    enc = _oracle_rows(oracle, blob, 0, k, v)
+    kd = np.stack([enc[0, h]["x"] for h in range(KVH)]); vd = np.stack([enc[1, h]["x"] for h in range(KVH)])
+    expect = oracle.tb_attend_f64(kd, vd, q, ctx, depth=depth)
+    for o, name in zip(outs, ("default", "3 splits", "97 splits")):
+        assert_attn_close(o, expect, name)
+
+
+def test_profiles_the_packed_cache_cannot_hold_are_refused(native):
+    with native.KvCache(head_dim=256, max_ctx=256) as kv:
+        for kw in (dict(kk=3), dict(kk=5, dirs=1), dict(kk=5, guard=2), dict(kk=5, flat_groups=(0,))):
+            with pytest.raises(native.YkaError, match="packed rows need"):
+                kv.set_profile(kvqp.synthetic(layers=1, **kw))
+        with pytest.raises(native.YkaError, match="cover"):
+            kv.set_profile(kvqp.synthetic(layers=1, kv_heads=2))
+        kv.set_profile(kvqp.synthetic(layers=1, kk=4))
+        with pytest.raises(native.YkaError, match="already"):
+            kv.set_profile(kvqp.synthetic(layers=1, kk=4))
+        with pytest.raises(native.YkaError, match="trellis"):
+            kv.ms_call(np.zeros((1, NH, 256), np.float16), None, None, np.zeros(1, np.int32), np.zeros(1, np.int32))
+    with native.KvCache(max_ctx=256) as kv:
+        with pytest.raises(native.YkaError, match="256"):
+            kv.set_profile(kvqp.synthetic(layers=1))

@@ -4,6 +4,7 @@
 #include "../../include/yka_abi.h"
 #include "yka_internal.h"
 #include <algorithm>
+#include <cmath>
 #include <cstdio>
 #include <cstring>
 #include <stdexcept>
@@ -31,6 +32,19 @@ struct yka_kv {
   int* d_pos = nullptr;            // position used by the host-pointer hooks
   hipStream_t stream = nullptr;    // stream of the host-pointer hooks
   int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0, opt_unrot = 0, opt_ctx_hint = 0;
+  // trellis-coded rows (set by yka_kv_set_profile; head_dim 256 only): rows as the reference lays them out, per layer
+  // [K payload n_kv * max_ctx * stride][V payload][K scales n_kv * max_ctx fp32][V scales]
+  struct Tb {
+    int kb = 0, stride = 0, nm = 0; bool has_mu = false;
+    uint8_t* blob = nullptr; uint16_t* tabs = nullptr; float* gfac = nullptr; float* mu = nullptr;
+    uint8_t* pool = nullptr; size_t layer_bytes = 0, pay_bytes = 0, scl_bytes = 0;
+    uint8_t* scr = nullptr; size_t scr_w_ofs = 0;
+    uint8_t* kpay(int layer) const { return pool + (size_t)layer * layer_bytes; }
+    uint8_t* vpay(int layer) const { return kpay(layer) + pay_bytes; }
+    float* kscl(int layer) const { return reinterpret_cast<float*>(kpay(layer) + 2 * pay_bytes); }
+    float* vscl(int layer) const { return reinterpret_cast<float*>(kpay(layer) + 2 * pay_bytes + scl_bytes); }
+  };
+  Tb* tb = nullptr;
   bool r256() const { return cfg.head_dim == 256; }   // the reference's own rows (attend256.hip); otherwise the 128-channel format
   int D() const { return cfg.head_dim; }
   KvView view(int layer) const {
@@ -90,8 +104,29 @@ void check_rows(const yka_kv* kv, int M) {
   if (M < 1 || M > kv->cfg.max_rows) throw std::runtime_error("M must be in [1, max_rows]");
 }
 
+constexpr int kTbTileTok = 128;     // tokens per launch of the trellis encoder (its scratch holds that many)
+// trellis encoder over the rows of a pass: fp32 rows, or fp16 rows if k32 == nullptr
+void tb_append(yka_kv* kv, int layer, const float* k32, const float* v32, const uint16_t* k16, const uint16_t* v16, int M, const int* d_pos,
+               int rot, hipStream_t st) {
+  const yka_kv::Tb& T = *kv->tb;
+  for (int t0 = 0; t0 < M; t0 += kTbTileTok) {
+    TbEncArgs A{};
+    A.blob = T.blob; A.nm = T.nm; A.has_trellis = 1;
+    A.k32 = k32; A.v32 = v32; A.k16 = k16; A.v16 = v16; A.d_pos = d_pos; A.layer = layer; A.tok0 = t0; A.n_kv = kv->cfg.n_kv_heads;
+    A.max_ctx = kv->cfg.max_ctx; A.rot = rot;
+    A.nrow = std::min(kTbTileTok, M - t0) * 2 * kv->cfg.n_kv_heads;
+    A.scr = T.scr; A.scr_w_ofs = T.scr_w_ofs;
+    A.pay0 = T.kpay(layer); A.pay1 = T.vpay(layer); A.scl0 = T.kscl(layer); A.scl1 = T.vscl(layer); A.stride = T.stride;
+    launch_tb_encode(A, st);
+  }
+}
+void no_trellis(const yka_kv* kv) {
+  if (kv->tb) throw std::runtime_error("this entry point does not work on trellis-coded rows");
+}
+
 void do_append(yka_kv* kv, int layer, const uint16_t* k16, const uint16_t* v16, int M, const int* d_pos, hipStream_t st) {
-  if (kv->r256()) launch_append256(AppendArgs{kv->view(layer), k16, v16, d_pos, M}, st);
+  if (kv->tb) tb_append(kv, layer, nullptr, nullptr, k16, v16, M, d_pos, 0, st);
+  else if (kv->r256()) launch_append256(AppendArgs{kv->view(layer), k16, v16, d_pos, M}, st);
   else launch_append(AppendArgs{kv->view(layer), k16, v16, d_pos, M}, st);
 }
 void need_128(const yka_kv* kv) {
@@ -103,6 +138,23 @@ void need_128(const yka_kv* kv) {
 void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_pos, const uint8_t* depth, uint16_t* out16,
                hipStream_t st, int mode = 0, const uint16_t* k16 = nullptr, const uint16_t* v16 = nullptr) {
   const int NH = kv->cfg.n_heads;
+  if (kv->tb) {
+    // trellis-coded rows: the encoder runs first (two launches), then row tiles of 2 tokens x 6 heads for every width
+    const yka_kv::Tb& T = *kv->tb;
+    if (k16) do_append(kv, layer, k16, v16, M, d_pos, st);
+    const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
+    for (int s0 = 0; s0 < M; s0 += kMaxSlice) {
+      const int Ms = std::min(kMaxSlice, M - s0), tiles = (Ms + 1) / 2;
+      int S = kv->opt_splits_narrow > 0 ? kv->opt_splits_narrow : std::min(512 / (kv->cfg.n_kv_heads * tiles), ((ctx + 31) / 32) / 2);
+      S = std::min(std::max(2, std::min(kMaxSplits, S)), (int)(kWsPairs / (size_t)Ms));
+      const TbAttnArgs A{T.kpay(layer), T.vpay(layer), T.kscl(layer), T.vscl(layer), kv->cfg.max_ctx, kv->cfg.n_kv_heads, T.stride,
+                         T.tabs, T.gfac, T.has_mu ? T.mu : nullptr, layer, q16 + (size_t)s0 * NH * 256, d_pos, depth, Ms, s0, NH, S,
+                         kv->pm, kv->pl, kv->pacc16};
+      launch_attend_tb(A, T.kb, st);
+      if (mode != 2) launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, kv->opt_unrot}, st);
+    }
+    return;
+  }
   if (kv->r256()) {
     // 256-channel rows: append first; rows of at most 2 tokens (or option key 3) run on row tiles of 2 tokens x 6 heads,
     // two workgroups per CU; wider slices on 128-row workgroups of 8 waves, one per CU
@@ -226,6 +278,11 @@ void yka_kv_close(yka_kv* kv) {
   (void)hipSetDevice(kv->cfg.device);
   (void)hipDeviceSynchronize();
   if (kv->stream) (void)hipStreamDestroy(kv->stream);
+  if (kv->tb) {
+    (void)hipFree(kv->tb->blob); (void)hipFree(kv->tb->tabs); (void)hipFree(kv->tb->gfac); (void)hipFree(kv->tb->mu); (void)hipFree(kv->tb->pool);
+    (void)hipFree(kv->tb->scr);
+    delete kv->tb;
+  }
   (void)hipFree(kv->pool); (void)hipFree(kv->tables); (void)hipFree(kv->pm); (void)hipFree(kv->pl); (void)hipFree(kv->pacc16); (void)hipFree(kv->d_pos);
   delete kv;
 }
@@ -293,7 +350,7 @@ int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16
 int yka_append_attend_ms(yka_kv* kv, const uint16_t* d_q16, const uint16_t* d_k16, const uint16_t* d_v16, int M,
                          const int* d_row_pos, const int* d_row_slot, uint16_t* d_out16, void* hip_stream) {
   YKA_TRY
-  on_device(kv); check_rows(kv, M);
+  on_device(kv); no_trellis(kv); check_rows(kv, M);
   if (!d_q16 || !d_row_pos || !d_row_slot || !d_out16) throw std::runtime_error("null pointer");
   if ((d_k16 == nullptr) != (d_v16 == nullptr)) throw std::runtime_error("new K and V rows come together or not at all");
   do_attend_ms(kv, d_q16, d_k16, d_v16, M, d_row_pos, d_row_slot, d_out16, (hipStream_t)hip_stream);
@@ -304,7 +361,7 @@ int yka_append_attend_ms(yka_kv* kv, const uint16_t* d_q16, const uint16_t* d_k1
 int yka_ms_call_host(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, const int32_t* row_pos,
                      const int32_t* row_slot, uint16_t* out16) {
   YKA_TRY
-  on_device(kv); check_rows(kv, M);
+  on_device(kv); no_trellis(kv); check_rows(kv, M);
   if (!q16 || !row_pos || !row_slot || !out16) throw std::runtime_error("null pointer");
   if ((k16 == nullptr) != (v16 == nullptr)) throw std::runtime_error("new K and V rows come together or not at all");
   const size_t nq = (size_t)M * kv->cfg.n_heads * kv->D(), nk = (size_t)M * kv->cfg.n_kv_heads * kv->D();
@@ -346,7 +403,7 @@ static void check_post(const yka_kv* kv, const yka_post_params* P) {
 int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float* d_xk, const float* d_xv, int M, const int* d_pos,
                   const yka_post_params* P, uint16_t* d_q16, void* hip_stream) {
   YKA_TRY
-  on_device(kv); check_layer(kv, layer); check_rows(kv, M); check_post(kv, P);
+  on_device(kv); no_trellis(kv); check_layer(kv, layer); check_rows(kv, M); check_post(kv, P);
   if (!d_xq || !d_xk || !d_xv || !d_pos || !d_q16) throw std::runtime_error("null pointer");
   const PostArgs A{kv->view(layer), d_xq, d_xk, d_xv, M, kv->cfg.n_heads, d_pos, P->d_qn_w16, P->d_kn_w16, P->eps,
                    P->d_rope, P->rope_dims, P->rope_rows, P->rotate != 0, d_q16};
@@ -359,7 +416,7 @@ int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, 
                        const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope, int rope_dims,
                        int rope_rows, int rotate, uint16_t* q16) {
   YKA_TRY
-  on_device(kv); check_layer(kv, layer); check_rows(kv, M);
+  on_device(kv); no_trellis(kv); check_layer(kv, layer); check_rows(kv, M);
   if (!xq || !xk || !xv || !qn_w16 || !kn_w16 || !q16) throw std::runtime_error("null pointer");
   if (pos < 0 || (long long)pos + M > kv->cfg.max_ctx) throw std::runtime_error("rows outside the container");
   const int kD = kv->D();                          // 128 or 256 channels per head
@@ -471,6 +528,89 @@ int yka_tb_pack_unpack(const uint8_t* blob, size_t blob_len, const float* x, con
   YKA_CATCH_INT
 }
 
+static uint16_t int_to_f16_bits(int v) {               // |v| <= 2048: exact
+  if (v == 0) return 0;
+  const unsigned a = (unsigned)(v < 0 ? -v : v);
+  int e = 31 - __builtin_clz(a);                       // a = 1.xxx * 2^e, e <= 11
+  const unsigned mant = (a << (10 - e)) & 0x3ffu;      // e <= 10 for a < 2048; a == 2048: e = 11, mant 0
+  return (uint16_t)((v < 0 ? 0x8000u : 0u) | ((unsigned)(e + 15) << 10) | (e <= 10 ? mant : 0u));
+}
+
+int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
+  YKA_TRY
+  on_device(kv);
+  if (!kv->r256()) throw std::runtime_error("trellis-coded rows need a handle opened with head_dim 256");
+  if (kv->cfg.paged) throw std::runtime_error("trellis-coded rows are not available in paged mode");
+  if (kv->tb) throw std::runtime_error("the handle already has a profile");
+  const TbInfo I = tb_check_blob(blob, blob_len);
+  const int n_kv = kv->cfg.n_kv_heads, need = kv->cfg.n_layers * n_kv * 2;
+  if (I.kv_heads != n_kv || I.ngrp < need) throw std::runtime_error("the profile does not cover the layers and kv heads of the handle");
+  auto u16 = [&](size_t o) { return (unsigned)blob[o] | ((unsigned)blob[o + 1] << 8); };
+  auto u32 = [&](size_t o) { return u16(o) | (u16(o + 2) << 16); };
+  const size_t off_t = u32(36), off_g = u32(40);
+  // what the reference asks of a layer before it keeps packed rows for it (kvqaxpk_packable, src/kvq_atxpk.hpp:61-72)
+  int kb = 0; bool has_mu = false;
+  std::vector<uint16_t> tabs((size_t)need * 256); std::vector<float> gfac(need), mu((size_t)need * 256, 0.f);
+  for (int g = 0; g < need; ++g) {
+    const size_t go = u32(off_g + 4 * (size_t)g);
+    const int mode = blob[go], kk = blob[go + 1], tix = blob[go + 2], guard = blob[go + 3], m = blob[go + 4];
+    if (mode != 0 || (kk != 4 && kk != 5) || guard != 0 || m != 0)
+      throw std::runtime_error("packed rows need every group trellis-coded with 4 or 5 bits, no guard position and no projected directions");
+    if (kb && kk != kb) throw std::runtime_error("packed rows need the same bits per element in every group");
+    kb = kk;
+    const size_t to = u32(off_t + 4 * (size_t)tix);
+    float gain; std::memcpy(&gain, blob + to + 4, 4);
+    if (!(gain > 0.f) || gain > 1e6f) throw std::runtime_error("profile blob: table gain must be positive and finite");
+    gfac[g] = 0.00390625f * gain;
+    for (int st = 0; st < 256; ++st) tabs[(size_t)g * 256 + st] = int_to_f16_bits((int)(short)u16(to + 12 + 2 * (size_t)st));
+    if (blob[go + 5]) {
+      has_mu = true;
+      for (int d = 0; d < 256; ++d) {
+        const unsigned h = u16(go + 8 + 2 * (size_t)d), sg = h >> 15, e = (h >> 10) & 31u, mm = h & 1023u;
+        float v = e == 0 ? std::ldexp((float)mm, -24) : std::ldexp((float)(mm | 1024u), (int)e - 25);
+        if (e == 31) throw std::runtime_error("profile blob: mean row is not finite");
+        mu[(size_t)g * 256 + d] = sg ? -v : v;
+      }
+    }
+  }
+  yka_kv::Tb* T = new yka_kv::Tb();
+  kv->tb = T;                                          // freed by yka_kv_close whatever happens below
+  T->kb = kb; T->stride = 32 * kb; T->nm = I.nm; T->has_mu = has_mu;
+  const size_t rows = (size_t)n_kv * kv->cfg.max_ctx;
+  T->pay_bytes = rows * T->stride; T->scl_bytes = rows * 4; T->layer_bytes = 2 * T->pay_bytes + 2 * T->scl_bytes;
+  const size_t jobs = (size_t)kTbTileTok * 2 * n_kv * I.nm;
+  T->scr_w_ofs = jobs * 256;
+  HIPCHK(hipMalloc((void**)&T->blob, blob_len)); HIPCHK(hipMemcpy(T->blob, blob, blob_len, hipMemcpyHostToDevice));
+  HIPCHK(hipMalloc((void**)&T->tabs, tabs.size() * 2)); HIPCHK(hipMemcpy(T->tabs, tabs.data(), tabs.size() * 2, hipMemcpyHostToDevice));
+  HIPCHK(hipMalloc((void**)&T->gfac, gfac.size() * 4)); HIPCHK(hipMemcpy(T->gfac, gfac.data(), gfac.size() * 4, hipMemcpyHostToDevice));
+  HIPCHK(hipMalloc((void**)&T->mu, mu.size() * 4)); HIPCHK(hipMemcpy(T->mu, mu.data(), mu.size() * 4, hipMemcpyHostToDevice));
+  HIPCHK(hipMalloc((void**)&T->pool, T->layer_bytes * kv->cfg.n_layers));
+  HIPCHK(hipMemset(T->pool, 0, T->layer_bytes * kv->cfg.n_layers));     // unwritten rows: state 0 everywhere, scale 0
+  HIPCHK(hipMalloc((void**)&T->scr, T->scr_w_ofs + jobs * 32));
+  HIPCHK(hipDeviceSynchronize());
+  YKA_CATCH_INT
+}
+
+int yka_kv_profile_bits(const yka_kv* kv) { return kv && kv->tb ? kv->tb->kb : 0; }
+
+int yka_kv_export_rows_tb(yka_kv* kv, int layer, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer);
+  if (!kv->tb) throw std::runtime_error("the handle has no profile");
+  if (pos0 < 0 || n < 1 || (long long)pos0 + n > kv->cfg.max_ctx) throw std::runtime_error("row range outside the container");
+  if (!kw || !ks || !vw || !vs) throw std::runtime_error("null pointer");
+  const yka_kv::Tb& T = *kv->tb;
+  HIPCHK(hipDeviceSynchronize());
+  for (int h = 0; h < kv->cfg.n_kv_heads; ++h) {
+    const size_t row = (size_t)h * kv->cfg.max_ctx + pos0, nb = (size_t)n * T.stride;
+    HIPCHK(hipMemcpy(reinterpret_cast<uint8_t*>(kw) + (size_t)h * nb, T.kpay(layer) + row * T.stride, nb, hipMemcpyDeviceToHost));
+    HIPCHK(hipMemcpy(reinterpret_cast<uint8_t*>(vw) + (size_t)h * nb, T.vpay(layer) + row * T.stride, nb, hipMemcpyDeviceToHost));
+    HIPCHK(hipMemcpy(ks + (size_t)h * n, T.kscl(layer) + row, (size_t)n * 4, hipMemcpyDeviceToHost));
+    HIPCHK(hipMemcpy(vs + (size_t)h * n, T.vscl(layer) + row, (size_t)n * 4, hipMemcpyDeviceToHost));
+  }
+  YKA_CATCH_INT
+}
+
 static void check_range(const yka_kv* kv, int pos0, int n) {
   if (pos0 < 0 || n < 1 || (long long)pos0 + n > kv->cfg.max_ctx) throw std::runtime_error("row range outside the container");
 }
@@ -516,7 +656,8 @@ int yka_append256_f32(yka_kv* kv, int layer, const float* d_k32, const float* d_
   if (!d_k32 || !d_v32 || !d_pos) throw std::runtime_error("null pointer");
   AppendArgs A{kv->view(layer), nullptr, nullptr, d_pos, M};
   A.k32 = d_k32; A.v32 = d_v32; A.rot = rotate != 0;
-  launch_append256(A, (hipStream_t)hip_stream);
+  if (kv->tb) tb_append(kv, layer, d_k32, d_v32, nullptr, nullptr, M, d_pos, rotate != 0, (hipStream_t)hip_stream);
+  else launch_append256(A, (hipStream_t)hip_stream);
   HIPCHK(hipGetLastError());
   YKA_CATCH_INT
 }
@@ -543,7 +684,8 @@ int yka_append256_f32_host(yka_kv* kv, int layer, const float* k32, const float*
   launch_set_int(kv->d_pos, pos, kv->stream);
   AppendArgs A{kv->view(layer), nullptr, nullptr, kv->d_pos, M};
   A.k32 = dk.as<float>(); A.v32 = dv.as<float>(); A.rot = rotate != 0;
-  launch_append256(A, kv->stream);
+  if (kv->tb) tb_append(kv, layer, dk.as<float>(), dv.as<float>(), nullptr, nullptr, M, kv->d_pos, rotate != 0, kv->stream);
+  else launch_append256(A, kv->stream);
   HIPCHK(hipGetLastError());
   HIPCHK(hipStreamSynchronize(kv->stream));
   YKA_CATCH_INT
@@ -592,6 +734,7 @@ int yka_attn_out256_host(const uint16_t* y16, const uint16_t* gate16, const int8
 int yka_kv_export_rows256(yka_kv* kv, int layer, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs) {
   YKA_TRY
   on_device(kv); check_layer(kv, layer); check_range(kv, pos0, n);
+  no_trellis(kv);
   if (!kv->r256()) throw std::runtime_error("this entry point exists for head_dim 256 only");
   if (!kw || !ks || !vw || !vs) throw std::runtime_error("null pointer");
   const size_t rows = (size_t)kv->cfg.n_kv_heads * n;
@@ -608,6 +751,7 @@ int yka_kv_export_rows256(yka_kv* kv, int layer, int pos0, int n, uint32_t* kw, 
 int yka_kv_import_rows256(yka_kv* kv, int layer, int pos0, int n, const uint32_t* kw, const float* ks, const uint32_t* vw, const float* vs) {
   YKA_TRY
   on_device(kv); check_layer(kv, layer); check_range(kv, pos0, n);
+  no_trellis(kv);
   if (!kv->r256()) throw std::runtime_error("this entry point exists for head_dim 256 only");
   if (!kw || !ks || !vw || !vs) throw std::runtime_error("null pointer");
   const size_t rows = (size_t)kv->cfg.n_kv_heads * n;
@@ -644,6 +788,8 @@ int yka_kv_replicate_layer(yka_kv* kv, int src) {
     if (l == src) continue;
     HIPCHK(hipMemcpy(kv->pool + (size_t)l * kv->layer_bytes, kv->pool + (size_t)src * kv->layer_bytes, kv->layer_bytes, hipMemcpyDeviceToDevice));
     if (kv->tables) HIPCHK(hipMemcpy(kv->tables + (size_t)l * kv->n_pages, kv->tables + (size_t)src * kv->n_pages, (size_t)kv->n_pages * 4, hipMemcpyDeviceToDevice));
+    // trellis-coded rows are copied as they are: meaningful only if both layers' groups share tables and mean rows
+    if (kv->tb) HIPCHK(hipMemcpy(kv->tb->kpay(l), kv->tb->kpay(src), kv->tb->layer_bytes, hipMemcpyDeviceToDevice));
   }
   HIPCHK(hipDeviceSynchronize());
   YKA_CATCH_INT

@@ -1,0 +1,248 @@
+// Split-KV attention over trellis-coded rows (the reference's KV4 / KV5 packed streams), gfx950, wave64, MFMA 16x16x32 f16.
+//   reference: launch_q35_atx_pk (src/q35_atxpk.hpp:14-17; decode helpers src/q35_atxpk.cu:70-106, scalar form
+//   tba_attention_kernel, src/kvq_attn.cuh:120-310).  Rows live as the reference lays them out: payload
+//   (kvh * max_ctx + pos) * stride bytes, one fp32 scale per row in a parallel array (src/q35_atxpk3.cuh:196-200).
+// A row is 4 chunks of 64 elements; element e of a chunk decodes to table[state] * scale with state = the last 8 bits of
+// the chunk's MSB-first stream up to the end of field e.  What is specific to this GPU:
+//   * the tile geometry of the 256-channel flat kernel (attend256.hip): a wave owns 32 keys, lane (i, g) holds key i's
+//     chunk g for the scores - so a lane decodes a whole chunk from its own 8 or 10 words, no neighbour needed - and
+//     the 8-channel block i + 16 hh of the 8 tokens whose probabilities it receives for O^T += V^T P^T;
+//   * the table holds the reference's integers (|value| <= 1100, exact in fp16), 512 bytes per table in LDS; the
+//     factor gain / 256 and the row scale are applied in fp32 to the MFMA's sums (K) or ride on the probability and
+//     the final accumulator (V), so no table value is rounded (the reference rounds its table to bf16);
+//   * states come from the words by one funnel shift with a compile-time distance each; the table read is one 16-bit
+//     LDS gather per element - the cost of this format (the flat kernel builds its operands with two ALU operations
+//     per 4 elements);
+//   * a mean row of K shifts every score of a query row by the same q.mu and cancels in the softmax: it is not added.
+//     A mean row of V is added to the normalised partial (the probabilities of a split sum to one).
+#include "yka_internal.h"
+#include <hip/hip_fp16.h>
+
+namespace yka {
+namespace {
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr int kD2 = 256;
+
+__device__ __forceinline__ uint32_t funnel(uint32_t hi, uint32_t lo, uint32_t sh) { return __builtin_amdgcn_alignbit(hi, lo, sh); }   // (hi:lo) >> sh
+__device__ __forceinline__ _Float16 lut(const uint16_t* tab, uint32_t state) {
+  return __builtin_bit_cast(_Float16, *reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(tab) + 2u * (state & 255u)));
+}
+
+// 8 consecutive elements q0 .. q0 + 7 (q0 a compile-time multiple of 8) of a chunk held as NW = 2 KB words
+template <int KB, int Q0>
+__device__ __forceinline__ h8 chunk_vals(const uint32_t* w, const uint16_t* tab) {
+  h8 v;
+#pragma unroll
+  for (int el = 0; el < 8; ++el) {
+    const int end = KB * (Q0 + el + 1), j = (end - 1) >> 5, r = 31 - ((end - 1) & 31);
+    const uint32_t st = r == 0 ? w[j] : funnel(j > 0 ? w[j - 1] : 0u, w[j], (uint32_t)r);
+    v[el] = lut(tab, st);
+  }
+  return v;
+}
+
+template <int KB>
+__global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
+  constexpr int NW = 2 * KB;                         // words per chunk
+  __shared__ float s_m[4][16], s_l[4][16];
+  __shared__ float s_acc[4][16][kD2 + 4];
+  __shared__ uint16_t s_tabK[256], s_tabV[256];
+  const int split = blockIdx.x, kvh = blockIdx.y, rt = blockIdx.z;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
+  const int gK = (A.layer * A.n_kv + kvh) * 2, gV = gK + 1;
+  s_tabK[threadIdx.x] = A.tabs[(size_t)gK * 256 + threadIdx.x];
+  s_tabV[threadIdx.x] = A.tabs[(size_t)gV * 256 + threadIdx.x];
+  const int pos = *A.d_pos;
+  const int tl = 2 * rt + i / kG;
+  const bool vrow = i < 2 * kG && tl < A.M;
+  const int head = kvh * kG + i % kG;
+  int len = 0;
+  if (vrow) { const int tg = A.tok0 + tl; len = min(pos + (A.depth ? (int)A.depth[tg] : tg) + 1, A.max_ctx); }
+  int maxlen = len, minlen = vrow ? len : 0x7fffffff;
+#pragma unroll
+  for (int o = 1; o < 16; o <<= 1) { maxlen = max(maxlen, __shfl_xor(maxlen, o, 64)); minlen = min(minlen, __shfl_xor(minlen, o, 64)); }
+  maxlen = __builtin_amdgcn_readfirstlane(maxlen); minlen = __builtin_amdgcn_readfirstlane(minlen);
+  const int ntiles = (maxlen + 31) >> 5;
+  const int s_used = min(A.S, max(1, ntiles >> 1));
+  if (split >= s_used) {                             // the "no keys" marker; the combiner does not read such rows
+    const int j = threadIdx.x, tj = 2 * rt + j / kG;
+    if (j < 2 * kG && tj < A.M) {
+      const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
+      A.pm[p] = -1e30f; A.pl[p] = 0.f;
+    }
+    return;
+  }
+  __syncthreads();                                   // tables
+  const int tps = (ntiles + s_used - 1) / s_used;
+  const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
+
+  h8 qf[8];                                          // k-step t: channels 64 g + 8 t .. + 7 of row i
+  {
+    const uint16_t* qrow = A.q16 + ((size_t)tl * A.n_heads + head) * kD2 + 64 * g;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) qf[t] = __builtin_bit_cast(h8, vrow ? *reinterpret_cast<const uint4*>(qrow + 8 * t) : make_uint4(0, 0, 0, 0));
+  }
+  const float sc_log2 = kLog2e * 0.0625f * A.gfac[gK];      // log2(e) / sqrt(256) x gain / 256 of the K table
+  const size_t row0 = (size_t)kvh * A.max_ctx;
+  const uint8_t* const kbase = A.kpay + row0 * A.stride + (uint32_t)g * (4u * NW);
+  const float* const kscl = A.kscl + row0;
+  const float* const vscl = A.vscl + row0;
+  // V: lane (i, g) needs, for hh = 0, 1, the 8 elements of block cb = i + 16 hh of 8 tokens.  Inside its chunk the block
+  // starts at bit KB * 8 * c (c = cb & 7); the window that also holds the 8 - KB bits before it (zero at a chunk start)
+  // starts at bit s0 = KB * 8 * c - (8 - KB), i.e. in word w0 = floor(s0 / 32) at offset off - never 0 for KB 4 or 5.
+  const int c8 = i & 7;
+  const int s0 = KB * 8 * c8 - (8 - KB);
+  const int w0 = s0 >> 5;                            // -1 for the first block of a chunk
+  const uint32_t sh = 32u - (uint32_t)(s0 & 31);
+  uint32_t voff[2];
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh) voff[hh] = (uint32_t)((i + 16 * hh) >> 3) * (4u * NW) + 4u * (uint32_t)max(w0, 0);
+  const bool first = c8 == 0;
+  const bool three = KB == 5 && w0 + 2 < NW;         // a third word exists (and is needed only for c = 4)
+
+  float m_run = -1e30f, l_run = 0.f;
+  f4 o[16];
+#pragma unroll
+  for (int b = 0; b < 16; ++b) o[b] = f4{0.f, 0.f, 0.f, 0.f};
+
+  for (int T = tile0 + wave; T < tile1; T += 4) {
+    const int t0 = T << 5;
+    // ---- loads: K chunk g of keys t0 + 16 kt + i; scales of the 4 keys whose scores this lane receives; V windows ----
+    uint32_t kw[2][NW];
+    f4 ksc[2], vsc[2];
+    uint32_t vw[2][8][3];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      const uint8_t* kr = kbase + (size_t)(t0 + 16 * kt + i) * A.stride;
+      if (KB == 4) {
+        const uint4 a = *reinterpret_cast<const uint4*>(kr), b = *reinterpret_cast<const uint4*>(kr + 16);
+        kw[kt][0] = a.x; kw[kt][1] = a.y; kw[kt][2] = a.z; kw[kt][3] = a.w; kw[kt][4] = b.x; kw[kt][5] = b.y; kw[kt][6] = b.z; kw[kt][7] = b.w;
+      } else {
+#pragma unroll
+        for (int p = 0; p < NW / 2; ++p) { const uint2 a = *reinterpret_cast<const uint2*>(kr + 8 * p); kw[kt][2 * p] = a.x; kw[kt][2 * p + 1] = a.y; }
+      }
+      ksc[kt] = *reinterpret_cast<const f4*>(kscl + t0 + 16 * kt + 4 * g);
+      vsc[kt] = *reinterpret_cast<const f4*>(vscl + t0 + 16 * kt + 4 * g);
+    }
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int tok = t0 + 16 * (e >> 2) + 4 * g + (e & 3);
+        const uint8_t* vr = A.vpay + (row0 + tok) * A.stride + voff[hh];
+        const uint32_t a = *reinterpret_cast<const uint32_t*>(vr);
+        const uint32_t b = first ? 0u : *reinterpret_cast<const uint32_t*>(vr + 4);
+        uint32_t c = 0u;
+        if (KB == 5) c = *reinterpret_cast<const uint32_t*>(vr + (first ? 4 : (three ? 8 : 4)));
+        // first block of a chunk: the window's word before the chunk is zero, then words 0 and 1
+        vw[hh][e][0] = first ? 0u : a;
+        vw[hh][e][1] = first ? a : b;
+        vw[hh][e][2] = KB == 5 ? ((first || three) ? c : 0u) : 0u;
+      }
+    const bool need_mask = t0 + 32 > minlen;
+    // ---- scores ----
+    float s[8];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) {
+      f4 part = f4{0.f, 0.f, 0.f, 0.f};
+      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 0>(kw[kt], s_tabK), qf[0], part, 0, 0, 0);
+      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 8>(kw[kt], s_tabK), qf[1], part, 0, 0, 0);
+      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 16>(kw[kt], s_tabK), qf[2], part, 0, 0, 0);
+      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 24>(kw[kt], s_tabK), qf[3], part, 0, 0, 0);
+      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 32>(kw[kt], s_tabK), qf[4], part, 0, 0, 0);
+      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 40>(kw[kt], s_tabK), qf[5], part, 0, 0, 0);
+      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 48>(kw[kt], s_tabK), qf[6], part, 0, 0, 0);
+      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 56>(kw[kt], s_tabK), qf[7], part, 0, 0, 0);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s[4 * kt + r] = part[r] * ksc[kt][r];          // key t0 + 16 kt + 4 g + r against row i
+    }
+    if (need_mask) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) { const int key = t0 + 16 * (e >> 2) + 4 * g + (e & 3); s[e] = key < len ? s[e] : -INFINITY; }
+    }
+    // ---- online softmax (one running maximum per row, shared by its 4 lane groups) ----
+    float tmax = s[0];
+#pragma unroll
+    for (int e = 1; e < 8; ++e) tmax = fmaxf(tmax, s[e]);
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax * sc_log2);          // the table's gain is positive (checked when the profile is set)
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    const bool first_tile = m_run < -1e29f;
+    m_run = m_new;
+    if (__any(alpha != 1.f && !first_tile)) {
+      l_run *= alpha;
+#pragma unroll
+      for (int b = 0; b < 16; ++b) { o[b][0] *= alpha; o[b][1] *= alpha; o[b][2] *= alpha; o[b][3] *= alpha; }
+    }
+    h8 pf;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[e], sc_log2, -m_new));
+      l_run += p;
+      pf[e] = (_Float16)(p * vsc[e >> 2][e & 3]);            // the V scale of the key rides on its probability
+    }
+    // ---- O^T += V^T P^T: accumulator hh * 8 + el covers channel 8 (i + 16 hh) + el ----
+#pragma unroll
+    for (int hh = 0; hh < 2; ++hh) {
+      uint32_t y0[8], y1[8];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        y0[e] = funnel(vw[hh][e][0], vw[hh][e][1], sh);
+        y1[e] = funnel(vw[hh][e][1], vw[hh][e][2], sh);
+      }
+#pragma unroll
+      for (int el = 0; el < 8; ++el) {
+        h8 vf;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const int lo = KB * el;                              // the state of element el = bits [lo, lo + 8) of y0:y1
+          const uint32_t st = lo + 8 <= 32 ? y0[e] >> (24 - lo) : funnel(y0[e], y1[e], (uint32_t)(56 - lo));
+          vf[e] = lut(s_tabV, st);
+        }
+        o[hh * 8 + el] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[hh * 8 + el], 0, 0, 0);
+      }
+    }
+  }
+  // ---- merge the 4 waves, write one partial per (row, split): o[hh*8 + el][r] = channel 8 (4g + r + 16 hh) + el of row i ----
+  l_run += __shfl_xor(l_run, 16, 64);
+  l_run += __shfl_xor(l_run, 32, 64);
+  if (g == 0) { s_m[wave][i] = m_run; s_l[wave][i] = l_run; }
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+    for (int el = 0; el < 8; ++el)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s_acc[wave][i][8 * (4 * g + r + 16 * hh) + el] = o[hh * 8 + el][r];
+  __syncthreads();
+  const float gv = A.gfac[gV];
+  for (int idx = threadIdx.x; idx < 2 * kG * kD2; idx += 256) {
+    const int j = idx >> 8, d = idx & (kD2 - 1);
+    const int tj = 2 * rt + j / kG;
+    if (tj >= A.M) continue;
+    const float m0 = s_m[0][j], m1 = s_m[1][j], m2 = s_m[2][j], m3 = s_m[3][j];
+    const float M2 = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
+    const float w0 = exp2f(m0 - M2), w1 = exp2f(m1 - M2), w2 = exp2f(m2 - M2), w3 = exp2f(m3 - M2);
+    const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
+    const float L = w0 * s_l[0][j] + w1 * s_l[1][j] + w2 * s_l[2][j] + w3 * s_l[3][j];
+    const float acc = w0 * s_acc[0][j][d] + w1 * s_acc[1][j][d] + w2 * s_acc[2][j][d] + w3 * s_acc[3][j][d];
+    float y = L > 0.f ? acc * gv / L : 0.f;
+    if (A.mu && L > 0.f) y += A.mu[(size_t)gV * 256 + d];
+    A.pacc16[p * kD2 + d] = __half_as_ushort(__float2half_rn(y));
+    if (d == 0) { A.pm[p] = M2; A.pl[p] = L; }
+  }
+}
+
+}  // namespace
+
+void launch_attend_tb(const TbAttnArgs& A, int kb, hipStream_t st) {
+  const dim3 grid(A.S, A.n_kv, (A.M + 1) / 2);
+  if (kb == 4) hipLaunchKernelGGL(attend_tb_kernel<4>, grid, dim3(256), 0, st, A);
+  else hipLaunchKernelGGL(attend_tb_kernel<5>, grid, dim3(256), 0, st, A);
+}
+
+}  // namespace yka

@@ -23,7 +23,9 @@ __device__ __forceinline__ unsigned tb_u16(const uint8_t* p) { return (unsigned)
 __device__ __forceinline__ unsigned tb_u32(const uint8_t* p) { return tb_u16(p) | (tb_u16(p + 2) << 16); }
 __device__ __forceinline__ float tb_f32(const uint8_t* p) { return __uint_as_float(tb_u32(p)); }
 __device__ __forceinline__ float tb_h2f(unsigned h) { return __half2float(__ushort_as_half((unsigned short)h)); }
-__device__ __forceinline__ float tb_f16r(float v) { return __half2float(__float2half_rn(v)); }
+// fp32 value -> nearest fp16 -> fp32.  The empty asm keeps the compiler from merging the operation that produced v with the
+// conversion into one mixed-precision instruction, which would skip the fp32 rounding the reference performs in between
+__device__ __forceinline__ float tb_f16r(float v) { asm volatile("" : "+v"(v)); return __half2float(__float2half_rn(v)); }
 __device__ __forceinline__ float tb_cdec(int ci, float gain) { return __fmul_rn(__fmul_rn((float)ci, 0.00390625f), gain); }
 
 struct Group { int nm, mode, kk, tix, guard, m, has_mu; unsigned go, off_m, off_t; bool ok; };
@@ -73,7 +75,8 @@ __device__ __forceinline__ Row tb_row(const TbEncArgs& A, int rj, int d, float* 
     const int tok = rj / (2 * A.n_kv), rem = rj - tok * 2 * A.n_kv;
     R.kind = rem / A.n_kv; R.kvh = rem - R.kind * A.n_kv;
     R.pos = *A.d_pos + A.tok0 + tok; R.g = (A.layer * A.n_kv + R.kvh) * 2 + R.kind;
-    R.y = (R.kind ? A.v32 : A.k32)[((size_t)(A.tok0 + tok) * A.n_kv + R.kvh) * 256 + d];
+    const size_t e = ((size_t)(A.tok0 + tok) * A.n_kv + R.kvh) * 256 + d;
+    R.y = A.k32 ? (R.kind ? A.v32 : A.k32)[e] : __half2float(__ushort_as_half((R.kind ? A.v16 : A.k16)[e]));
     R.out = (size_t)R.kvh * A.max_ctx + (size_t)max(0, min(R.pos, A.max_ctx - 1));
   }
   if (A.rot) R.y = rotate256(R.y, buf, false);

@@ -83,13 +83,23 @@ struct PostArgs {
 // pay0 (K) / pay1 (V) + (kvh * max_ctx + pos) * stride and its scale to scl0 / scl1 [kvh * max_ctx + pos].
 struct TbEncArgs {
   const uint8_t* blob; int nm; int has_trellis;
-  const float* k32; const float* v32; const int* d_pos; int layer, tok0, n_kv, max_ctx, rot;
+  const float* k32; const float* v32; const uint16_t* k16; const uint16_t* v16;   // cache form: fp32 rows, or fp16 rows if k32 == nullptr
+  const int* d_pos; int layer, tok0, n_kv, max_ctx, rot;
   const float* yin; const int* grp; const int* pos; int row0;
   float* yout; uint32_t* side; int* coded;
   int nrow;
   uint8_t* scr; size_t scr_w_ofs;     // scratch: states [nrow * nm][256] bytes, then at scr_w_ofs error sums [nrow * nm][8] fp32
   uint8_t* pay0; uint8_t* pay1; float* scl0; float* scl1; int stride;
 };
+// attention over trellis-coded rows (attend_tb.hip).  tabs [groups][256]: the tables' integers as fp16; gfac [groups]:
+// gain / 256; mu [groups][256] fp32 mean rows (zero rows where a group has none) or nullptr if no group has one
+struct TbAttnArgs {
+  const uint8_t* kpay; const uint8_t* vpay; const float* kscl; const float* vscl; int max_ctx, n_kv, stride;
+  const uint16_t* tabs; const float* gfac; const float* mu; int layer;
+  const uint16_t* q16; const int* d_pos; const uint8_t* depth; int M, tok0, n_heads, S;
+  float* pm; float* pl; uint16_t* pacc16;
+};
+void launch_attend_tb(const TbAttnArgs&, int kb, hipStream_t);
 void launch_tb_encode(const TbEncArgs&, hipStream_t);
 void launch_tb_unpack(const uint8_t* blob, const int* grp, const int* pos, const uint8_t* pay, const uint32_t* side, int stride, const float* yin,
                       float* y, int rows, hipStream_t);

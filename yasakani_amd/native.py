@@ -54,6 +54,9 @@ def _load():
         "yka_kvx256_probe": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_attn_post": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
         "yka_tb_pack_unpack": (i32, [vp, C.c_size_t, vp, vp, vp, i32, i32, vp, vp, vp, vp]),
+        "yka_kv_set_profile": (i32, [vp, vp, C.c_size_t]),
+        "yka_kv_profile_bits": (i32, [vp]),
+        "yka_kv_export_rows_tb": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_kv_export_rows256": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_append256_f32": (i32, [vp, i32, vp, vp, i32, vp, i32, vp]),
         "yka_attn_out256": (i32, [vp, vp, vp, i32, i32, vp, vp, vp]),
@@ -83,7 +86,7 @@ def _load():
 
 
 EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "yka_set_opt", "yka_kv_set_page_table",
-           "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kvx256_probe", "yka_tb_pack_unpack", "yka_attn_post", "yka_append_attend_ms", "yka_ms_call_host",
+           "yka_append", "yka_attend", "yka_append_attend", "yka_codec_probe", "yka_kvx256_probe", "yka_tb_pack_unpack", "yka_kv_set_profile", "yka_kv_profile_bits", "yka_kv_export_rows_tb", "yka_attn_post", "yka_append_attend_ms", "yka_ms_call_host",
            "yka_attn_post_host", "yka_kv_export_rows", "yka_kv_export_rows256", "yka_kv_import_rows256",
            "yka_attn_out256", "yka_attn_out256_host", "yka_append256_f32", "yka_rotate_q256", "yka_append256_f32_host", "yka_rotate_q256_host",
            "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
@@ -271,9 +274,21 @@ class KvCache:
     def append_attend(self, layer, d_q16, d_k16, d_v16, M, d_pos, d_out16, d_depth=None, stream=0):
         _chk(lib().yka_append_attend(self._h, layer, d_q16, d_k16, d_v16, M, d_pos, d_depth, d_out16, stream))
 
+    def set_profile(self, blob):
+        """switch a head_dim-256 handle to trellis-coded rows under a KVQP profile blob (see yasakani_amd.kvqp)"""
+        b = np.frombuffer(bytes(blob), np.uint8)
+        _chk(lib().yka_kv_set_profile(self._h, _ptr(b), b.size))
+        self.profile_bits = lib().yka_kv_profile_bits(self._h)
+
     # -- hooks: host arrays --
     def export_rows(self, layer, pos0, n):
         kvh = self.cfg.n_kv_heads
+        bits = getattr(self, "profile_bits", 0)
+        if bits:                            # trellis-coded rows: payload words [kvh, n, 8 * bits] u32, row scales [kvh, n] f32
+            kw = np.empty((kvh, n, 8 * bits), np.uint32); vw = np.empty_like(kw)
+            ks = np.empty((kvh, n), np.float32); vs = np.empty_like(ks)
+            _chk(lib().yka_kv_export_rows_tb(self._h, layer, pos0, n, _ptr(kw), _ptr(ks), _ptr(vw), _ptr(vs)))
+            return kw, ks, vw, vs
         if self.cfg.head_dim == 256:        # words [kvh, n, 32] u32 and row scales [kvh, n] f32
             kw = np.empty((kvh, n, 32), np.uint32); vw = np.empty_like(kw)
             ks = np.empty((kvh, n), np.float32); vs = np.empty_like(ks)
