@@ -137,6 +137,38 @@ def r256_figures(native, ctx=32768, L=16):
     return out
 
 
+def trellis_figures(native, ctx=32768, L=16, bits=5):
+    """Trellis-coded rows (the reference's KV5 / KV4 packed streams) under a synthetic profile of the production shape:
+    4 x 2 x (32 * bits + 4) bytes per token per layer.  One layer call = trellis encoder for the new rows (two launches) +
+    attention on row tiles of 2 tokens + combine; `encode_us` is what the encoder adds to a layer call."""
+    from yasakani_amd import kvqp
+    rng = np.random.default_rng(500 + bits)
+    D2 = 256
+    k = rng.standard_normal((4096 + 64, KVH, D2)).astype(np.float16)
+    v = rng.standard_normal((4096 + 64, KVH, D2)).astype(np.float16)
+    q = rng.standard_normal((64, NH, D2)).astype(np.float16)
+    kv = native.KvCache(n_layers=L, head_dim=D2, max_ctx=ctx + 256, max_rows=64)
+    kv.set_profile(kvqp.synthetic(layers=L, kk=bits, seed=7))
+    for p in range(0, ctx, 64):                       # 4096 distinct rows tiled over the context
+        s0 = p % 4096
+        kv.append_host(0, k[s0:s0 + 64], v[s0:s0 + 64], p)
+    kv.replicate_layer(0)                             # the synthetic profile gives every layer the same tables
+    out = {}
+    token_bytes = KVH * 2 * (32 * bits + 4)
+    for rows in (1, 16, 64):
+        ms, _ = kv.bench(q[:rows], k[4096:4096 + rows], v[4096:4096 + rows], ctx, mode=0, use_graph=True, reps=10)
+        us = float(np.median(ms)) * 1e3 / L
+        ms1, _ = kv.bench(q[:rows], None, None, ctx, mode=1, use_graph=True, reps=10)
+        ms2, _ = kv.bench(q[:rows], None, None, ctx, mode=2, use_graph=True, reps=10)
+        k_us = float(np.median(ms2)) * 1e3 / L
+        by = ctx * token_bytes + rows * (2 * token_bytes + 2 * KVH * D2 * 2 + 2 * NH * D2 * 2)
+        out[f"rows_{rows}"] = {"us_per_layer": us, "encode_us": us - float(np.median(ms1)) * 1e3 / L, "kernel_us": k_us,
+                               "value_GBs": by / (us * 1e-6) / 1e9, "kernel_hbm_frac": by / (k_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
+                               "kernel_tflops": 4.0 * rows * NH * D2 * ctx / (k_us * 1e-6) / 1e12}
+    kv.close()
+    return out
+
+
 def big_configs(native):
     """Secondary figures for the two large configurations: a 2048-row prefill chunk on 131072 cached tokens (cut into
     64-row slices inside the library) and decode / verify-64 on 262144 tokens in shuffled 256-token pages."""
@@ -275,6 +307,8 @@ def main():
                     help="run only the multi-stream (batched decode) passes and print their figures (for profiling that kernel)")
     ap.add_argument("--r256-only", action="store_true",
                     help="run only the passes over the reference's 256-channel rows and print their figures (for profiling those kernels)")
+    ap.add_argument("--trellis-only", action="store_true",
+                    help="run only the passes over trellis-coded rows (5 and 4 bits per element) and print their figures")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three device-to-device copies of 256 MiB (a kernel of known traffic, for scaling FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -288,6 +322,9 @@ def main():
 
     if args.r256_only:
         print(json.dumps({"reference_rows_head_dim_256": r256_figures(native, args.ctx)}))
+        return
+    if args.trellis_only:
+        print(json.dumps({"trellis_rows": {f"bits_{b}": trellis_figures(native, args.ctx, bits=b) for b in (5, 4)}}))
         return
     ctx, M, L = args.ctx, args.rows, args.layers
     max_ctx = ((ctx + 64 + 255) // 256) * 256
@@ -369,6 +406,7 @@ def main():
     if not args.no_extra:
         line["other_configs"] = big_configs(native)
         line["reference_rows_head_dim_256"] = r256_figures(native)
+        line["trellis_rows"] = {"bits_5": trellis_figures(native)}
     print(json.dumps(line))
 
 

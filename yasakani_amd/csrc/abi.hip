@@ -36,7 +36,7 @@ struct yka_kv {
   // [K payload n_kv * max_ctx * stride][V payload][K scales n_kv * max_ctx fp32][V scales]
   struct Tb {
     int kb = 0, stride = 0, nm = 0; bool has_mu = false;
-    uint8_t* blob = nullptr; uint16_t* tabs = nullptr; float* gfac = nullptr; float* mu = nullptr;
+    uint8_t* blob = nullptr; uint32_t* pairs = nullptr; float* gfac = nullptr; float* mu = nullptr;
     uint8_t* pool = nullptr; size_t layer_bytes = 0, pay_bytes = 0, scl_bytes = 0;
     uint8_t* scr = nullptr; size_t scr_w_ofs = 0;
     uint8_t* kpay(int layer) const { return pool + (size_t)layer * layer_bytes; }
@@ -148,7 +148,7 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
       int S = kv->opt_splits_narrow > 0 ? kv->opt_splits_narrow : std::min(512 / (kv->cfg.n_kv_heads * tiles), ((ctx + 31) / 32) / 2);
       S = std::min(std::max(2, std::min(kMaxSplits, S)), (int)(kWsPairs / (size_t)Ms));
       const TbAttnArgs A{T.kpay(layer), T.vpay(layer), T.kscl(layer), T.vscl(layer), kv->cfg.max_ctx, kv->cfg.n_kv_heads, T.stride,
-                         T.tabs, T.gfac, T.has_mu ? T.mu : nullptr, layer, q16 + (size_t)s0 * NH * 256, d_pos, depth, Ms, s0, NH, S,
+                         T.pairs, T.gfac, T.has_mu ? T.mu : nullptr, layer, q16 + (size_t)s0 * NH * 256, d_pos, depth, Ms, s0, NH, S,
                          kv->pm, kv->pl, kv->pacc16};
       launch_attend_tb(A, T.kb, st);
       if (mode != 2) launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, kv->opt_unrot}, st);
@@ -279,7 +279,7 @@ void yka_kv_close(yka_kv* kv) {
   (void)hipDeviceSynchronize();
   if (kv->stream) (void)hipStreamDestroy(kv->stream);
   if (kv->tb) {
-    (void)hipFree(kv->tb->blob); (void)hipFree(kv->tb->tabs); (void)hipFree(kv->tb->gfac); (void)hipFree(kv->tb->mu); (void)hipFree(kv->tb->pool);
+    (void)hipFree(kv->tb->blob); (void)hipFree(kv->tb->pairs); (void)hipFree(kv->tb->gfac); (void)hipFree(kv->tb->mu); (void)hipFree(kv->tb->pool);
     (void)hipFree(kv->tb->scr);
     delete kv->tb;
   }
@@ -551,6 +551,7 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
   // what the reference asks of a layer before it keeps packed rows for it (kvqaxpk_packable, src/kvq_atxpk.hpp:61-72)
   int kb = 0; bool has_mu = false;
   std::vector<uint16_t> tabs((size_t)need * 256); std::vector<float> gfac(need), mu((size_t)need * 256, 0.f);
+  std::vector<uint32_t> pairs;
   for (int g = 0; g < need; ++g) {
     const size_t go = u32(off_g + 4 * (size_t)g);
     const int mode = blob[go], kk = blob[go + 1], tix = blob[go + 2], guard = blob[go + 3], m = blob[go + 4];
@@ -573,6 +574,12 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
       }
     }
   }
+  // pair tables: entry i decodes two consecutive elements from the 8 + kb stream bits that end with the second one
+  const size_t npair = (size_t)1 << (8 + kb);
+  pairs.resize((size_t)need * npair);
+  for (int g = 0; g < need; ++g)
+    for (size_t i = 0; i < npair; ++i)
+      pairs[(size_t)g * npair + i] = (uint32_t)tabs[(size_t)g * 256 + ((i >> kb) & 255)] | ((uint32_t)tabs[(size_t)g * 256 + (i & 255)] << 16);
   yka_kv::Tb* T = new yka_kv::Tb();
   kv->tb = T;                                          // freed by yka_kv_close whatever happens below
   T->kb = kb; T->stride = 32 * kb; T->nm = I.nm; T->has_mu = has_mu;
@@ -581,7 +588,7 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
   const size_t jobs = (size_t)kTbTileTok * 2 * n_kv * I.nm;
   T->scr_w_ofs = jobs * 256;
   HIPCHK(hipMalloc((void**)&T->blob, blob_len)); HIPCHK(hipMemcpy(T->blob, blob, blob_len, hipMemcpyHostToDevice));
-  HIPCHK(hipMalloc((void**)&T->tabs, tabs.size() * 2)); HIPCHK(hipMemcpy(T->tabs, tabs.data(), tabs.size() * 2, hipMemcpyHostToDevice));
+  HIPCHK(hipMalloc((void**)&T->pairs, pairs.size() * 4)); HIPCHK(hipMemcpy(T->pairs, pairs.data(), pairs.size() * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMalloc((void**)&T->gfac, gfac.size() * 4)); HIPCHK(hipMemcpy(T->gfac, gfac.data(), gfac.size() * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMalloc((void**)&T->mu, mu.size() * 4)); HIPCHK(hipMemcpy(T->mu, mu.data(), mu.size() * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMalloc((void**)&T->pool, T->layer_bytes * kv->cfg.n_layers));

@@ -7,12 +7,14 @@
 //   * the tile geometry of the 256-channel flat kernel (attend256.hip): a wave owns 32 keys, lane (i, g) holds key i's
 //     chunk g for the scores - so a lane decodes a whole chunk from its own 8 or 10 words, no neighbour needed - and
 //     the 8-channel block i + 16 hh of the 8 tokens whose probabilities it receives for O^T += V^T P^T;
-//   * the table holds the reference's integers (|value| <= 1100, exact in fp16), 512 bytes per table in LDS; the
-//     factor gain / 256 and the row scale are applied in fp32 to the MFMA's sums (K) or ride on the probability and
-//     the final accumulator (V), so no table value is rounded (the reference rounds its table to bf16);
-//   * states come from the words by one funnel shift with a compile-time distance each; the table read is one 16-bit
-//     LDS gather per element - the cost of this format (the flat kernel builds its operands with two ALU operations
-//     per 4 elements);
+//   * the table holds the reference's integers (|value| <= 1100, exact in fp16); the factor gain / 256 and the row scale
+//     are applied in fp32 to the MFMA's sums (K) or ride on the probability and the final accumulator (V), so no table
+//     value is rounded (the reference rounds its table to bf16);
+//   * one LDS read decodes TWO elements: the states of elements e and e + 1 are both contained in the 8 + kb stream bits
+//     that end with field e + 1, so a table of 2^(8 + kb) entries of two fp16 values (16 KB at 4 bits, 32 KB at 5, per
+//     table; built when the profile is set, copied into LDS by every workgroup, in the space the wave merge uses
+//     afterwards) turns one funnel shift, one mask and one 32-bit gather into a finished pair of MFMA operand halves.
+//     The reference keeps a 4096-entry pair table for 4-bit rows (src/q35_atxpk3.cuh:66-78);
 //   * a mean row of K shifts every score of a query row by the same q.mu and cancels in the softmax: it is not added.
 //     A mean row of V is added to the normalised partial (the probabilities of a split sum to one).
 #include "yka_internal.h"
@@ -27,35 +29,41 @@ constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kD2 = 256;
 
 __device__ __forceinline__ uint32_t funnel(uint32_t hi, uint32_t lo, uint32_t sh) { return __builtin_amdgcn_alignbit(hi, lo, sh); }   // (hi:lo) >> sh
-__device__ __forceinline__ _Float16 lut(const uint16_t* tab, uint32_t state) {
-  return __builtin_bit_cast(_Float16, *reinterpret_cast<const uint16_t*>(reinterpret_cast<const uint8_t*>(tab) + 2u * (state & 255u)));
+// byte offset (entry index x 4) of the pair entry for the KB + 8 stream bits that end at bit `endbit` (exclusive) of a chunk
+// held as words w[]; bits before the chunk start count as zero.  Everything but w is a compile-time constant.
+template <int KB>
+__device__ __forceinline__ uint32_t pair_offset(const uint32_t* w, int endbit) {
+  constexpr uint32_t mask4 = ((1u << (8 + KB)) - 1u) << 2;
+  const int j = (endbit - 1) >> 5, r = 31 - ((endbit - 1) & 31);            // word of the last bit, bits to its right
+  const uint32_t hi = j > 0 ? w[j - 1] : 0u;
+  if (r >= 2) return (r == 2 ? w[j] : funnel(hi, w[j], (uint32_t)(r - 2))) & mask4;
+  return (funnel(hi, w[j], (uint32_t)r) << 2) & mask4;
 }
+__device__ __forceinline__ uint32_t pair_at(const uint8_t* tab, uint32_t off) { return *reinterpret_cast<const uint32_t*>(tab + off); }
 
-// 8 consecutive elements q0 .. q0 + 7 (q0 a compile-time multiple of 8) of a chunk held as NW = 2 KB words
+// 8 consecutive elements Q0 .. Q0 + 7 (Q0 a compile-time multiple of 8) of a chunk held as 2 KB words
 template <int KB, int Q0>
-__device__ __forceinline__ h8 chunk_vals(const uint32_t* w, const uint16_t* tab) {
-  h8 v;
+__device__ __forceinline__ h8 chunk_vals(const uint32_t* w, const uint8_t* tab) {
+  uint32_t d[4];
 #pragma unroll
-  for (int el = 0; el < 8; ++el) {
-    const int end = KB * (Q0 + el + 1), j = (end - 1) >> 5, r = 31 - ((end - 1) & 31);
-    const uint32_t st = r == 0 ? w[j] : funnel(j > 0 ? w[j - 1] : 0u, w[j], (uint32_t)r);
-    v[el] = lut(tab, st);
-  }
-  return v;
+  for (int p = 0; p < 4; ++p) d[p] = pair_at(tab, pair_offset<KB>(w, KB * (Q0 + 2 * p + 2)));
+  return __builtin_bit_cast(h8, uint4{d[0], d[1], d[2], d[3]});
 }
 
 template <int KB>
 __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
   constexpr int NW = 2 * KB;                         // words per chunk
+  constexpr int kTabBytes = 4 << (8 + KB);           // one pair table
+  constexpr int kAccBytes = 4 * 16 * (kD2 + 4) * 4;
   __shared__ float s_m[4][16], s_l[4][16];
-  __shared__ float s_acc[4][16][kD2 + 4];
-  __shared__ uint16_t s_tabK[256], s_tabV[256];
+  __shared__ __align__(16) uint8_t s_buf[kAccBytes > 2 * kTabBytes ? kAccBytes : 2 * kTabBytes];   // pair tables, then the wave merge
+  float (*s_acc)[16][kD2 + 4] = reinterpret_cast<float (*)[16][kD2 + 4]>(s_buf);
+  const uint8_t* const s_tabK = s_buf;
+  const uint8_t* const s_tabV = s_buf + kTabBytes;
   const int split = blockIdx.x, kvh = blockIdx.y, rt = blockIdx.z;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
   const int gK = (A.layer * A.n_kv + kvh) * 2, gV = gK + 1;
-  s_tabK[threadIdx.x] = A.tabs[(size_t)gK * 256 + threadIdx.x];
-  s_tabV[threadIdx.x] = A.tabs[(size_t)gV * 256 + threadIdx.x];
   const int pos = *A.d_pos;
   const int tl = 2 * rt + i / kG;
   const bool vrow = i < 2 * kG && tl < A.M;
@@ -76,7 +84,14 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
     }
     return;
   }
-  __syncthreads();                                   // tables
+  {                                                  // the K and V pair tables of this kv head: global (L2) -> LDS
+    const uint4* srcK = reinterpret_cast<const uint4*>(A.pairs + (size_t)gK * (kTabBytes / 4));
+    const uint4* srcV = reinterpret_cast<const uint4*>(A.pairs + (size_t)gV * (kTabBytes / 4));
+    uint4* dst = reinterpret_cast<uint4*>(s_buf);
+#pragma unroll 4
+    for (int x = threadIdx.x; x < kTabBytes / 16; x += 256) { dst[x] = srcK[x]; dst[kTabBytes / 16 + x] = srcV[x]; }
+  }
+  __syncthreads();
   const int tps = (ntiles + s_used - 1) / s_used;
   const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
 
@@ -98,11 +113,15 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
   const int s0 = KB * 8 * c8 - (8 - KB);
   const int w0 = s0 >> 5;                            // -1 for the first block of a chunk
   const uint32_t sh = 32u - (uint32_t)(s0 & 31);
-  uint32_t voff[2];
+  // byte offsets, inside a V row, of the window's three words for hh = 0, 1.  The word before a chunk start is read as
+  // word 0 and masked to zero; a third word past the chunk end is not needed by any state and is read as the last word.
+  uint32_t vo0[2], vo1[2], vo2[2];
 #pragma unroll
-  for (int hh = 0; hh < 2; ++hh) voff[hh] = (uint32_t)((i + 16 * hh) >> 3) * (4u * NW) + 4u * (uint32_t)max(w0, 0);
-  const bool first = c8 == 0;
-  const bool three = KB == 5 && w0 + 2 < NW;         // a third word exists (and is needed only for c = 4)
+  for (int hh = 0; hh < 2; ++hh) {
+    const uint32_t base = (uint32_t)((i + 16 * hh) >> 3) * (4u * NW);
+    vo0[hh] = base + 4u * (uint32_t)max(w0, 0); vo1[hh] = base + 4u * (uint32_t)(w0 + 1); vo2[hh] = base + 4u * (uint32_t)min(w0 + 2, NW - 1);
+  }
+  const uint32_t keep0 = c8 == 0 ? 0u : 0xffffffffu;
 
   float m_run = -1e30f, l_run = 0.f;
   f4 o[16];
@@ -133,15 +152,10 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int tok = t0 + 16 * (e >> 2) + 4 * g + (e & 3);
-        const uint8_t* vr = A.vpay + (row0 + tok) * A.stride + voff[hh];
-        const uint32_t a = *reinterpret_cast<const uint32_t*>(vr);
-        const uint32_t b = first ? 0u : *reinterpret_cast<const uint32_t*>(vr + 4);
-        uint32_t c = 0u;
-        if (KB == 5) c = *reinterpret_cast<const uint32_t*>(vr + (first ? 4 : (three ? 8 : 4)));
-        // first block of a chunk: the window's word before the chunk is zero, then words 0 and 1
-        vw[hh][e][0] = first ? 0u : a;
-        vw[hh][e][1] = first ? a : b;
-        vw[hh][e][2] = KB == 5 ? ((first || three) ? c : 0u) : 0u;
+        const uint8_t* vr = A.vpay + (row0 + tok) * A.stride;
+        vw[hh][e][0] = *reinterpret_cast<const uint32_t*>(vr + vo0[hh]) & keep0;
+        vw[hh][e][1] = *reinterpret_cast<const uint32_t*>(vr + vo1[hh]);
+        vw[hh][e][2] = KB == 5 ? *reinterpret_cast<const uint32_t*>(vr + vo2[hh]) : 0u;
       }
     const bool need_mask = t0 + 32 > minlen;
     // ---- scores ----
@@ -196,18 +210,30 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
         y1[e] = funnel(vw[hh][e][1], vw[hh][e][2], sh);
       }
 #pragma unroll
-      for (int el = 0; el < 8; ++el) {
-        h8 vf;
+      for (int el = 0; el < 8; el += 2) {                      // elements el, el + 1 = bits [KB el, KB el + KB + 8) of y0:y1
+        constexpr uint32_t mask4 = ((1u << (8 + KB)) - 1u) << 2;
+        const int q = KB * el + 8 + KB;                        // end of the pair's bits
+        uint32_t pr[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-          const int lo = KB * el;                              // the state of element el = bits [lo, lo + 8) of y0:y1
-          const uint32_t st = lo + 8 <= 32 ? y0[e] >> (24 - lo) : funnel(y0[e], y1[e], (uint32_t)(56 - lo));
-          vf[e] = lut(s_tabV, st);
+          uint32_t off;
+          if (q <= 30) off = (y0[e] >> (30 - q)) & mask4;
+          else if (q <= 32) off = (y0[e] << (q - 30)) & mask4;
+          else off = funnel(y0[e], y1[e], (uint32_t)(62 - q)) & mask4;
+          pr[e] = pair_at(s_tabV, off);
         }
-        o[hh * 8 + el] = __builtin_amdgcn_mfma_f32_16x16x32_f16(vf, pf, o[hh * 8 + el], 0, 0, 0);
+        uint32_t a[4], b[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          a[t] = __builtin_amdgcn_perm(pr[2 * t + 1], pr[2 * t], 0x05040100u);     // element el of tokens 2t, 2t + 1
+          b[t] = __builtin_amdgcn_perm(pr[2 * t + 1], pr[2 * t], 0x07060302u);     // element el + 1
+        }
+        o[hh * 8 + el] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, uint4{a[0], a[1], a[2], a[3]}), pf, o[hh * 8 + el], 0, 0, 0);
+        o[hh * 8 + el + 1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, uint4{b[0], b[1], b[2], b[3]}), pf, o[hh * 8 + el + 1], 0, 0, 0);
       }
     }
   }
+  __syncthreads();                                   // every wave is done with the tables: their space now holds the merge
   // ---- merge the 4 waves, write one partial per (row, split): o[hh*8 + el][r] = channel 8 (4g + r + 16 hh) + el of row i ----
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);

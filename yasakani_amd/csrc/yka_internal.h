@@ -91,11 +91,12 @@ struct TbEncArgs {
   uint8_t* scr; size_t scr_w_ofs;     // scratch: states [nrow * nm][256] bytes, then at scr_w_ofs error sums [nrow * nm][8] fp32
   uint8_t* pay0; uint8_t* pay1; float* scl0; float* scl1; int stride;
 };
-// attention over trellis-coded rows (attend_tb.hip).  tabs [groups][256]: the tables' integers as fp16; gfac [groups]:
+// attention over trellis-coded rows (attend_tb.hip).  pairs [groups][2^(8 + kb)]: entry i = the table's integers, as two
+// fp16 values, of the states (i >> kb) & 255 and i & 255 (two consecutive elements from 8 + kb stream bits); gfac [groups]:
 // gain / 256; mu [groups][256] fp32 mean rows (zero rows where a group has none) or nullptr if no group has one
 struct TbAttnArgs {
   const uint8_t* kpay; const uint8_t* vpay; const float* kscl; const float* vscl; int max_ctx, n_kv, stride;
-  const uint16_t* tabs; const float* gfac; const float* mu; int layer;
+  const uint32_t* pairs; const float* gfac; const float* mu; int layer;
   const uint16_t* q16; const int* d_pos; const uint8_t* depth; int M, tok0, n_heads, S;
   float* pm; float* pl; uint16_t* pacc16;
 };
