@@ -113,14 +113,13 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
   const int s0 = KB * 8 * c8 - (8 - KB);
   const int w0 = s0 >> 5;                            // -1 for the first block of a chunk
   const uint32_t sh = 32u - (uint32_t)(s0 & 31);
-  // byte offsets, inside a V row, of the window's three words for hh = 0, 1.  The word before a chunk start is read as
-  // word 0 and masked to zero; a third word past the chunk end is not needed by any state and is read as the last word.
-  uint32_t vo0[2], vo1[2], vo2[2];
+  // byte offset, inside a V row, of the window's first word for hh = 0, 1.  For the first block of a chunk that is the
+  // word BEFORE the chunk (w0 = -1): it is loaded like any other (the word before row 0 of the V payload is the last
+  // word of the K payload, the word after a row's last chunk is the next row or the scale array: same allocation) and
+  // masked to zero; words past the window's last needed bit are never used.
+  uint32_t vo[2];
 #pragma unroll
-  for (int hh = 0; hh < 2; ++hh) {
-    const uint32_t base = (uint32_t)((i + 16 * hh) >> 3) * (4u * NW);
-    vo0[hh] = base + 4u * (uint32_t)max(w0, 0); vo1[hh] = base + 4u * (uint32_t)(w0 + 1); vo2[hh] = base + 4u * (uint32_t)min(w0 + 2, NW - 1);
-  }
+  for (int hh = 0; hh < 2; ++hh) vo[hh] = (uint32_t)((i + 16 * hh) >> 3) * (4u * NW) + 4u * (uint32_t)w0;
   const uint32_t keep0 = c8 == 0 ? 0u : 0xffffffffu;
 
   float m_run = -1e30f, l_run = 0.f;
@@ -128,12 +127,12 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
 #pragma unroll
   for (int b = 0; b < 16; ++b) o[b] = f4{0.f, 0.f, 0.f, 0.f};
 
-  for (int T = tile0 + wave; T < tile1; T += 4) {
+  // K words and K scales of a tile are requested one tile ahead (right after the scores of the tile before have consumed
+  // the registers they land in); V words at the top of their own tile, a whole score phase before their first use
+  uint32_t kw[2][NW];
+  f4 ksc[2];
+  auto load_k = [&](int T) __attribute__((always_inline)) {
     const int t0 = T << 5;
-    // ---- loads: K chunk g of keys t0 + 16 kt + i; scales of the 4 keys whose scores this lane receives; V windows ----
-    uint32_t kw[2][NW];
-    f4 ksc[2], vsc[2];
-    uint32_t vw[2][8][3];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
       const uint8_t* kr = kbase + (size_t)(t0 + 16 * kt + i) * A.stride;
@@ -141,21 +140,29 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
         const uint4 a = *reinterpret_cast<const uint4*>(kr), b = *reinterpret_cast<const uint4*>(kr + 16);
         kw[kt][0] = a.x; kw[kt][1] = a.y; kw[kt][2] = a.z; kw[kt][3] = a.w; kw[kt][4] = b.x; kw[kt][5] = b.y; kw[kt][6] = b.z; kw[kt][7] = b.w;
       } else {
-#pragma unroll
-        for (int p = 0; p < NW / 2; ++p) { const uint2 a = *reinterpret_cast<const uint2*>(kr + 8 * p); kw[kt][2 * p] = a.x; kw[kt][2 * p + 1] = a.y; }
+        __builtin_memcpy(&kw[kt][0], __builtin_assume_aligned(kr, 8), 16);          // 40-byte chunks: 8-byte aligned
+        __builtin_memcpy(&kw[kt][4], __builtin_assume_aligned(kr + 16, 8), 16);
+        __builtin_memcpy(&kw[kt][8], __builtin_assume_aligned(kr + 32, 8), 8);
       }
       ksc[kt] = *reinterpret_cast<const f4*>(kscl + t0 + 16 * kt + 4 * g);
-      vsc[kt] = *reinterpret_cast<const f4*>(vscl + t0 + 16 * kt + 4 * g);
     }
+  };
+  if (tile0 + wave < tile1) load_k(tile0 + wave);
+  for (int T = tile0 + wave; T < tile1; T += 4) {
+    const int t0 = T << 5;
+    f4 vsc[2];
+    uint32_t vw[2][8][3];
+#pragma unroll
+    for (int kt = 0; kt < 2; ++kt) vsc[kt] = *reinterpret_cast<const f4*>(vscl + t0 + 16 * kt + 4 * g);
 #pragma unroll
     for (int hh = 0; hh < 2; ++hh)
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int tok = t0 + 16 * (e >> 2) + 4 * g + (e & 3);
         const uint8_t* vr = A.vpay + (row0 + tok) * A.stride;
-        vw[hh][e][0] = *reinterpret_cast<const uint32_t*>(vr + vo0[hh]) & keep0;
-        vw[hh][e][1] = *reinterpret_cast<const uint32_t*>(vr + vo1[hh]);
-        vw[hh][e][2] = KB == 5 ? *reinterpret_cast<const uint32_t*>(vr + vo2[hh]) : 0u;
+        vw[hh][e][2] = 0u;
+        __builtin_memcpy(&vw[hh][e][0], __builtin_assume_aligned(vr + (int32_t)vo[hh], 4), KB == 5 ? 12 : 8);
+        vw[hh][e][0] &= keep0;
       }
     const bool need_mask = t0 + 32 > minlen;
     // ---- scores ----
@@ -174,6 +181,7 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) s[4 * kt + r] = part[r] * ksc[kt][r];          // key t0 + 16 kt + 4 g + r against row i
     }
+    if (T + 4 < tile1) load_k(T + 4);
     if (need_mask) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) { const int key = t0 + 16 * (e >> 2) + 4 * g + (e & 3); s[e] = key < len ? s[e] : -INFINITY; }
