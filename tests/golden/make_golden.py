@@ -6,7 +6,7 @@ comes from the reference: the fixtures freeze the oracle's outputs on small seed
 has been pinned by tests/test_oracle_*.py), so that (i) a later change of the oracle is noticed and (ii) the GPU
 tests can compare against committed data.
 
-    python tests/golden/make_golden.py        # rewrites codec_v1.npz, attention_v1.npz, row256_v1.npz, post_v1.npz and post256_v1.npz
+    python tests/golden/make_golden.py        # rewrites codec_v1.npz, attention_v1.npz, row256_v1.npz, post_v1.npz, post256_v1.npz and trellis_v1.npz
 """
 import os
 import sys
@@ -124,11 +124,32 @@ def post256_fixture():
     np.savez_compressed(os.path.join(HERE, "post256_v1.npz"), **out)
 
 
+def trellis_fixture():
+    """Trellis-coded rows under two synthetic profiles (5 bits with mean rows and two directions; 4 bits plain): the blob,
+    the rows, and what the oracle codes them to.  The blob is stored so that the fixture does not depend on the generator of
+    synthetic profiles staying as it is."""
+    from yasakani_amd import kvqp
+    rng = np.random.default_rng(20261129)
+    out = {}
+    for name, blob in (("a", kvqp.synthetic(layers=1, kk=5, seed=41, mu=True, dirs=2, flat_groups=(6,))), ("b", kvqp.synthetic(layers=1, kk=4, seed=42))):
+        n = 48
+        y = (rng.standard_normal((n, 256)) * rng.uniform(0.1, 5, (n, 1))).astype(np.float32)
+        y[:, [5, 77, 130, 201]] *= 8
+        y[2] = 0
+        grp = (np.arange(n) % 8).astype(np.int32); pos = np.arange(n, dtype=np.int32)
+        enc = yko.tb_encode_rows(blob, grp, pos, y)
+        out.update({f"{name}.blob": np.frombuffer(blob, np.uint8), f"{name}.y": y, f"{name}.grp": grp, f"{name}.pos": pos,
+                    f"{name}.words": enc["words"], f"{name}.scale": enc["scale"], f"{name}.pc": enc["pc"], f"{name}.x": enc["x"],
+                    f"{name}.best_mi": enc["best_mi"]})
+    np.savez_compressed(os.path.join(HERE, "trellis_v1.npz"), **out)
+
+
 if __name__ == "__main__":
     codec_fixture()
     attention_fixture()
     row256_fixture()
     post_fixture()
     post256_fixture()
-    for f in ("codec_v1.npz", "attention_v1.npz", "row256_v1.npz", "post_v1.npz", "post256_v1.npz"):
+    trellis_fixture()
+    for f in ("codec_v1.npz", "attention_v1.npz", "row256_v1.npz", "post_v1.npz", "post256_v1.npz", "trellis_v1.npz"):
         print(f, os.path.getsize(os.path.join(HERE, f)), "bytes")

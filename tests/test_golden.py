@@ -138,3 +138,25 @@ def test_gpu_reproduces_post256_fixture(native):
         assert (q16.view(np.uint16) == g[f"r{rot}.q16"]).all()
         assert (kw == g[f"r{rot}.kw"]).all() and (vw == g[f"r{rot}.vw"]).all()
         assert (ks.view(np.uint32) == g[f"r{rot}.ks"].view(np.uint32)).all() and (vs.view(np.uint32) == g[f"r{rot}.vs"].view(np.uint32)).all()
+
+
+def _check_trellis(code, g, name):
+    enc = code(g[f"{name}.blob"].tobytes(), g[f"{name}.grp"], g[f"{name}.pos"], g[f"{name}.y"])
+    assert (enc["words"][:, :40] == g[f"{name}.words"][:, :40]).all()
+    assert (enc["scale"].view(np.uint32) == g[f"{name}.scale"].view(np.uint32)).all() and (enc["pc"] == g[f"{name}.pc"]).all()
+    assert (enc["x"].view(np.uint32) == g[f"{name}.x"].view(np.uint32)).all()
+    return enc
+
+
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_oracle_reproduces_trellis_fixture(oracle, name):
+    enc = _check_trellis(lambda b, grp, pos, y: oracle.tb_encode_rows(b, grp, pos, y), _load("trellis_v1.npz"), name)
+    assert (enc["best_mi"] == _load("trellis_v1.npz")[f"{name}.best_mi"]).all()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_gpu_reproduces_trellis_fixture(native, name):
+    g = _load("trellis_v1.npz")
+    enc = _check_trellis(lambda b, grp, pos, y: native.tb_pack_unpack(b, y, grp, pos), g, name)
+    assert (enc["dec"].view(np.uint32) == g[f"{name}.x"].view(np.uint32)).all()
