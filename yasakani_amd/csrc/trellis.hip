@@ -9,8 +9,9 @@
 // ONE wave; lane l holds the costs of states l, l + 64, l + 128, l + 192.  The predecessors of state d are the states
 // p with p mod U == d >> kk (U = 256 >> kk), and 64 is a multiple of U, so all four states of a lane feed the same
 // group u = l mod U: the minimum of a group is a per-lane minimum of 4 followed by a butterfly over the lane bits above
-// log2(U) - 3 exchanges for 5-bit fields, 2 for 4-bit fields - with no barrier and no cost array in LDS.  The smallest
-// predecessor among equal costs is found by a second butterfly on the candidate indices.  Back-pointers (one per group
+// log2(U) - 3 exchanges for 5-bit fields, 2 for 4-bit fields, done with a row rotation and the row / half swap
+// instructions of gfx950 - with no barrier, no cost array in LDS and no LDS round trip.  The smallest predecessor among
+// equal costs is found by a second butterfly on the candidate indices.  Back-pointers (one per group
 // and step) go to a 2 KB LDS block private to the wave; one lane walks them back.
 #include "yka_internal.h"
 #include "rot256_device.h"
@@ -100,31 +101,47 @@ __device__ __forceinline__ Pre tb_pre(float* red, const uint8_t* b, const Group&
   return Q;
 }
 
+// min over the lane pair (l, l ^ O) without an LDS round trip: a row rotation for O = 8, the gfx950 row / half swaps for
+// O = 16 and 32 (after swapping a register with a copy of itself the two results hold, in every lane, the values of the
+// lane and of its partner)
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+template <int O>
+__device__ __forceinline__ int pair_min(int v) {
+  if constexpr (O == 8) return min(v, __builtin_amdgcn_update_dpp(v, v, 0x128, 0xf, 0xf, false));      // row_ror:8
+  else if constexpr (O == 16) { const u32x2 r = __builtin_amdgcn_permlane16_swap((unsigned)v, (unsigned)v, false, false); return min((int)r[0], (int)r[1]); }
+  else { const u32x2 r = __builtin_amdgcn_permlane32_swap((unsigned)v, (unsigned)v, false, false); return min((int)r[0], (int)r[1]); }
+}
+template <int U>
+__device__ __forceinline__ int group_min(int v) {       // min over the lanes congruent modulo U (U = 8, 16, 32)
+  if constexpr (U <= 8) v = pair_min<8>(v);
+  if constexpr (U <= 16) v = pair_min<16>(v);
+  return pair_min<32>(v);
+}
+
 // One chunk in one wave.  xi: the chunk's 64 integer targets (LDS), ci4: table values of the lane's four states,
 // bp: 64 x 32 bytes of LDS private to the wave, st_out: 64 bytes of LDS private to the wave.
 template <int KK>
 __device__ __forceinline__ void wave_chunk(const int* xi, const int (&ci4)[4], uint8_t* bp, uint8_t* st_out) {
   constexpr int U = 256 >> KK, PER = 64 / U;          // PER = predecessor indices j a lane step covers: j = l / U + PER * k
   const int lane = threadIdx.x & 63;
+  const int xreg = xi[lane];                           // target t lives in lane t
   int cost[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) cost[k] = (lane == 0 && k == 0) ? 0 : 0x40000000;
 #pragma unroll 1
   for (int t = 0; t < 64; ++t) {
-    int mn = min(min(cost[0], cost[1]), min(cost[2], cost[3]));
-#pragma unroll
-    for (int o = U; o < 64; o <<= 1) mn = min(mn, __shfl_xor(mn, o, 64));
+    const int mn = group_min<U>(min(min(cost[0], cost[1]), min(cost[2], cost[3])));
     int jb = 255;
 #pragma unroll
     for (int k = 3; k >= 0; --k) jb = cost[k] == mn ? lane / U + PER * k : jb;
-#pragma unroll
-    for (int o = U; o < 64; o <<= 1) jb = min(jb, __shfl_xor(jb, o, 64));
+    jb = group_min<U>(jb);
     if (lane < U) bp[t * 32 + lane] = (uint8_t)jb;
-    const int x = xi[t];
+    const int x = __builtin_amdgcn_readlane(xreg, t);
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-      const int u = (lane + 64 * k) >> KK;              // the group this state continues; lane u holds its minimum
-      const int m = __shfl(mn, u, 64);
+      // the group this state continues is u = (lane + 64 k) >> KK; lane u holds its minimum (reading the minima into
+      // scalar registers and selecting per lane was measured slower than this gather)
+      const int m = __shfl(mn, (lane + 64 * k) >> KK, 64);
       const int dx = x - ci4[k];
       cost[k] = dx * dx + m;
     }
