@@ -99,7 +99,7 @@ def _oracle_rows(oracle, blob, layer, k, v):
 
 
 @pytest.mark.parametrize("kk,mu", [(5, False), (4, False), (5, True), (4, True)])
-@pytest.mark.parametrize("ctx,M", [(0, 1), (70, 2), (300, 5), (1000, 1), (1500, 16)])
+@pytest.mark.parametrize("ctx,M", [(0, 1), (0, 7), (70, 2), (300, 5), (1000, 1), (1500, 16), (2100, 64)])
 def test_cache_rows_bit_exact_and_attention_within_the_bars(native, oracle, kk, mu, ctx, M):
     from tolerances import assert_attn_close
     layer = 1
@@ -165,3 +165,27 @@ def test_profiles_the_packed_cache_cannot_hold_are_refused(native):
     with native.KvCache(max_ctx=256) as kv:
         with pytest.raises(native.YkaError, match="256"):
             kv.set_profile(kvqp.synthetic(layers=1))
+
+
+@pytest.mark.parametrize("kk", [4, 5])
+def test_wide_and_narrow_kernels_agree_on_a_window(native, oracle, kk):
+    """the same 40-row window through the 128-row workgroups and (option key 3) through row tiles of 2 tokens"""
+    from tolerances import assert_attn_close
+    blob = kvqp.synthetic(layers=1, kk=kk, seed=21, mu=True)
+    ctx, M = 900, 40
+    k, v = _kv_rows(kk, ctx + M)
+    q = np.random.default_rng(kk).standard_normal((M, NH, 256)).astype(np.float16)
+    with native.KvCache(head_dim=256, max_ctx=1024) as kv:
+        kv.set_profile(blob)
+        for p in range(0, ctx + M, 64):
+            m = min(64, ctx + M - p)
+            kv.append256_f32_host(0, k[p:p + m], v[p:p + m], p, rotate=False)
+        wide = kv.layer_call(0, q, None, None, ctx)
+        kv.set_opt(2, 5)
+        wide5 = kv.layer_call(0, q, None, None, ctx)
+        kv.set_opt(3, 1)
+        narrow = kv.layer_call(0, q, None, None, ctx)
+    enc = _oracle_rows(oracle, blob, 0, k, v)
+    kd = np.stack([enc[0, h]["x"] for h in range(KVH)]); vd = np.stack([enc[1, h]["x"] for h in range(KVH)])
+    expect = oracle.tb_attend_f64(kd, vd, q, ctx)
+    assert_attn_close(wide, expect, "wide"); assert_attn_close(wide5, expect, "wide, 5 splits"); assert_attn_close(narrow, expect, "narrow")

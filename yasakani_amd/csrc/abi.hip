@@ -39,7 +39,8 @@ struct yka_kv {
     uint8_t* blob = nullptr; uint32_t* pairs = nullptr; float* gfac = nullptr; float* mu = nullptr;
     uint8_t* pool = nullptr; size_t layer_bytes = 0, pay_bytes = 0, scl_bytes = 0;
     uint8_t* scr = nullptr; size_t scr_w_ofs = 0;
-    uint8_t* kpay(int layer) const { return pool + (size_t)layer * layer_bytes; }
+    // 256 bytes in front of the first row: windows of the attention kernels begin in the word before a chunk
+    uint8_t* kpay(int layer) const { return pool + 256 + (size_t)layer * layer_bytes; }
     uint8_t* vpay(int layer) const { return kpay(layer) + pay_bytes; }
     float* kscl(int layer) const { return reinterpret_cast<float*>(kpay(layer) + 2 * pay_bytes); }
     float* vscl(int layer) const { return reinterpret_cast<float*>(kpay(layer) + 2 * pay_bytes + scl_bytes); }
@@ -139,18 +140,21 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
                hipStream_t st, int mode = 0, const uint16_t* k16 = nullptr, const uint16_t* v16 = nullptr) {
   const int NH = kv->cfg.n_heads;
   if (kv->tb) {
-    // trellis-coded rows: the encoder runs first (two launches), then row tiles of 2 tokens x 6 heads for every width
+    // trellis-coded rows: the encoder runs first (two launches); rows of at most 2 tokens (or option key 3) run on row
+    // tiles of 2 tokens x 6 heads, wider slices on 128-row workgroups that decode every tile once into LDS
     const yka_kv::Tb& T = *kv->tb;
     if (k16) do_append(kv, layer, k16, v16, M, d_pos, st);
     const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
     for (int s0 = 0; s0 < M; s0 += kMaxSlice) {
-      const int Ms = std::min(kMaxSlice, M - s0), tiles = (Ms + 1) / 2;
-      int S = kv->opt_splits_narrow > 0 ? kv->opt_splits_narrow : std::min(512 / (kv->cfg.n_kv_heads * tiles), ((ctx + 31) / 32) / 2);
-      S = std::min(std::max(2, std::min(kMaxSplits, S)), (int)(kWsPairs / (size_t)Ms));
+      const int Ms = std::min(kMaxSlice, M - s0), tiles = (Ms + 1) / 2, rb = (kG * Ms + 127) / 128;
+      const bool narrow = Ms <= 2 || kv->opt_force_narrow;
+      int S = narrow ? (kv->opt_splits_narrow > 0 ? kv->opt_splits_narrow : std::min(512 / (kv->cfg.n_kv_heads * tiles), ((ctx + 31) / 32) / 2))
+                     : (kv->opt_splits_wide > 0 ? kv->opt_splits_wide : std::min(256 / (kv->cfg.n_kv_heads * rb), ((ctx + 31) / 32) / (2 * rb)));
+      S = std::min(std::max(narrow ? 2 : 1, std::min(kMaxSplits, S)), (int)(kWsPairs / (size_t)Ms));
       const TbAttnArgs A{T.kpay(layer), T.vpay(layer), T.kscl(layer), T.vscl(layer), kv->cfg.max_ctx, kv->cfg.n_kv_heads, T.stride,
                          T.pairs, T.gfac, T.has_mu ? T.mu : nullptr, layer, q16 + (size_t)s0 * NH * 256, d_pos, depth, Ms, s0, NH, S,
                          kv->pm, kv->pl, kv->pacc16};
-      launch_attend_tb(A, T.kb, st);
+      if (narrow) launch_attend_tb(A, T.kb, st); else launch_attend_tb_wide(A, T.kb, st);
       if (mode != 2) launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, kv->opt_unrot}, st);
     }
     return;
@@ -591,8 +595,8 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
   HIPCHK(hipMalloc((void**)&T->pairs, pairs.size() * 4)); HIPCHK(hipMemcpy(T->pairs, pairs.data(), pairs.size() * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMalloc((void**)&T->gfac, gfac.size() * 4)); HIPCHK(hipMemcpy(T->gfac, gfac.data(), gfac.size() * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMalloc((void**)&T->mu, mu.size() * 4)); HIPCHK(hipMemcpy(T->mu, mu.data(), mu.size() * 4, hipMemcpyHostToDevice));
-  HIPCHK(hipMalloc((void**)&T->pool, T->layer_bytes * kv->cfg.n_layers));
-  HIPCHK(hipMemset(T->pool, 0, T->layer_bytes * kv->cfg.n_layers));     // unwritten rows: state 0 everywhere, scale 0
+  HIPCHK(hipMalloc((void**)&T->pool, 256 + T->layer_bytes * kv->cfg.n_layers + 256));
+  HIPCHK(hipMemset(T->pool, 0, 256 + T->layer_bytes * kv->cfg.n_layers + 256));     // unwritten rows: state 0 everywhere, scale 0
   HIPCHK(hipMalloc((void**)&T->scr, T->scr_w_ofs + jobs * 32));
   HIPCHK(hipDeviceSynchronize());
   YKA_CATCH_INT

@@ -100,7 +100,8 @@ struct TbAttnArgs {
   const uint16_t* q16; const int* d_pos; const uint8_t* depth; int M, tok0, n_heads, S;
   float* pm; float* pl; uint16_t* pacc16;
 };
-void launch_attend_tb(const TbAttnArgs&, int kb, hipStream_t);
+void launch_attend_tb(const TbAttnArgs&, int kb, hipStream_t);        // row tiles of 2 tokens x 6 heads (decode; any width)
+void launch_attend_tb_wide(const TbAttnArgs&, int kb, hipStream_t);   // 3..64 rows: 128 query rows per workgroup, tiles decoded once into LDS
 void launch_tb_encode(const TbEncArgs&, hipStream_t);
 void launch_tb_unpack(const uint8_t* blob, const int* grp, const int* pos, const uint8_t* pay, const uint32_t* side, int stride, const float* yin,
                       float* y, int rows, hipStream_t);
