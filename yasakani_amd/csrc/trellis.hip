@@ -125,16 +125,35 @@ __device__ __forceinline__ void wave_chunk(const int* xi, const int (&ci4)[4], u
   constexpr int U = 256 >> KK, PER = 64 / U;          // PER = predecessor indices j a lane step covers: j = l / U + PER * k
   const int lane = threadIdx.x & 63;
   const int xreg = xi[lane];                           // target t lives in lane t
+  // Costs are kept relative to a common offset (only differences decide) and, for 4- and 5-bit fields, carried as
+  // cost * 2^KK + j with j the state's index among the predecessors of its group: ONE minimum then yields the smallest
+  // cost and, among equal costs, the smallest predecessor.  At any step two states differ by at most two (three at 3
+  // bits) steps' worth of squared error, < 2 * 3148^2, so the packed value fits 32 bits once the offset - the minimum of
+  // group 0 - is subtracted at every step.  States that cannot be reached yet start 40,000,000 above state 0: more than
+  // any path costs before every state is reachable, like the reference's 2^30, and small enough to be packed.
+  constexpr bool kPacked = KK >= 4;
+  constexpr int kFar = kPacked ? 40000000 : 0x40000000;
   int cost[4];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) cost[k] = (lane == 0 && k == 0) ? 0 : 0x40000000;
+  for (int k = 0; k < 4; ++k) cost[k] = (lane == 0 && k == 0) ? 0 : kFar;
 #pragma unroll 1
   for (int t = 0; t < 64; ++t) {
-    const int mn = group_min<U>(min(min(cost[0], cost[1]), min(cost[2], cost[3])));
-    int jb = 255;
+    int mn, jb;
+    if constexpr (kPacked) {
+      int key[4];
 #pragma unroll
-    for (int k = 3; k >= 0; --k) jb = cost[k] == mn ? lane / U + PER * k : jb;
-    jb = group_min<U>(jb);
+      for (int k = 0; k < 4; ++k) key[k] = (cost[k] << KK) | (lane / U + PER * k);
+      const int km = group_min<U>(min(min(key[0], key[1]), min(key[2], key[3])));
+      jb = km & ((1 << KK) - 1);
+      mn = km >> KK;
+      mn -= __builtin_amdgcn_readlane(mn, 0);           // the common offset: group 0's minimum
+    } else {
+      mn = group_min<U>(min(min(cost[0], cost[1]), min(cost[2], cost[3])));
+      jb = 255;
+#pragma unroll
+      for (int k = 3; k >= 0; --k) jb = cost[k] == mn ? lane / U + PER * k : jb;
+      jb = group_min<U>(jb);
+    }
     if (lane < U) bp[t * 32 + lane] = (uint8_t)jb;
     const int x = __builtin_amdgcn_readlane(xreg, t);
 #pragma unroll
