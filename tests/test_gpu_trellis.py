@@ -189,3 +189,24 @@ def test_wide_and_narrow_kernels_agree_on_a_window(native, oracle, kk):
     kd = np.stack([enc[0, h]["x"] for h in range(KVH)]); vd = np.stack([enc[1, h]["x"] for h in range(KVH)])
     expect = oracle.tb_attend_f64(kd, vd, q, ctx)
     assert_attn_close(wide, expect, "wide"); assert_attn_close(wide5, expect, "wide, 5 splits"); assert_attn_close(narrow, expect, "narrow")
+
+
+def test_graph_replay_equals_eager_calls(native):
+    """the captured form of a layer call (encoder, attention, combine recorded into a graph and replayed over every
+    container) gives the bytes of the eager call, for a decode step and for a window"""
+    blob = kvqp.synthetic(layers=3, kk=5, seed=2)
+    ctx = 600
+    k, v = _kv_rows(31, ctx + 20)
+    k16, v16 = k.astype(np.float16), v.astype(np.float16)
+    rng = np.random.default_rng(32)
+    with native.KvCache(n_layers=3, head_dim=256, max_ctx=768) as kv:
+        kv.set_profile(blob)
+        for layer in range(3):
+            for p in range(0, ctx, 64):
+                m = min(64, ctx - p)
+                kv.append_host(layer, k16[p:p + m], v16[p:p + m], p)
+        for M in (1, 20):
+            q = rng.standard_normal((M, NH, 256)).astype(np.float16)
+            eager = kv.layer_call(2, q, k16[ctx:ctx + M], v16[ctx:ctx + M], ctx)
+            _, replay = kv.bench(q, k16[ctx:ctx + M], v16[ctx:ctx + M], ctx, mode=0, use_graph=True, reps=3)
+            assert np.array_equal(eager.view(np.uint16), replay.view(np.uint16)), M

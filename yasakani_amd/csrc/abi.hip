@@ -584,8 +584,17 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
   for (int g = 0; g < need; ++g)
     for (size_t i = 0; i < npair; ++i)
       pairs[(size_t)g * npair + i] = (uint32_t)tabs[(size_t)g * 256 + ((i >> kb) & 255)] | ((uint32_t)tabs[(size_t)g * 256 + (i & 255)] << 16);
+  struct TbGuard {                                     // a profile that could not be set up completely leaves the handle as it was
+    yka_kv* kv; bool done = false;
+    ~TbGuard() {
+      if (done || !kv->tb) return;
+      yka_kv::Tb* t = kv->tb;
+      (void)hipFree(t->blob); (void)hipFree(t->pairs); (void)hipFree(t->gfac); (void)hipFree(t->mu); (void)hipFree(t->pool); (void)hipFree(t->scr);
+      delete t; kv->tb = nullptr;
+    }
+  } guard{kv};
   yka_kv::Tb* T = new yka_kv::Tb();
-  kv->tb = T;                                          // freed by yka_kv_close whatever happens below
+  kv->tb = T;
   T->kb = kb; T->stride = 32 * kb; T->nm = I.nm; T->has_mu = has_mu;
   const size_t rows = (size_t)n_kv * kv->cfg.max_ctx;
   T->pay_bytes = rows * T->stride; T->scl_bytes = rows * 4; T->layer_bytes = 2 * T->pay_bytes + 2 * T->scl_bytes;
@@ -599,6 +608,7 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
   HIPCHK(hipMemset(T->pool, 0, 256 + T->layer_bytes * kv->cfg.n_layers + 256));     // unwritten rows: state 0 everywhere, scale 0
   HIPCHK(hipMalloc((void**)&T->scr, T->scr_w_ofs + jobs * 32));
   HIPCHK(hipDeviceSynchronize());
+  guard.done = true;
   YKA_CATCH_INT
 }
 
