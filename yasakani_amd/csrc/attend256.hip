@@ -199,6 +199,7 @@ template <bool MS>
 __global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
   constexpr int TPT = MS ? 1 : 2;
   __shared__ float s_m[4][16], s_l[4][16];
+  __shared__ __align__(16) float s_wn[16][4];
   __shared__ float s_acc[4][16][kD2 + 4];
   const int split = blockIdx.x, kvh = blockIdx.y, rt = blockIdx.z;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -362,18 +363,33 @@ __global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) s_acc[wave][i][8 * (4 * g + r + 16 * hh) + el] = o[hh * 8 + el][r];
   __syncthreads();
+  // per row: the weight of each wave's accumulator, already divided by the row's sum - computed once per row by 4 lanes,
+  // not once per output element
+  if (threadIdx.x < 64) {
+    const int j = threadIdx.x >> 2, w = threadIdx.x & 3;
+    const float mw = s_m[w][j];
+    float M2 = fmaxf(mw, __shfl_xor(mw, 1, 64));
+    M2 = fmaxf(M2, __shfl_xor(M2, 2, 64));
+    const float ww = exp2f(mw - M2);
+    float L = ww * s_l[w][j];
+    L += __shfl_xor(L, 1, 64);
+    L += __shfl_xor(L, 2, 64);
+    s_wn[j][w] = L > 0.f ? ww / L : 0.f;
+    const int tj = TPT * rt + j / kG;
+    if (w == 0 && j < TPT * kG && tj < A.M) {
+      const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
+      A.pm[p] = M2; A.pl[p] = L;
+    }
+  }
+  __syncthreads();
   for (int idx = threadIdx.x; idx < TPT * kG * kD2; idx += 256) {
     const int j = idx >> 8, d = idx & (kD2 - 1);
     const int tj = TPT * rt + j / kG;
     if (tj >= A.M) continue;
-    const float m0 = s_m[0][j], m1 = s_m[1][j], m2 = s_m[2][j], m3 = s_m[3][j];
-    const float M2 = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
-    const float w0 = exp2f(m0 - M2), w1 = exp2f(m1 - M2), w2 = exp2f(m2 - M2), w3 = exp2f(m3 - M2);
+    const f4 w4 = *reinterpret_cast<const f4*>(s_wn[j]);
     const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
-    const float L = w0 * s_l[0][j] + w1 * s_l[1][j] + w2 * s_l[2][j] + w3 * s_l[3][j];
-    const float acc = w0 * s_acc[0][j][d] + w1 * s_acc[1][j][d] + w2 * s_acc[2][j][d] + w3 * s_acc[3][j][d];
-    A.pacc16[p * kD2 + d] = __half_as_ushort(__float2half_rn(L > 0.f ? acc / L : 0.f));
-    if (d == 0) { A.pm[p] = M2; A.pl[p] = L; }
+    const float y = w4[0] * s_acc[0][j][d] + w4[1] * s_acc[1][j][d] + w4[2] * s_acc[2][j][d] + w4[3] * s_acc[3][j][d];
+    A.pacc16[p * kD2 + d] = __half_as_ushort(__float2half_rn(y));
   }
 }
 

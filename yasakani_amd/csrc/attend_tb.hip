@@ -56,6 +56,7 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
   constexpr int kTabBytes = 4 << (8 + KB);           // one pair table
   constexpr int kAccBytes = 4 * 16 * (kD2 + 4) * 4;
   __shared__ float s_m[4][16], s_l[4][16];
+  __shared__ __align__(16) float s_wn[16][4];
   __shared__ __align__(16) uint8_t s_buf[kAccBytes > 2 * kTabBytes ? kAccBytes : 2 * kTabBytes];   // pair tables, then the wave merge
   float (*s_acc)[16][kD2 + 4] = reinterpret_cast<float (*)[16][kD2 + 4]>(s_buf);
   const uint8_t* const s_tabK = s_buf;
@@ -253,21 +254,34 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) s_acc[wave][i][8 * (4 * g + r + 16 * hh) + el] = o[hh * 8 + el][r];
   __syncthreads();
-  const float gv = A.gfac[gV];
+  // per row: the weight of each wave's accumulator, already divided by the row's sum and multiplied by gain / 256 of the
+  // V table - computed once per row by 4 lanes, not once per output element
+  if (threadIdx.x < 64) {
+    const int j = threadIdx.x >> 2, w = threadIdx.x & 3;
+    const float mw = s_m[w][j];
+    float M2 = fmaxf(mw, __shfl_xor(mw, 1, 64));
+    M2 = fmaxf(M2, __shfl_xor(M2, 2, 64));
+    const float ww = exp2f(mw - M2);
+    float L = ww * s_l[w][j];
+    L += __shfl_xor(L, 1, 64);
+    L += __shfl_xor(L, 2, 64);
+    s_wn[j][w] = L > 0.f ? ww * A.gfac[gV] / L : 0.f;
+    const int tj = 2 * rt + j / kG;
+    if (w == 0 && j < 2 * kG && tj < A.M) {
+      const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
+      A.pm[p] = M2; A.pl[p] = L;
+    }
+  }
+  __syncthreads();
   for (int idx = threadIdx.x; idx < 2 * kG * kD2; idx += 256) {
     const int j = idx >> 8, d = idx & (kD2 - 1);
     const int tj = 2 * rt + j / kG;
     if (tj >= A.M) continue;
-    const float m0 = s_m[0][j], m1 = s_m[1][j], m2 = s_m[2][j], m3 = s_m[3][j];
-    const float M2 = fmaxf(fmaxf(m0, m1), fmaxf(m2, m3));
-    const float w0 = exp2f(m0 - M2), w1 = exp2f(m1 - M2), w2 = exp2f(m2 - M2), w3 = exp2f(m3 - M2);
+    const f4 w4 = *reinterpret_cast<const f4*>(s_wn[j]);
     const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
-    const float L = w0 * s_l[0][j] + w1 * s_l[1][j] + w2 * s_l[2][j] + w3 * s_l[3][j];
-    const float acc = w0 * s_acc[0][j][d] + w1 * s_acc[1][j][d] + w2 * s_acc[2][j][d] + w3 * s_acc[3][j][d];
-    float y = L > 0.f ? acc * gv / L : 0.f;
-    if (A.mu && L > 0.f) y += A.mu[(size_t)gV * 256 + d];
+    float y = w4[0] * s_acc[0][j][d] + w4[1] * s_acc[1][j][d] + w4[2] * s_acc[2][j][d] + w4[3] * s_acc[3][j][d];
+    if (A.mu && w4[0] + w4[1] + w4[2] + w4[3] > 0.f) y += A.mu[(size_t)gV * 256 + d];
     A.pacc16[p * kD2 + d] = __half_as_ushort(__float2half_rn(y));
-    if (d == 0) { A.pm[p] = M2; A.pl[p] = L; }
   }
 }
 
