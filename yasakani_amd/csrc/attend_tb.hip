@@ -155,8 +155,9 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
     uint32_t vw[2][8][3];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) vsc[kt] = *reinterpret_cast<const f4*>(vscl + t0 + 16 * kt + 4 * g);
-#pragma unroll
-    for (int hh = 0; hh < 2; ++hh)
+    // V windows of the channel blocks hh = 0 now (their latency runs under the score phase), those of hh = 1 after the
+    // score phase (under the softmax and the first half of the PV product): the registers are needed in between
+    auto load_v = [&](int hh) __attribute__((always_inline)) {
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const int tok = t0 + 16 * (e >> 2) + 4 * g + (e & 3);
@@ -165,23 +166,41 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
         __builtin_memcpy(&vw[hh][e][0], __builtin_assume_aligned(vr + (int32_t)vo[hh], 4), KB == 5 ? 12 : 8);
         vw[hh][e][0] &= keep0;
       }
+    };
+    load_v(0);
     const bool need_mask = t0 + 32 > minlen;
     // ---- scores ----
     float s[8];
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt) {
+      // at 4 bits per element all 32 table reads of the key block are issued ahead of the MFMA chain, so that the chain
+      // does not wait for LDS between links (measured 6 % on the decode kernel); at 5 bits the registers do not allow it
       f4 part = f4{0.f, 0.f, 0.f, 0.f};
-      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 0>(kw[kt], s_tabK), qf[0], part, 0, 0, 0);
-      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 8>(kw[kt], s_tabK), qf[1], part, 0, 0, 0);
-      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 16>(kw[kt], s_tabK), qf[2], part, 0, 0, 0);
-      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 24>(kw[kt], s_tabK), qf[3], part, 0, 0, 0);
-      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 32>(kw[kt], s_tabK), qf[4], part, 0, 0, 0);
-      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 40>(kw[kt], s_tabK), qf[5], part, 0, 0, 0);
-      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 48>(kw[kt], s_tabK), qf[6], part, 0, 0, 0);
-      part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 56>(kw[kt], s_tabK), qf[7], part, 0, 0, 0);
+      if constexpr (KB == 4) {
+        h8 kf[8];
+        kf[0] = chunk_vals<KB, 0>(kw[kt], s_tabK); kf[1] = chunk_vals<KB, 8>(kw[kt], s_tabK);
+        kf[2] = chunk_vals<KB, 16>(kw[kt], s_tabK); kf[3] = chunk_vals<KB, 24>(kw[kt], s_tabK);
+        kf[4] = chunk_vals<KB, 32>(kw[kt], s_tabK); kf[5] = chunk_vals<KB, 40>(kw[kt], s_tabK);
+        kf[6] = chunk_vals<KB, 48>(kw[kt], s_tabK); kf[7] = chunk_vals<KB, 56>(kw[kt], s_tabK);
+#pragma unroll
+        for (int t = 0; t < 8; ++t) part = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[t], qf[t], part, 0, 0, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, 70, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 32, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 8, 0);
+      } else {
+        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 0>(kw[kt], s_tabK), qf[0], part, 0, 0, 0);
+        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 8>(kw[kt], s_tabK), qf[1], part, 0, 0, 0);
+        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 16>(kw[kt], s_tabK), qf[2], part, 0, 0, 0);
+        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 24>(kw[kt], s_tabK), qf[3], part, 0, 0, 0);
+        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 32>(kw[kt], s_tabK), qf[4], part, 0, 0, 0);
+        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 40>(kw[kt], s_tabK), qf[5], part, 0, 0, 0);
+        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 48>(kw[kt], s_tabK), qf[6], part, 0, 0, 0);
+        part = __builtin_amdgcn_mfma_f32_16x16x32_f16(chunk_vals<KB, 56>(kw[kt], s_tabK), qf[7], part, 0, 0, 0);
+      }
 #pragma unroll
       for (int r = 0; r < 4; ++r) s[4 * kt + r] = part[r] * ksc[kt][r];          // key t0 + 16 kt + 4 g + r against row i
     }
+    load_v(1);
     if (T + 4 < tile1) load_k(T + 4);
     if (need_mask) {
 #pragma unroll
