@@ -332,9 +332,10 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
         acc[0] += w[wv] * a0.x; acc[1] += w[wv] * a0.y; acc[2] += w[wv] * a0.z; acc[3] += w[wv] * a0.w;
         acc[4] += w[wv] * a1.x; acc[5] += w[wv] * a1.y; acc[6] += w[wv] * a1.z; acc[7] += w[wv] * a1.w;
       }
+      const float inv = L > 0.f ? 1.f / L : 0.f;            // one division per lane, not one per channel
       h8 v;
 #pragma unroll
-      for (int e = 0; e < 8; ++e) v[e] = (_Float16)(L > 0.f ? acc[e] / L : 0.f);
+      for (int e = 0; e < 8; ++e) v[e] = (_Float16)(acc[e] * inv);
       *reinterpret_cast<uint4*>(A.pacc16 + p * kD + c8) = __builtin_bit_cast(uint4, v);
       if (c8 == 0) { A.pm[p] = M2; A.pl[p] = L; }
     }
