@@ -325,12 +325,15 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
       const float w[4] = {exp2f(m0 - M2), exp2f(m1 - M2), exp2f(m2 - M2), exp2f(m3 - M2)};
       const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
       const float L = w[0] * s_l[0][j] + w[1] * s_l[1][j] + w[2] * s_l[2][j] + w[3] * s_l[3][j];
+      float4 a0[4], a1[4];                                    // all eight reads first: one LDS round trip, not eight
+#pragma unroll
+      for (int wv = 0; wv < 4; ++wv) { a0[wv] = *reinterpret_cast<const float4*>(&s_acc[wv][j][c8]); a1[wv] = *reinterpret_cast<const float4*>(&s_acc[wv][j][c8 + 4]); }
+      __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);
       float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int wv = 0; wv < 4; ++wv) {
-        const float4 a0 = *reinterpret_cast<const float4*>(&s_acc[wv][j][c8]), a1 = *reinterpret_cast<const float4*>(&s_acc[wv][j][c8 + 4]);
-        acc[0] += w[wv] * a0.x; acc[1] += w[wv] * a0.y; acc[2] += w[wv] * a0.z; acc[3] += w[wv] * a0.w;
-        acc[4] += w[wv] * a1.x; acc[5] += w[wv] * a1.y; acc[6] += w[wv] * a1.z; acc[7] += w[wv] * a1.w;
+        acc[0] += w[wv] * a0[wv].x; acc[1] += w[wv] * a0[wv].y; acc[2] += w[wv] * a0[wv].z; acc[3] += w[wv] * a0[wv].w;
+        acc[4] += w[wv] * a1[wv].x; acc[5] += w[wv] * a1[wv].y; acc[6] += w[wv] * a1[wv].z; acc[7] += w[wv] * a1[wv].w;
       }
       const float inv = L > 0.f ? 1.f / L : 0.f;            // one division per lane, not one per channel
       h8 v;
