@@ -210,3 +210,22 @@ def test_graph_replay_equals_eager_calls(native):
             eager = kv.layer_call(2, q, k16[ctx:ctx + M], v16[ctx:ctx + M], ctx)
             _, replay = kv.bench(q, k16[ctx:ctx + M], v16[ctx:ctx + M], ctx, mode=0, use_graph=True, reps=3)
             assert np.array_equal(eager.view(np.uint16), replay.view(np.uint16)), M
+
+
+def test_rotated_rows_are_rotated_before_they_are_coded(native, oracle):
+    """yka_append256_f32 with rotate = 1 on a handle with a profile: signed Hadamard rotation (kvx_rotate), then the
+    trellis encoder - stored words and scales against the oracle's rotation followed by the oracle's encoder"""
+    blob = kvqp.synthetic(layers=1, kk=5, seed=17)
+    n = 70
+    k, v = _kv_rows(77, n)
+    with native.KvCache(head_dim=256, max_ctx=256) as kv:
+        kv.set_profile(blob)
+        kv.append256_f32_host(0, k[:64], v[:64], 0, rotate=True)
+        kv.append256_f32_host(0, k[64:], v[64:], 64, rotate=True)
+        kw, ks, vw, vs = kv.export_rows(0, 0, n)
+    kr = np.stack([oracle.kvx_rotate256(k[:, h]) for h in range(KVH)], 1)
+    vr = np.stack([oracle.kvx_rotate256(v[:, h]) for h in range(KVH)], 1)
+    enc = _oracle_rows(oracle, blob, 0, kr, vr)
+    for h in range(KVH):
+        assert np.array_equal(kw[h], enc[0, h]["words"][:, :40]) and np.array_equal(vw[h], enc[1, h]["words"][:, :40]), h
+        assert _same(ks[h], enc[0, h]["scale"]) and _same(vs[h], enc[1, h]["scale"])
