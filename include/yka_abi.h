@@ -200,7 +200,8 @@ YKA_API int yka_tb_pack_unpack(const uint8_t* blob, size_t blob_len, const float
  * the reference lays them out: payload (kv head * max_ctx + pos) * 32 * bits bytes, one fp32 scale per row in a parallel
  * array (q35_atxpk3.cuh:196-200).  From then on yka_append / yka_append256_f32 / yka_append_attend encode rows with the
  * trellis encoder (launch_tb_requant -> launch_tb_fast, q35_kernels.cu:1084-1092) and yka_attend / yka_append_attend
- * read them (launch_q35_atx_pk); yka_attn_post, the multi-stream pass and the flat-row export / import refuse.
+ * read them (launch_q35_atx_pk); yka_attn_post hands its finished K / V rows to the encoder (as launch_q35_attn_post is
+ * followed by launch_tb_requant); the multi-stream pass and the flat-row export / import refuse.
  * Synchronous; allocates (the only call of the trellis path that does). */
 YKA_API int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len);
 /* bits per element of the handle's trellis-coded rows, 0 if it has no profile */

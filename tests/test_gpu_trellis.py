@@ -229,3 +229,30 @@ def test_rotated_rows_are_rotated_before_they_are_coded(native, oracle):
     for h in range(KVH):
         assert np.array_equal(kw[h], enc[0, h]["words"][:, :40]) and np.array_equal(vw[h], enc[1, h]["words"][:, :40]), h
         assert _same(ks[h], enc[0, h]["scale"]) and _same(vs[h], enc[1, h]["scale"])
+
+
+@pytest.mark.parametrize("rot", [False, True])
+def test_attn_post_feeds_the_encoder(native, oracle, rot):
+    """yka_attn_post on a handle with a profile: RMS norm + rotary + rotation as on flat rows (Q rows bit-exact), and the
+    finished K / V rows coded by the trellis encoder: stored words and scales against the oracle's post step followed by
+    the oracle's encoder"""
+    blob = kvqp.synthetic(layers=1, kk=5, seed=23)
+    rng = np.random.default_rng(24)
+    M, rd, pos, ctx = 5, 64, 250, 512
+    xq = (rng.standard_normal((M, NH, 256)) * 2).astype(np.float32)
+    xk = (rng.standard_normal((M, KVH, 256)) * 0.7).astype(np.float32)
+    xk[:, :, [5, 77, 130, 201]] *= 8
+    xv = rng.standard_normal((M, KVH, 256)).astype(np.float32)
+    qw = (rng.standard_normal(256) * 0.1).astype(np.float16).view(np.uint16)
+    kw_ = (rng.standard_normal(256) * 0.1).astype(np.float16).view(np.uint16)
+    rope = oracle.rope_table(ctx, rd)
+    q16, k32, v32 = oracle.attn_post256(xq, xk, xv, qw, kw_, 1e-6, rope, rd, pos, int(rot))
+    with native.KvCache(head_dim=256, max_ctx=ctx) as kv:
+        kv.set_profile(blob)
+        got_q = kv.attn_post_host(0, xq, xk, xv, pos, qw, kw_, 1e-6, rope, rd, rotate=rot)
+        kw, ks, vw, vs = kv.export_rows(0, pos, M)
+    assert np.array_equal(got_q.view(np.uint16), q16)
+    for h in range(KVH):
+        for kind, x, w, s in ((0, k32, kw, ks), (1, v32, vw, vs)):
+            enc = oracle.tb_encode_rows(blob, np.full(M, h * 2 + kind, np.int32), np.arange(pos, pos + M, dtype=np.int32), x[:, h])
+            assert np.array_equal(w[h], enc["words"][:, :40]) and _same(s[h], enc["scale"]), (h, kind)

@@ -39,6 +39,7 @@ struct yka_kv {
     uint8_t* blob = nullptr; uint32_t* pairs = nullptr; float* gfac = nullptr; float* mu = nullptr;
     uint8_t* pool = nullptr; size_t layer_bytes = 0, pay_bytes = 0, scl_bytes = 0;
     uint8_t* scr = nullptr; size_t scr_w_ofs = 0;
+    float* stage = nullptr;          // fp32 K rows then V rows of one pass ([max_rows][n_kv][256] each): yka_attn_post -> encoder
     // 256 bytes in front of the first row: windows of the attention kernels begin in the word before a chunk
     uint8_t* kpay(int layer) const { return pool + 256 + (size_t)layer * layer_bytes; }
     uint8_t* vpay(int layer) const { return kpay(layer) + pay_bytes; }
@@ -108,18 +109,30 @@ void check_rows(const yka_kv* kv, int M) {
 constexpr int kTbTileTok = 128;     // tokens per launch of the trellis encoder (its scratch holds that many)
 // trellis encoder over the rows of a pass: fp32 rows, or fp16 rows if k32 == nullptr
 void tb_append(yka_kv* kv, int layer, const float* k32, const float* v32, const uint16_t* k16, const uint16_t* v16, int M, const int* d_pos,
-               int rot, hipStream_t st) {
+               int rot, hipStream_t st, int pos_limit = 0) {
   const yka_kv::Tb& T = *kv->tb;
   for (int t0 = 0; t0 < M; t0 += kTbTileTok) {
     TbEncArgs A{};
     A.blob = T.blob; A.nm = T.nm; A.has_trellis = 1;
     A.k32 = k32; A.v32 = v32; A.k16 = k16; A.v16 = v16; A.d_pos = d_pos; A.layer = layer; A.tok0 = t0; A.n_kv = kv->cfg.n_kv_heads;
-    A.max_ctx = kv->cfg.max_ctx; A.rot = rot;
+    A.max_ctx = kv->cfg.max_ctx; A.rot = rot; A.pos_limit = pos_limit;
     A.nrow = std::min(kTbTileTok, M - t0) * 2 * kv->cfg.n_kv_heads;
     A.scr = T.scr; A.scr_w_ofs = T.scr_w_ofs;
     A.pay0 = T.kpay(layer); A.pay1 = T.vpay(layer); A.scl0 = T.kscl(layer); A.scl1 = T.vscl(layer); A.stride = T.stride;
     launch_tb_encode(A, st);
   }
+}
+// the step between the projection and the cache.  On trellis-coded rows the finished K / V rows go to a staging buffer
+// as fp32 and the encoder runs on them (the reference: launch_q35_attn_post, then launch_tb_requant, q35_kernels.cu:1084-1092)
+void post_launch(yka_kv* kv, int layer, PostArgs& A, hipStream_t st) {
+  if (kv->tb) {
+    A.k32_out = kv->tb->stage;
+    A.v32_out = kv->tb->stage + (size_t)kv->cfg.max_rows * kv->cfg.n_kv_heads * 256;
+    launch_attn_post256(A, st);
+    // rows the post kernel drops (beyond the rotary table) are not stored by the encoder either
+    tb_append(kv, layer, A.k32_out, A.v32_out, nullptr, nullptr, A.M, A.d_pos, 0, st, A.rd > 0 ? A.rope_rows : 0);
+  } else if (kv->r256()) launch_attn_post256(A, st);
+  else launch_attn_post(A, st);
 }
 void no_trellis(const yka_kv* kv) {
   if (kv->tb) throw std::runtime_error("this entry point does not work on trellis-coded rows");
@@ -284,7 +297,7 @@ void yka_kv_close(yka_kv* kv) {
   if (kv->stream) (void)hipStreamDestroy(kv->stream);
   if (kv->tb) {
     (void)hipFree(kv->tb->blob); (void)hipFree(kv->tb->pairs); (void)hipFree(kv->tb->gfac); (void)hipFree(kv->tb->mu); (void)hipFree(kv->tb->pool);
-    (void)hipFree(kv->tb->scr);
+    (void)hipFree(kv->tb->scr); (void)hipFree(kv->tb->stage);
     delete kv->tb;
   }
   (void)hipFree(kv->pool); (void)hipFree(kv->tables); (void)hipFree(kv->pm); (void)hipFree(kv->pl); (void)hipFree(kv->pacc16); (void)hipFree(kv->d_pos);
@@ -407,11 +420,11 @@ static void check_post(const yka_kv* kv, const yka_post_params* P) {
 int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float* d_xk, const float* d_xv, int M, const int* d_pos,
                   const yka_post_params* P, uint16_t* d_q16, void* hip_stream) {
   YKA_TRY
-  on_device(kv); no_trellis(kv); check_layer(kv, layer); check_rows(kv, M); check_post(kv, P);
+  on_device(kv); check_layer(kv, layer); check_rows(kv, M); check_post(kv, P);
   if (!d_xq || !d_xk || !d_xv || !d_pos || !d_q16) throw std::runtime_error("null pointer");
-  const PostArgs A{kv->view(layer), d_xq, d_xk, d_xv, M, kv->cfg.n_heads, d_pos, P->d_qn_w16, P->d_kn_w16, P->eps,
-                   P->d_rope, P->rope_dims, P->rope_rows, P->rotate != 0, d_q16};
-  if (kv->r256()) launch_attn_post256(A, (hipStream_t)hip_stream); else launch_attn_post(A, (hipStream_t)hip_stream);
+  PostArgs A{kv->view(layer), d_xq, d_xk, d_xv, M, kv->cfg.n_heads, d_pos, P->d_qn_w16, P->d_kn_w16, P->eps,
+             P->d_rope, P->rope_dims, P->rope_rows, P->rotate != 0, d_q16};
+  post_launch(kv, layer, A, (hipStream_t)hip_stream);
   HIPCHK(hipGetLastError());
   YKA_CATCH_INT
 }
@@ -420,7 +433,7 @@ int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, 
                        const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope, int rope_dims,
                        int rope_rows, int rotate, uint16_t* q16) {
   YKA_TRY
-  on_device(kv); no_trellis(kv); check_layer(kv, layer); check_rows(kv, M);
+  on_device(kv); check_layer(kv, layer); check_rows(kv, M);
   if (!xq || !xk || !xv || !qn_w16 || !kn_w16 || !q16) throw std::runtime_error("null pointer");
   if (pos < 0 || (long long)pos + M > kv->cfg.max_ctx) throw std::runtime_error("rows outside the container");
   const int kD = kv->D();                          // 128 or 256 channels per head
@@ -438,9 +451,9 @@ int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, 
   yka_post_params P{dqw.as<uint16_t>(), dkw.as<uint16_t>(), eps, dr.as<float>(), rope_dims, rope_rows, rotate};
   check_post(kv, &P);
   launch_set_int(kv->d_pos, pos, kv->stream);
-  const PostArgs A{kv->view(layer), dq.as<float>(), dk.as<float>(), dv.as<float>(), M, kv->cfg.n_heads, kv->d_pos,
-                   P.d_qn_w16, P.d_kn_w16, eps, P.d_rope, rope_dims, rope_rows, rotate != 0, dq16.as<uint16_t>()};
-  if (kv->r256()) launch_attn_post256(A, kv->stream); else launch_attn_post(A, kv->stream);
+  PostArgs A{kv->view(layer), dq.as<float>(), dk.as<float>(), dv.as<float>(), M, kv->cfg.n_heads, kv->d_pos,
+             P.d_qn_w16, P.d_kn_w16, eps, P.d_rope, rope_dims, rope_rows, rotate != 0, dq16.as<uint16_t>()};
+  post_launch(kv, layer, A, kv->stream);
   HIPCHK(hipGetLastError());
   HIPCHK(hipStreamSynchronize(kv->stream));
   HIPCHK(hipMemcpy(q16, dq16.p, nq * 2, hipMemcpyDeviceToHost));
@@ -589,7 +602,7 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
     ~TbGuard() {
       if (done || !kv->tb) return;
       yka_kv::Tb* t = kv->tb;
-      (void)hipFree(t->blob); (void)hipFree(t->pairs); (void)hipFree(t->gfac); (void)hipFree(t->mu); (void)hipFree(t->pool); (void)hipFree(t->scr);
+      (void)hipFree(t->blob); (void)hipFree(t->pairs); (void)hipFree(t->gfac); (void)hipFree(t->mu); (void)hipFree(t->pool); (void)hipFree(t->scr); (void)hipFree(t->stage);
       delete t; kv->tb = nullptr;
     }
   } guard{kv};
@@ -607,6 +620,7 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
   HIPCHK(hipMalloc((void**)&T->pool, 256 + T->layer_bytes * kv->cfg.n_layers + 256));
   HIPCHK(hipMemset(T->pool, 0, 256 + T->layer_bytes * kv->cfg.n_layers + 256));     // unwritten rows: state 0 everywhere, scale 0
   HIPCHK(hipMalloc((void**)&T->scr, T->scr_w_ofs + jobs * 32));
+  HIPCHK(hipMalloc((void**)&T->stage, (size_t)2 * kv->cfg.max_rows * n_kv * 256 * sizeof(float)));
   HIPCHK(hipDeviceSynchronize());
   guard.done = true;
   YKA_CATCH_INT

@@ -139,6 +139,8 @@ __global__ void __launch_bounds__(256) attn_post256_kernel(PostArgs A) {
   if (isq) {
     asm volatile("" : "+v"(out));                  // the rotation's last multiply is rounded to fp32 before the fp16 rounding
     A.q16[((size_t)tok * NH + head) * kD2 + d] = __half_as_ushort(__float2half_rn(out));
+  } else if (A.k32_out) {
+    (isk ? A.k32_out : A.v32_out)[((size_t)tok * KVH + head) * kD2 + d] = out;
   } else {
     quant_store_row256(A.kv, head, pos, !isk, out, d, red, fld);
   }

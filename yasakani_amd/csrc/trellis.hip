@@ -270,7 +270,7 @@ __global__ void __launch_bounds__(256) tb_select_kernel(TbEncArgs A) {
     if (P.has_mu) x = __fadd_rn(x, Q.mud);
     pc = (unsigned)__half_as_ushort(__float2half_rn(Q.cj0)) | ((unsigned)__half_as_ushort(__float2half_rn(Q.cj1)) << 16);
   }
-  const bool in_range = A.yin || (R.pos >= 0 && R.pos < A.max_ctx);
+  const bool in_range = A.yin || (R.pos >= 0 && R.pos < A.max_ctx && (A.pos_limit == 0 || R.pos < A.pos_limit));
   uint8_t* const payb = R.kind ? A.pay1 : A.pay0;
   if (payb && in_range) {
     uint32_t* const wrow = reinterpret_cast<uint32_t*>(payb + R.out * (size_t)A.stride);

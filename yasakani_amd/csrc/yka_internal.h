@@ -75,6 +75,9 @@ struct PostArgs {
   const uint16_t* qn_w16; const uint16_t* kn_w16; float eps;
   const float* rope; int rd; int rope_rows;      // rope [rope_rows][rd/2] (cos, sin) pairs; rd = 0: no rotary step
   int rot; uint16_t* q16;
+  // 256-channel heads only: if set, the finished K / V rows are written here as fp32 [M][n_kv][256] instead of being
+  // quantized into kv (a handle with trellis-coded rows runs its encoder on them afterwards)
+  float* k32_out = nullptr; float* v32_out = nullptr;
 };
 
 // Trellis-coded rows (trellis.hip; reference TbFastArgs, src/kvq_fast.hpp:16-37).  Probe form (yin != nullptr): rows
@@ -90,6 +93,7 @@ struct TbEncArgs {
   int nrow;
   uint8_t* scr; size_t scr_w_ofs;     // scratch: states [nrow * nm][256] bytes, then at scr_w_ofs error sums [nrow * nm][8] fp32
   uint8_t* pay0; uint8_t* pay1; float* scl0; float* scl1; int stride;
+  int pos_limit;                      // cache form: rows at positions >= pos_limit are not stored (0: no limit besides max_ctx)
 };
 // attention over trellis-coded rows (attend_tb.hip).  pairs [groups][2^(8 + kb)]: entry i = the table's integers, as two
 // fp16 values, of the states (i >> kb) & 255 and i & 255 (two consecutive elements from 8 + kb stream bits); gfac [groups]:
