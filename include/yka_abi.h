@@ -62,7 +62,10 @@ YKA_API const char* yka_build_info(void);
  * key 5: context length (tokens) the caller expects, used only to size the decode grid (the reference picks its split
  *        count from the length known on the host, engine35.hpp:434-439); 0 = the max_ctx of the handle.  Any actual
  *        position stays correct: positions are read on the device and the kernel uses as many of the launched
- *        splits as the length it finds there justifies. */
+ *        splits as the length it finds there justifies;
+ * key 6: handles with trellis-coded rows, multi-stream passes only: the profile layer whose groups code and decode the
+ *        rows (the containers of such a handle are the streams of that one layer; the reference passes the layer in
+ *        TbFastArgs::layer / Q35PkArgs::layer). */
 YKA_API int yka_set_opt(yka_kv* kv, int key, int value);
 
 /* Paged mode: logical page p of `layer` (-1 = every layer) lives in physical page h_table[p]; n_pages = max_ctx/256
@@ -201,7 +204,10 @@ YKA_API int yka_tb_pack_unpack(const uint8_t* blob, size_t blob_len, const float
  * array (q35_atxpk3.cuh:196-200).  From then on yka_append / yka_append256_f32 / yka_append_attend encode rows with the
  * trellis encoder (launch_tb_requant -> launch_tb_fast, q35_kernels.cu:1084-1092) and yka_attend / yka_append_attend
  * read them (launch_q35_atx_pk); yka_attn_post hands its finished K / V rows to the encoder (as launch_q35_attn_post is
- * followed by launch_tb_requant); the multi-stream pass and the flat-row export / import refuse.
+ * followed by launch_tb_requant); the multi-stream pass runs on them with the groups of the layer option
+ * key 6 names (launch_tb_fast_ms, kvq_fast.cuh:236-392; launch_q35_atx_pk_ms, q35_atxpk.hpp:18-20); the flat-row export /
+ * import refuse.  The profile's layers are model layers: a single-stream call names one of them, so its `layer` must be
+ * below both n_layers of the handle and the number of layers the profile has groups for.
  * Synchronous; allocates (the only call of the trellis path that does). */
 YKA_API int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len);
 /* bits per element of the handle's trellis-coded rows, 0 if it has no profile */

@@ -160,7 +160,8 @@ def test_profiles_the_packed_cache_cannot_hold_are_refused(native):
         kv.set_profile(kvqp.synthetic(layers=1, kk=4))
         with pytest.raises(native.YkaError, match="already"):
             kv.set_profile(kvqp.synthetic(layers=1, kk=4))
-        with pytest.raises(native.YkaError, match="trellis"):
+        with pytest.raises(native.YkaError, match="no groups for this layer"):
+            kv.set_opt(6, 1)                                   # the multi-stream pass would use the groups of layer 1
             kv.ms_call(np.zeros((1, NH, 256), np.float16), None, None, np.zeros(1, np.int32), np.zeros(1, np.int32))
     with native.KvCache(max_ctx=256) as kv:
         with pytest.raises(native.YkaError, match="256"):
@@ -256,3 +257,71 @@ def test_attn_post_feeds_the_encoder(native, oracle, rot):
         for kind, x, w, s in ((0, k32, kw, ks), (1, v32, vw, vs)):
             enc = oracle.tb_encode_rows(blob, np.full(M, h * 2 + kind, np.int32), np.arange(pos, pos + M, dtype=np.int32), x[:, h])
             assert np.array_equal(w[h], enc["words"][:, :40]) and _same(s[h], enc["scale"]), (h, kind)
+
+
+# ---- multi-stream passes over trellis-coded rows: every row names its own container (stream) and position ----
+MS_CTX = 1024
+MS_LENS = [300, 17, 900, 512, 0]                       # cached tokens per stream; the last stream is empty
+
+
+def _streams(native, oracle, blob, layer):
+    rng = np.random.default_rng(55)
+    kv = native.KvCache(n_layers=len(MS_LENS), head_dim=256, max_ctx=MS_CTX, max_rows=64)
+    kv.set_profile(blob)
+    kv.set_opt(6, layer)
+    rows = []
+    for s, n in enumerate(MS_LENS):
+        k = np.zeros((MS_CTX, KVH, 256), np.float16); v = np.zeros_like(k)
+        if n:
+            kn = rng.standard_normal((n, KVH, 256)).astype(np.float16); kn[:, :, [5, 77, 130, 201]] *= 4
+            vn = rng.standard_normal((n, KVH, 256)).astype(np.float16)
+            k[:n] = kn; v[:n] = vn
+            # fill through the multi-stream pass itself: rows of stream s at positions 0 .. n-1, 32 at a time
+            for p in range(0, n, 32):
+                m = min(32, n - p)
+                kv.ms_call(np.zeros((m, NH, 256), np.float16), kn[p:p + m], vn[p:p + m], np.arange(p, p + m, dtype=np.int32), np.full(m, s, np.int32))
+        rows.append([k, v, n])
+    return kv, rows, rng
+
+
+def _stream_expect(oracle, blob, layer, k, v, n, q, pos):
+    """fp64 attention of one row at position pos over the oracle-coded rows [0, pos] of its stream"""
+    enc = _oracle_rows(oracle, blob, layer, k[:n].astype(np.float32), v[:n].astype(np.float32))
+    kd = np.stack([enc[0, h]["x"] for h in range(KVH)]); vd = np.stack([enc[1, h]["x"] for h in range(KVH)])
+    return oracle.tb_attend_f64(kd, vd, q, pos), enc
+
+
+def test_multi_stream_pass_over_trellis_rows(native, oracle):
+    from tolerances import assert_attn_close
+    layer = 1
+    blob = kvqp.synthetic(layers=2, kk=5, seed=13, mu=True)
+    kv, rows, rng = _streams(native, oracle, blob, layer)
+    with kv:
+        # one new row per stream, in any slot order; plus a row whose slot does not exist and one beyond its container
+        slots = np.array([2, 0, 4, 1, 3, 9, 1], np.int32)
+        pos = np.array([MS_LENS[s] if s < len(MS_LENS) else 5 for s in slots], np.int32)
+        pos[6] = MS_CTX
+        M = len(slots)
+        q = rng.standard_normal((M, NH, 256)).astype(np.float16)
+        kn = rng.standard_normal((M, KVH, 256)).astype(np.float16); vn = rng.standard_normal((M, KVH, 256)).astype(np.float16)
+        out = kv.ms_call(q, kn, vn, pos, slots)
+        assert not out[5:7].view(np.uint16).any()                       # rejected rows yield zeros
+        for t in range(5):
+            s = int(slots[t]); k, v, n = rows[s]
+            k[n] = kn[t]; v[n] = vn[t]
+            expect, enc = _stream_expect(oracle, blob, layer, k, v, n + 1, q[t:t + 1], n)
+            assert_attn_close(out[t:t + 1], expect, f"row {t} stream {s}")
+            kw, ks, vw, vs = kv.export_rows(s, n, 1)
+            for h in range(KVH):                                          # the row the pass stored for this stream: bit-exact
+                assert np.array_equal(kw[h, 0], enc[0, h]["words"][n, :40]) and np.array_equal(vw[h, 0], enc[1, h]["words"][n, :40])
+                assert _same(ks[h, 0:1], enc[0, h]["scale"][n:n + 1]) and _same(vs[h, 0:1], enc[1, h]["scale"][n:n + 1])
+        # rows of one stream that follow each other see each other's keys; attend only for the rest
+        slots = np.array([0, 0, 0, 2], np.int32); pos = np.array([301, 302, 303, 900], np.int32)
+        q = rng.standard_normal((4, NH, 256)).astype(np.float16)
+        kn = rng.standard_normal((4, KVH, 256)).astype(np.float16); vn = rng.standard_normal((4, KVH, 256)).astype(np.float16)
+        out = kv.ms_call(q, kn, vn, pos, slots)
+        k, v, _ = rows[0]
+        k[301:304] = kn[:3]; v[301:304] = vn[:3]
+        for t in range(3):
+            expect, _ = _stream_expect(oracle, blob, layer, k, v, 302 + t, q[t:t + 1], 301 + t)
+            assert_attn_close(out[t:t + 1], expect, f"stream 0 row {t}")

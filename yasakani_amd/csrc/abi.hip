@@ -31,11 +31,11 @@ struct yka_kv {
   size_t ws_rows = 0;              // capacity of the partial workspace in (token, split) pairs
   int* d_pos = nullptr;            // position used by the host-pointer hooks
   hipStream_t stream = nullptr;    // stream of the host-pointer hooks
-  int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0, opt_unrot = 0, opt_ctx_hint = 0;
+  int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0, opt_unrot = 0, opt_ctx_hint = 0, opt_profile_layer = 0;
   // trellis-coded rows (set by yka_kv_set_profile; head_dim 256 only): rows as the reference lays them out, per layer
   // [K payload n_kv * max_ctx * stride][V payload][K scales n_kv * max_ctx fp32][V scales]
   struct Tb {
-    int kb = 0, stride = 0, nm = 0; bool has_mu = false;
+    int kb = 0, stride = 0, nm = 0, layers = 0; bool has_mu = false;   // layers: layers the profile has groups for
     uint8_t* blob = nullptr; uint32_t* pairs = nullptr; float* gfac = nullptr; float* mu = nullptr;
     uint8_t* pool = nullptr; size_t layer_bytes = 0, pay_bytes = 0, scl_bytes = 0;
     uint8_t* scr = nullptr; size_t scr_w_ofs = 0;
@@ -106,11 +106,16 @@ void check_rows(const yka_kv* kv, int M) {
   if (M < 1 || M > kv->cfg.max_rows) throw std::runtime_error("M must be in [1, max_rows]");
 }
 
+void check_tb_layer(const yka_kv* kv, int layer) {
+  if (kv->tb && layer >= kv->tb->layers) throw std::runtime_error("the profile has no groups for this layer");
+}
 constexpr int kTbTileTok = 128;     // tokens per launch of the trellis encoder (its scratch holds that many)
 // trellis encoder over the rows of a pass: fp32 rows, or fp16 rows if k32 == nullptr
 void tb_append(yka_kv* kv, int layer, const float* k32, const float* v32, const uint16_t* k16, const uint16_t* v16, int M, const int* d_pos,
-               int rot, hipStream_t st, int pos_limit = 0) {
+               int rot, hipStream_t st, int pos_limit = 0, const RowMap* rows = nullptr) {
   const yka_kv::Tb& T = *kv->tb;
+  const int container = rows ? 0 : layer;            // multi-stream pass: containers are streams, `layer` only names the groups
+  check_tb_layer(kv, layer);
   for (int t0 = 0; t0 < M; t0 += kTbTileTok) {
     TbEncArgs A{};
     A.blob = T.blob; A.nm = T.nm; A.has_trellis = 1;
@@ -118,7 +123,8 @@ void tb_append(yka_kv* kv, int layer, const float* k32, const float* v32, const 
     A.max_ctx = kv->cfg.max_ctx; A.rot = rot; A.pos_limit = pos_limit;
     A.nrow = std::min(kTbTileTok, M - t0) * 2 * kv->cfg.n_kv_heads;
     A.scr = T.scr; A.scr_w_ofs = T.scr_w_ofs;
-    A.pay0 = T.kpay(layer); A.pay1 = T.vpay(layer); A.scl0 = T.kscl(layer); A.scl1 = T.vscl(layer); A.stride = T.stride;
+    A.pay0 = T.kpay(container); A.pay1 = T.vpay(container); A.scl0 = T.kscl(container); A.scl1 = T.vscl(container); A.stride = T.stride;
+    if (rows) A.rows = *rows;
     launch_tb_encode(A, st);
   }
 }
@@ -156,6 +162,7 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
     // trellis-coded rows: the encoder runs first (two launches); rows of at most 2 tokens (or option key 3) run on row
     // tiles of 2 tokens x 6 heads, wider slices on 128-row workgroups that decode every tile once into LDS
     const yka_kv::Tb& T = *kv->tb;
+    check_tb_layer(kv, layer);
     if (k16) do_append(kv, layer, k16, v16, M, d_pos, st);
     const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
     for (int s0 = 0; s0 < M; s0 += kMaxSlice) {
@@ -213,6 +220,26 @@ void do_attend_ms(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const ui
                   const int* row_slot, uint16_t* out16, hipStream_t st) {
   const int NH = kv->cfg.n_heads, D = kv->D();
   const bool r256 = kv->r256();
+  if (kv->tb) {
+    // trellis-coded rows: every container is a stream of the layer option key 6 names; its groups code and decode the rows
+    const yka_kv::Tb& T = *kv->tb;
+    const int pl = kv->opt_profile_layer;
+    check_tb_layer(kv, pl);
+    const RowMap R{row_pos, row_slot, kv->cfg.n_layers, T.layer_bytes, 0};
+    if (k16) tb_append(kv, pl, nullptr, nullptr, k16, v16, M, nullptr, 0, st, 0, &R);
+    for (int s0 = 0; s0 < M; s0 += kMaxSlice) {
+      const int Ms = std::min(kMaxSlice, M - s0);
+      int S = kv->opt_splits_narrow > 0 ? kv->opt_splits_narrow : 512 / (kv->cfg.n_kv_heads * Ms);
+      S = std::min(std::max(2, std::min(kMaxSplits, S)), (int)(kWsPairs / (size_t)Ms));
+      RowMap Rs = R; Rs.pos += s0; Rs.slot += s0;
+      const TbAttnArgs A{T.kpay(0), T.vpay(0), T.kscl(0), T.vscl(0), kv->cfg.max_ctx, kv->cfg.n_kv_heads, T.stride,
+                         T.pairs, T.gfac, T.has_mu ? T.mu : nullptr, pl, q16 + (size_t)s0 * NH * 256, nullptr, nullptr, Ms, s0, NH, S,
+                         kv->pm, kv->pl, kv->pacc16, Rs};
+      launch_attend_tb(A, T.kb, st);
+      launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, kv->opt_unrot}, st);
+    }
+    return;
+  }
   const RowMap R{row_pos, row_slot, kv->cfg.n_layers, kv->layer_bytes, kv->n_pages};
   if (k16) { const AppendArgs P{kv->view(0), k16, v16, nullptr, M, R}; if (r256) launch_append256(P, st); else launch_append(P, st); }
   for (int s0 = 0; s0 < M; s0 += kMaxSlice) {
@@ -313,6 +340,7 @@ int yka_set_opt(yka_kv* kv, int key, int value) {
     case 3: kv->opt_force_narrow = value != 0; break;
     case 4: kv->opt_unrot = value != 0; break;
     case 5: if (value < 0) throw std::runtime_error("context hint must be >= 0"); kv->opt_ctx_hint = value; break;
+    case 6: if (value < 0) throw std::runtime_error("profile layer must be >= 0"); kv->opt_profile_layer = value; break;
     default: throw std::runtime_error("unknown option key");
   }
   YKA_CATCH_INT
@@ -367,7 +395,7 @@ int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16
 int yka_append_attend_ms(yka_kv* kv, const uint16_t* d_q16, const uint16_t* d_k16, const uint16_t* d_v16, int M,
                          const int* d_row_pos, const int* d_row_slot, uint16_t* d_out16, void* hip_stream) {
   YKA_TRY
-  on_device(kv); no_trellis(kv); check_rows(kv, M);
+  on_device(kv); check_rows(kv, M);
   if (!d_q16 || !d_row_pos || !d_row_slot || !d_out16) throw std::runtime_error("null pointer");
   if ((d_k16 == nullptr) != (d_v16 == nullptr)) throw std::runtime_error("new K and V rows come together or not at all");
   do_attend_ms(kv, d_q16, d_k16, d_v16, M, d_row_pos, d_row_slot, d_out16, (hipStream_t)hip_stream);
@@ -378,7 +406,7 @@ int yka_append_attend_ms(yka_kv* kv, const uint16_t* d_q16, const uint16_t* d_k1
 int yka_ms_call_host(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, const int32_t* row_pos,
                      const int32_t* row_slot, uint16_t* out16) {
   YKA_TRY
-  on_device(kv); no_trellis(kv); check_rows(kv, M);
+  on_device(kv); check_rows(kv, M);
   if (!q16 || !row_pos || !row_slot || !out16) throw std::runtime_error("null pointer");
   if ((k16 == nullptr) != (v16 == nullptr)) throw std::runtime_error("new K and V rows come together or not at all");
   const size_t nq = (size_t)M * kv->cfg.n_heads * kv->D(), nk = (size_t)M * kv->cfg.n_kv_heads * kv->D();
@@ -560,8 +588,11 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
   if (kv->cfg.paged) throw std::runtime_error("trellis-coded rows are not available in paged mode");
   if (kv->tb) throw std::runtime_error("the handle already has a profile");
   const TbInfo I = tb_check_blob(blob, blob_len);
-  const int n_kv = kv->cfg.n_kv_heads, need = kv->cfg.n_layers * n_kv * 2;
-  if (I.kv_heads != n_kv || I.ngrp < need) throw std::runtime_error("the profile does not cover the layers and kv heads of the handle");
+  // The profile's layers are model layers.  A handle's containers are model layers too in single-stream use (a call then
+  // names a layer the profile must have) or the streams of ONE layer in multi-stream passes (option key 6 names it).
+  const int n_kv = kv->cfg.n_kv_heads;
+  if (I.kv_heads != n_kv || I.ngrp < n_kv * 2) throw std::runtime_error("the profile does not cover the kv heads of the handle");
+  const int need = (I.ngrp / (n_kv * 2)) * n_kv * 2;
   auto u16 = [&](size_t o) { return (unsigned)blob[o] | ((unsigned)blob[o + 1] << 8); };
   auto u32 = [&](size_t o) { return u16(o) | (u16(o + 2) << 16); };
   const size_t off_t = u32(36), off_g = u32(40);
@@ -608,7 +639,7 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
   } guard{kv};
   yka_kv::Tb* T = new yka_kv::Tb();
   kv->tb = T;
-  T->kb = kb; T->stride = 32 * kb; T->nm = I.nm; T->has_mu = has_mu;
+  T->kb = kb; T->stride = 32 * kb; T->nm = I.nm; T->has_mu = has_mu; T->layers = need / (n_kv * 2);
   const size_t rows = (size_t)n_kv * kv->cfg.max_ctx;
   T->pay_bytes = rows * T->stride; T->scl_bytes = rows * 4; T->layer_bytes = 2 * T->pay_bytes + 2 * T->scl_bytes;
   const size_t jobs = (size_t)kTbTileTok * 2 * n_kv * I.nm;

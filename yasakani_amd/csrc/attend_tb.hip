@@ -50,8 +50,11 @@ __device__ __forceinline__ h8 chunk_vals(const uint32_t* w, const uint8_t* tab) 
   return __builtin_bit_cast(h8, uint4{d[0], d[1], d[2], d[3]});
 }
 
-template <int KB>
+// MS: multi-stream pass (reference: src/q35_atxpk_ms.cu:13-33, which runs on packed rows) - one token per row tile, which
+// reads the container and the position its row map names
+template <int KB, bool MS>
 __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
+  constexpr int TPT = MS ? 1 : 2;                    // tokens per row tile
   constexpr int NW = 2 * KB;                         // words per chunk
   constexpr int kTabBytes = 4 << (8 + KB);           // one pair table
   constexpr int kAccBytes = 4 * 16 * (kD2 + 4) * 4;
@@ -65,12 +68,27 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
   const int gK = (A.layer * A.n_kv + kvh) * 2, gV = gK + 1;
-  const int pos = *A.d_pos;
-  const int tl = 2 * rt + i / kG;
-  const bool vrow = i < 2 * kG && tl < A.M;
+  int pos; bool row_ok = true;
+  if (MS) {
+    pos = A.rows.pos[rt];
+    const int slot = A.rows.slot[rt];
+    row_ok = pos >= 0 && pos < A.max_ctx && slot >= 0 && slot < A.rows.n_slots;   // a bad row reads nothing and yields zeros
+    const size_t off = row_ok ? (size_t)slot * A.rows.slot_bytes : 0;
+    A.kpay += off; A.vpay += off;
+    A.kscl = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(A.kscl) + off);
+    A.vscl = reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(A.vscl) + off);
+  } else {
+    pos = *A.d_pos;
+  }
+  const int tl = TPT * rt + i / kG;
+  const bool vrow = i < TPT * kG && tl < A.M && row_ok;
   const int head = kvh * kG + i % kG;
   int len = 0;
-  if (vrow) { const int tg = A.tok0 + tl; len = min(pos + (A.depth ? (int)A.depth[tg] : tg) + 1, A.max_ctx); }
+  if (vrow) {
+    if (MS) len = pos + 1;
+    else { const int tg = A.tok0 + tl; len = pos + (A.depth ? (int)A.depth[tg] : tg) + 1; }
+    len = min(len, A.max_ctx);
+  }
   int maxlen = len, minlen = vrow ? len : 0x7fffffff;
 #pragma unroll
   for (int o = 1; o < 16; o <<= 1) { maxlen = max(maxlen, __shfl_xor(maxlen, o, 64)); minlen = min(minlen, __shfl_xor(minlen, o, 64)); }
@@ -78,8 +96,8 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
   const int ntiles = (maxlen + 31) >> 5;
   const int s_used = min(A.S, max(1, ntiles >> 1));
   if (split >= s_used) {                             // the "no keys" marker; the combiner does not read such rows
-    const int j = threadIdx.x, tj = 2 * rt + j / kG;
-    if (j < 2 * kG && tj < A.M) {
+    const int j = threadIdx.x, tj = TPT * rt + j / kG;
+    if (j < TPT * kG && tj < A.M) {
       const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
       A.pm[p] = -1e30f; A.pl[p] = 0.f;
     }
@@ -285,16 +303,16 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
     L += __shfl_xor(L, 1, 64);
     L += __shfl_xor(L, 2, 64);
     s_wn[j][w] = L > 0.f ? ww * A.gfac[gV] / L : 0.f;
-    const int tj = 2 * rt + j / kG;
-    if (w == 0 && j < 2 * kG && tj < A.M) {
+    const int tj = TPT * rt + j / kG;
+    if (w == 0 && j < TPT * kG && tj < A.M) {
       const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
       A.pm[p] = M2; A.pl[p] = L;
     }
   }
   __syncthreads();
-  for (int idx = threadIdx.x; idx < 2 * kG * kD2; idx += 256) {
+  for (int idx = threadIdx.x; idx < TPT * kG * kD2; idx += 256) {
     const int j = idx >> 8, d = idx & (kD2 - 1);
-    const int tj = 2 * rt + j / kG;
+    const int tj = TPT * rt + j / kG;
     if (tj >= A.M) continue;
     const f4 w4 = *reinterpret_cast<const f4*>(s_wn[j]);
     const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
@@ -307,9 +325,15 @@ __global__ void __launch_bounds__(256, 2) attend_tb_kernel(TbAttnArgs A) {
 }  // namespace
 
 void launch_attend_tb(const TbAttnArgs& A, int kb, hipStream_t st) {
+  if (A.rows.pos) {
+    const dim3 grid(A.S, A.n_kv, A.M);
+    if (kb == 4) hipLaunchKernelGGL((attend_tb_kernel<4, true>), grid, dim3(256), 0, st, A);
+    else hipLaunchKernelGGL((attend_tb_kernel<5, true>), grid, dim3(256), 0, st, A);
+    return;
+  }
   const dim3 grid(A.S, A.n_kv, (A.M + 1) / 2);
-  if (kb == 4) hipLaunchKernelGGL(attend_tb_kernel<4>, grid, dim3(256), 0, st, A);
-  else hipLaunchKernelGGL(attend_tb_kernel<5>, grid, dim3(256), 0, st, A);
+  if (kb == 4) hipLaunchKernelGGL((attend_tb_kernel<4, false>), grid, dim3(256), 0, st, A);
+  else hipLaunchKernelGGL((attend_tb_kernel<5, false>), grid, dim3(256), 0, st, A);
 }
 
 }  // namespace yka

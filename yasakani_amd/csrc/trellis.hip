@@ -65,17 +65,27 @@ __device__ __forceinline__ float block_max(float* red, float v) {
   return t;
 }
 
-struct Row { float y; int g, pos; size_t out; int kind, kvh; };
+struct Row { float y; int g, pos; size_t out; int kind, kvh; size_t slot_off; bool ok; };
 // row rj of the launch, element d.  Probe form: rows with their own group and position.  Cache form: rj = (token, K|V, kv head)
 __device__ __forceinline__ Row tb_row(const TbEncArgs& A, int rj, int d, float* buf) {
   Row R;
   if (A.yin) {
     const int ri = A.row0 + rj;
     R.g = A.grp[ri]; R.pos = A.pos[ri]; R.y = A.yin[(size_t)ri * 256 + d]; R.out = (size_t)ri; R.kind = 0; R.kvh = 0;
+    R.slot_off = 0; R.ok = true;
   } else {
     const int tok = rj / (2 * A.n_kv), rem = rj - tok * 2 * A.n_kv;
     R.kind = rem / A.n_kv; R.kvh = rem - R.kind * A.n_kv;
-    R.pos = *A.d_pos + A.tok0 + tok; R.g = (A.layer * A.n_kv + R.kvh) * 2 + R.kind;
+    R.slot_off = 0; R.ok = true;
+    if (A.rows.pos) {                                                           // multi-stream pass: the row's own container and position
+      R.pos = A.rows.pos[A.tok0 + tok];
+      const int slot = A.rows.slot[A.tok0 + tok];
+      R.ok = slot >= 0 && slot < A.rows.n_slots;
+      R.slot_off = R.ok ? (size_t)slot * A.rows.slot_bytes : 0;
+    } else {
+      R.pos = *A.d_pos + A.tok0 + tok;
+    }
+    R.g = (A.layer * A.n_kv + R.kvh) * 2 + R.kind;
     const size_t e = ((size_t)(A.tok0 + tok) * A.n_kv + R.kvh) * 256 + d;
     R.y = A.k32 ? (R.kind ? A.v32 : A.k32)[e] : __half2float(__ushort_as_half((R.kind ? A.v16 : A.k16)[e]));
     R.out = (size_t)R.kvh * A.max_ctx + (size_t)max(0, min(R.pos, A.max_ctx - 1));
@@ -270,8 +280,9 @@ __global__ void __launch_bounds__(256) tb_select_kernel(TbEncArgs A) {
     if (P.has_mu) x = __fadd_rn(x, Q.mud);
     pc = (unsigned)__half_as_ushort(__float2half_rn(Q.cj0)) | ((unsigned)__half_as_ushort(__float2half_rn(Q.cj1)) << 16);
   }
-  const bool in_range = A.yin || (R.pos >= 0 && R.pos < A.max_ctx && (A.pos_limit == 0 || R.pos < A.pos_limit));
-  uint8_t* const payb = R.kind ? A.pay1 : A.pay0;
+  const bool in_range = A.yin || (R.ok && R.pos >= 0 && R.pos < A.max_ctx && (A.pos_limit == 0 || R.pos < A.pos_limit));
+  uint8_t* const payb0 = R.kind ? A.pay1 : A.pay0;
+  uint8_t* const payb = payb0 ? payb0 + R.slot_off : nullptr;
   if (payb && in_range) {
     uint32_t* const wrow = reinterpret_cast<uint32_t*>(payb + R.out * (size_t)A.stride);
     fld[d] = (uint8_t)field;
@@ -286,7 +297,7 @@ __global__ void __launch_bounds__(256) tb_select_kernel(TbEncArgs A) {
     }
     if (d == 0) {
       float* const scl = R.kind ? A.scl1 : A.scl0;
-      if (scl) scl[R.out] = psc;
+      if (scl) reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(scl) + R.slot_off)[R.out] = psc;
       if (A.side) { A.side[2 * R.out] = __float_as_uint(psc); A.side[2 * R.out + 1] = pc; }
       if (A.coded) A.coded[R.out] = pack ? 1 : 0;
     }

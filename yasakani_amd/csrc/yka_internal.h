@@ -94,6 +94,7 @@ struct TbEncArgs {
   uint8_t* scr; size_t scr_w_ofs;     // scratch: states [nrow * nm][256] bytes, then at scr_w_ofs error sums [nrow * nm][8] fp32
   uint8_t* pay0; uint8_t* pay1; float* scl0; float* scl1; int stride;
   int pos_limit;                      // cache form: rows at positions >= pos_limit are not stored (0: no limit besides max_ctx)
+  RowMap rows;                        // cache form, multi-stream pass: token t sits at rows.pos[t] of container rows.slot[t] (pay / scl = container 0)
 };
 // attention over trellis-coded rows (attend_tb.hip).  pairs [groups][2^(8 + kb)]: entry i = the table's integers, as two
 // fp16 values, of the states (i >> kb) & 255 and i & 255 (two consecutive elements from 8 + kb stream bits); gfac [groups]:
@@ -103,6 +104,7 @@ struct TbAttnArgs {
   const uint32_t* pairs; const float* gfac; const float* mu; int layer;
   const uint16_t* q16; const int* d_pos; const uint8_t* depth; int M, tok0, n_heads, S;
   float* pm; float* pl; uint16_t* pacc16;
+  RowMap rows;  // narrow kernel only: multi-stream pass (one token per workgroup column; kpay .. vscl = container 0, `layer` = the profile's layer)
 };
 void launch_attend_tb(const TbAttnArgs&, int kb, hipStream_t);        // row tiles of 2 tokens x 6 heads (decode; any width)
 void launch_attend_tb_wide(const TbAttnArgs&, int kb, hipStream_t);   // 3..64 rows: 128 query rows per workgroup, tiles decoded once into LDS
