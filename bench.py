@@ -137,7 +137,7 @@ def r256_figures(native, ctx=32768, L=16):
     return out
 
 
-def trellis_figures(native, ctx=32768, L=16, bits=5):
+def trellis_figures(native, ctx=32768, L=16, bits=5, torch=None):
     """Trellis-coded rows (the reference's KV5 / KV4 packed streams) under a synthetic profile of the production shape:
     4 x 2 x (32 * bits + 4) bytes per token per layer.  One layer call = trellis encoder for the new rows (two launches) +
     attention on row tiles of 2 tokens + combine; `encode_us` is what the encoder adds to a layer call."""
@@ -165,6 +165,11 @@ def trellis_figures(native, ctx=32768, L=16, bits=5):
         out[f"rows_{rows}"] = {"us_per_layer": us, "encode_us": us - float(np.median(ms1)) * 1e3 / L, "kernel_us": k_us,
                                "value_GBs": by / (us * 1e-6) / 1e9, "kernel_hbm_frac": by / (k_us * 1e-6) / 1e9 / HBM_PEAK_GBS,
                                "kernel_tflops": 4.0 * rows * NH * D2 * ctx / (k_us * 1e-6) / 1e12}
+    if torch is not None:
+        # batched decode: the containers as streams of profile layer 0, one row per stream (encoder + attention + combine)
+        kv.set_opt(6, 0)
+        out["batched_decode"] = batched_decode(torch, native, kv, ctx, L, k[4096:4097], v[4096:4097], q[:1], calls=100,
+                                               row_bytes=ctx * token_bytes + 2 * token_bytes + 2 * KVH * D2 * 2 + 2 * NH * D2 * 2)
     kv.close()
     return out
 
@@ -202,7 +207,7 @@ def big_configs(native):
     return out
 
 
-def batched_decode(torch, native, kv, ctx, L, k_new, v_new, q, calls=200):
+def batched_decode(torch, native, kv, ctx, L, k_new, v_new, q, calls=200, row_bytes=None):
     """Multi-stream passes on the containers already filled for the headline run: one row per stream, B streams at `ctx`
     cached tokens each (one pass = append + attention + combine for all B rows; B x 18.9 MB of KV)."""
     dev = torch.device("cuda:0")
@@ -231,7 +236,7 @@ def batched_decode(torch, native, kv, ctx, L, k_new, v_new, q, calls=200):
             fn(i)
         e1.record(); torch.cuda.synchronize()
         us = e0.elapsed_time(e1) * 1e3 / calls
-        by = B * algorithmic_bytes(ctx, 1)
+        by = B * (row_bytes if row_bytes else algorithmic_bytes(ctx, 1))
         out[f"streams_{B}"] = {"us_per_pass": us, "us_per_row": us / B, "value_GBs": by / (us * 1e-6) / 1e9,
                                "hbm_peak_frac": by / (us * 1e-6) / 1e9 / HBM_PEAK_GBS}
     return out
@@ -324,7 +329,7 @@ def main():
         print(json.dumps({"reference_rows_head_dim_256": r256_figures(native, args.ctx)}))
         return
     if args.trellis_only:
-        print(json.dumps({"trellis_rows": {f"bits_{b}": trellis_figures(native, args.ctx, bits=b) for b in (5, 4)}}))
+        print(json.dumps({"trellis_rows": {f"bits_{b}": trellis_figures(native, args.ctx, bits=b, torch=torch) for b in (5, 4)}}))
         return
     ctx, M, L = args.ctx, args.rows, args.layers
     max_ctx = ((ctx + 64 + 255) // 256) * 256
@@ -406,7 +411,7 @@ def main():
     if not args.no_extra:
         line["other_configs"] = big_configs(native)
         line["reference_rows_head_dim_256"] = r256_figures(native)
-        line["trellis_rows"] = {"bits_5": trellis_figures(native)}
+        line["trellis_rows"] = {"bits_5": trellis_figures(native, torch=torch)}
     print(json.dumps(line))
 
 
