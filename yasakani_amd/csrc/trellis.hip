@@ -240,6 +240,19 @@ __global__ void __launch_bounds__(256) tb_search_kernel(TbEncArgs A) {
   A.scr[job * 256 + d] = (uint8_t)st;
 }
 
+// word d of a row's MSB-first stream of KB-bit fields: the fields that overlap bits [32 d, 32 d + 32)
+template <int KB>
+__device__ __forceinline__ uint32_t pack_word(const uint8_t* fld, int d) {
+  const int e0 = (32 * d) / KB;                          // first field with bits in the word (division by a constant)
+  uint32_t w = 0u;
+#pragma unroll
+  for (int k = 0; k < 32 / KB + 2; ++k) {
+    const int e = e0 + k, sh = 32 * d + 32 - KB * (e + 1);   // distance of the field's last bit from the word's last bit
+    if (e < 256 && sh > -KB) w |= sh >= 0 ? (uint32_t)fld[e] << sh : (uint32_t)fld[e] >> -sh;
+  }
+  return w;
+}
+
 // grid rows, block 256: keeps the best multiplier (or runs the flat row quantizer), rebuilds the row, packs the fields
 __global__ void __launch_bounds__(256) tb_select_kernel(TbEncArgs A) {
   __shared__ float red[8];
@@ -290,9 +303,7 @@ __global__ void __launch_bounds__(256) tb_select_kernel(TbEncArgs A) {
     const int nw = A.stride >> 2;
     if (d < nw) {
       uint32_t w = 0u;
-      if (pack && d < 8 * kb) {
-        for (int i = 0; i < 32; ++i) { const int g = 32 * d + i; const int e = g / kb, jb = g - e * kb; w |= (((uint32_t)fld[e] >> (kb - 1 - jb)) & 1u) << (31 - i); }
-      }
+      if (pack && d < 8 * kb) w = kb == 5 ? pack_word<5>(fld, d) : kb == 4 ? pack_word<4>(fld, d) : pack_word<3>(fld, d);
       wrow[d] = w;
     }
     if (d == 0) {
