@@ -325,3 +325,42 @@ def test_multi_stream_pass_over_trellis_rows(native, oracle):
         for t in range(3):
             expect, _ = _stream_expect(oracle, blob, layer, k, v, 302 + t, q[t:t + 1], 301 + t)
             assert_attn_close(out[t:t + 1], expect, f"stream 0 row {t}")
+
+
+@pytest.mark.parametrize("kk", [5, 4])
+def test_full_length_32768_decode_and_window(native, oracle, kk):
+    """32,768 cached tokens (4,096 distinct rows tiled over the context): the rows the GPU stored are decoded by the oracle
+    and a decode step, a 3-row window (wide kernel) and the same window on row tiles are checked against fp64 attention."""
+    from tolerances import assert_attn_close
+    ctx, U, M = 32768, 4096, 3
+    blob = kvqp.synthetic(layers=1, kk=kk, seed=61, mu=True)
+    rng = np.random.default_rng(62 + kk)
+    k = rng.standard_normal((U + M, KVH, 256)).astype(np.float16); k[:, :, [5, 77, 130, 201]] *= 4
+    v = rng.standard_normal((U + M, KVH, 256)).astype(np.float16)
+    q = rng.standard_normal((M, NH, 256)).astype(np.float16)
+    with native.KvCache(head_dim=256, max_ctx=ctx + 256) as kv:
+        kv.set_profile(blob)
+        for p in range(0, ctx, 64):
+            s0 = p % U
+            kv.append_host(0, k[s0:s0 + 64], v[s0:s0 + 64], p)
+        dec1 = kv.layer_call(0, q[:1], k[U:U + 1], v[U:U + 1], ctx)
+        win = kv.layer_call(0, q, k[U:], v[U:], ctx)
+        kv.set_opt(3, 1)
+        win_tiles = kv.layer_call(0, q, None, None, ctx)
+        kw, ks, vw, vs = kv.export_rows(0, 0, U)
+        kw2, ks2, vw2, vs2 = kv.export_rows(0, ctx, M)
+        tail = kv.export_rows(0, ctx - U, U)
+    assert np.array_equal(tail[0], kw) and np.array_equal(tail[2], vw)          # the tiling repeats bit for bit
+    kd = np.empty((KVH, ctx + M, 256), np.float32); vd = np.empty_like(kd)
+    for h in range(KVH):
+        for kind, w, s, w2, s2, dst in ((0, kw, ks, kw2, ks2, kd), (1, vw, vs, vw2, vs2, vd)):
+            g = np.full(U + M, h * 2 + kind, np.int32)
+            words = np.zeros((U + M, 40), np.uint32)
+            words[:U, :8 * kk] = w[h]; words[U:, :8 * kk] = w2[h]
+            rows = oracle.tb_decode_rows(blob, g, words, np.concatenate([s[h], s2[h]]), np.zeros(U + M, np.uint32))
+            dst[h, :ctx] = np.tile(rows[:U], (ctx // U, 1)); dst[h, ctx:] = rows[U:]
+    expect = oracle.tb_attend_f64(kd, vd, q, ctx)
+    assert_attn_close(dec1, expect[:1], f"decode kk={kk}")
+    assert_attn_close(win, expect, f"window kk={kk}")
+    assert_attn_close(win_tiles, expect, f"window on row tiles kk={kk}")
+    assert np.abs(win.astype(np.float64) - expect).max() <= 2e-3                # the plain absolute bar at the measured size
