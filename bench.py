@@ -363,7 +363,7 @@ def main():
         return
     us, gbs, roof, out = measure(M, args.steps, args.warmup)
     line = {
-        # the headline workload carries BASELINE.json's metric text verbatim; `value` is its effective-KV-GB/s component,
+        # the headline workload carries the published metric's text verbatim; `value` is its effective-KV-GB/s component,
         # `us_per_layer` and `hbm_peak_frac` are the other two
         "metric": ("\u00b5s/layer + effective KV GB/s (% HBM peak), int4-KV GQA verify-64 at 32k ctx" if (M, ctx) == (64, 32768) else
                    f"\u00b5s/layer + effective KV GB/s (% HBM peak), int4-KV GQA verify-{M} at {ctx} ctx" if M > 1 else
