@@ -29,7 +29,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the dominant kernel from two `rocprofv3 --pmc` runs (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00,
 # factors from a 256 MiB copy in the same runs; see profiles/attend_*_ctx32768.md).  Keyed by (rows, ctx, containers
 # irrelevant); any other workload reports null.
-MEASURED_TRAFFIC_BYTES = {(64, 32768): 39.9e6, (1, 32768): 20.1e6}
+MEASURED_TRAFFIC_BYTES = {(64, 32768): 39.9e6, (1, 32768): 19.6e6}
 
 
 def algorithmic_bytes(ctx, M):
