@@ -192,3 +192,28 @@ def test_blob_checks():
     P = kvqp.parse(blob)
     assert P["dim"] == 256 and len(P["groups"]) == 8 and P["groups"][0]["kk"] == 5
     assert yko.tb_group(blob, 5) == {k: P["groups"][5][k] for k in ("mode", "kk", "table", "guard", "m", "has_mu")}
+
+
+def test_attention_over_decoded_rows_closed_forms():
+    """tb_attend_f64 (textbook softmax(QK^T/16)V in fp64 on decoded rows): uniform V rows give that row; one dominant key
+    gives its V row; a row sees exactly the keys up to its own position"""
+    rng = np.random.default_rng(12)
+    n, M = 40, 3
+    k = rng.standard_normal((4, n, 256)).astype(np.float32)
+    v = np.tile(rng.standard_normal((4, 1, 256)).astype(np.float32), (1, n, 1))
+    q = rng.standard_normal((M, 24, 256)).astype(np.float16)
+    out = yko.tb_attend_f64(k, v, q, n - M)
+    for h in range(24):
+        assert np.allclose(out[:, h], v[h // 6, 0], atol=1e-12)
+    v = rng.standard_normal((4, n, 256)).astype(np.float32)
+    k2 = k.copy(); k2[:, 7] = 0
+    for h in range(4):
+        k2[h, 7] = 50 * q[0, 6 * h].astype(np.float32) / np.linalg.norm(q[0, 6 * h].astype(np.float32))
+    out = yko.tb_attend_f64(k2, v, q[:1], n - 1)
+    for h in range(4):
+        assert np.allclose(out[0, 6 * h], v[h, 7], atol=1e-6)
+    # causal window: changing a key beyond a row's own position changes nothing for that row
+    base = yko.tb_attend_f64(k, v, q, n - M)
+    k3 = k.copy(); k3[:, n - 1] += 5
+    moved = yko.tb_attend_f64(k3, v, q, n - M)
+    assert np.array_equal(base[:M - 1], moved[:M - 1]) and not np.array_equal(base[M - 1], moved[M - 1])
