@@ -364,3 +364,28 @@ def test_full_length_32768_decode_and_window(native, oracle, kk):
     assert_attn_close(win, expect, f"window kk={kk}")
     assert_attn_close(win_tiles, expect, f"window on row tiles kk={kk}")
     assert np.abs(win.astype(np.float64) - expect).max() <= 2e-3                # the plain absolute bar at the measured size
+
+
+def test_pass_wider_than_a_slice(native, oracle):
+    """200 rows in one call: the encoder runs in tiles of 128 tokens, attention in 64-row slices, later rows see the keys
+    of earlier rows of the same pass"""
+    from tolerances import assert_attn_close
+    blob = kvqp.synthetic(layers=1, kk=4, seed=33)
+    ctx, M = 300, 200
+    k, v = _kv_rows(34, ctx + M)
+    k16, v16 = k[ctx:].astype(np.float16), v[ctx:].astype(np.float16)
+    k[ctx:] = k16; v[ctx:] = v16
+    q = np.random.default_rng(35).standard_normal((M, NH, 256)).astype(np.float16)
+    with native.KvCache(head_dim=256, max_ctx=512, max_rows=256) as kv:
+        kv.set_profile(blob)
+        for p in range(0, ctx, 64):
+            m = min(64, ctx - p)
+            kv.append256_f32_host(0, k[p:p + m], v[p:p + m], p, rotate=False)
+        out = kv.layer_call(0, q, k16, v16, ctx)
+        kw, ks, vw, vs = kv.export_rows(0, 0, ctx + M)
+    enc = _oracle_rows(oracle, blob, 0, k, v)
+    for h in range(KVH):
+        assert np.array_equal(kw[h], enc[0, h]["words"][:, :32]) and np.array_equal(vw[h], enc[1, h]["words"][:, :32]), h
+        assert _same(ks[h], enc[0, h]["scale"]) and _same(vs[h], enc[1, h]["scale"])
+    kd = np.stack([enc[0, h]["x"] for h in range(KVH)]); vd = np.stack([enc[1, h]["x"] for h in range(KVH)])
+    assert_attn_close(out, oracle.tb_attend_f64(kd, vd, q, ctx), "200-row pass")
