@@ -159,3 +159,29 @@ def test_output_step_gate_hadamard_int8(native, oracle):
     assert np.allclose(alpha, ra, rtol=2e-3, atol=0)
     diff = np.abs(qx.astype(np.int32) - rq.astype(np.int32))
     assert diff.max() <= 1 and (diff != 0).mean() < 0.01, (diff.max(), (diff != 0).mean())
+
+
+@pytest.mark.parametrize("M", [1, 16, 64])
+def test_full_length_32768(native, oracle, M):
+    """32,768 cached tokens (4,096 distinct rows tiled over the context): decode, and windows on the 128-row workgroups,
+    against the threaded oracle on the cache image the GPU built"""
+    ctx, U = 32768, 4096
+    rng = np.random.default_rng(3300 + M)
+    k = rng.standard_normal((U + M, KVH, D)).astype(np.float32); k[:, :, [5, 77, 130, 201]] *= 8
+    k = k.astype(np.float16)
+    v = rng.standard_normal((U + M, KVH, D)).astype(np.float16)
+    q = rng.standard_normal((M, NH, D)).astype(np.float16)
+    ref = oracle.Cache(ctx + 256, NH, KVH, D)
+    with native.KvCache(head_dim=D, max_ctx=ctx + 256) as kv:
+        for p in range(0, ctx, 64):
+            s0 = p % U
+            kv.append_host(0, k[s0:s0 + 64], v[s0:s0 + 64], p)
+        out = kv.layer_call(0, q, k[U:], v[U:], ctx)
+        kw, ks, vw, vs = kv.export_rows(0, 0, ctx + M)
+    ref.kc[:, :ctx + M], ref.ks[:, :ctx + M], ref.vc[:, :ctx + M], ref.vs[:, :ctx + M] = kw, ks, vw, vs
+    chk = oracle.Cache(256, NH, KVH, D)                    # the image is what the oracle's quantizer gives (first rows)
+    chk.append(k[:200], v[:200], 0)
+    assert np.array_equal(chk.kc[:, :200], kw[:, :200]) and np.array_equal(chk.vs[:, :200].view(np.uint32), vs[:, :200].view(np.uint32))
+    expect = ref.attend_f32(q, ctx, threads=16, want_f32=True)[1]
+    assert_attn_close(out, expect, f"32k M={M}")
+    assert np.abs(out.astype(np.float64) - expect).max() <= 2e-3
