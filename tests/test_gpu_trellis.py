@@ -389,3 +389,40 @@ def test_pass_wider_than_a_slice(native, oracle):
         assert _same(ks[h], enc[0, h]["scale"]) and _same(vs[h], enc[1, h]["scale"])
     kd = np.stack([enc[0, h]["x"] for h in range(KVH)]); vd = np.stack([enc[1, h]["x"] for h in range(KVH)])
     assert_attn_close(out, oracle.tb_attend_f64(kd, vd, q, ctx), "200-row pass")
+
+
+def test_engine_shaped_sequence_post_attend_unrotate(native, oracle):
+    """the sequence a caller with the engine's head size runs on packed rows: yka_attn_post with rotation (norm, rotary,
+    rotation, trellis encoder), attention over the rotated rows, outputs rotated back by the combiner (option key 4)"""
+    from tolerances import assert_attn_close
+    blob = kvqp.synthetic(layers=1, kk=5, seed=29)
+    rng = np.random.default_rng(30)
+    ctx, M, rd = 400, 4, 64
+    n = ctx + M
+    xq = rng.standard_normal((M, NH, 256)).astype(np.float32)
+    xk = (rng.standard_normal((n, KVH, 256)) * 0.8).astype(np.float32); xk[:, :, [5, 77, 130, 201]] *= 6
+    xv = rng.standard_normal((n, KVH, 256)).astype(np.float32)
+    qw = (rng.standard_normal(256) * 0.1).astype(np.float16).view(np.uint16)
+    kw_ = (rng.standard_normal(256) * 0.1).astype(np.float16).view(np.uint16)
+    rope = oracle.rope_table(512, rd)
+    zq = np.zeros((64, NH, 256), np.float32)
+    with native.KvCache(head_dim=256, max_ctx=512) as kv:
+        kv.set_profile(blob)
+        kv.set_opt(4, 1)
+        for p in range(0, ctx, 64):                              # cached rows: the same step, their Q rows are not needed
+            m = min(64, ctx - p)
+            kv.attn_post_host(0, zq[:m], xk[p:p + m], xv[p:p + m], p, qw, kw_, 1e-6, rope, rd, rotate=True)
+        q16 = kv.attn_post_host(0, xq, xk[ctx:], xv[ctx:], ctx, qw, kw_, 1e-6, rope, rd, rotate=True)
+        out = kv.layer_call(0, q16, None, None, ctx)
+    # oracle: the post step row by row position, the encoder, fp64 attention in the rotated basis, inverse rotation
+    k32 = np.empty((n, KVH, 256), np.float32); v32 = np.empty_like(k32)
+    for p in range(0, n, 64):
+        m = min(64, n - p)
+        _, k32[p:p + m], v32[p:p + m] = oracle.attn_post256(np.zeros((m, NH, 256), np.float32), xk[p:p + m], xv[p:p + m], qw, kw_, 1e-6, rope, rd, p, 1)
+    ref_q, _, _ = oracle.attn_post256(xq, xk[ctx:], xv[ctx:], qw, kw_, 1e-6, rope, rd, ctx, 1)
+    assert np.array_equal(q16.view(np.uint16), ref_q)
+    enc = _oracle_rows(oracle, blob, 0, k32, v32)
+    kd = np.stack([enc[0, h]["x"] for h in range(KVH)]); vd = np.stack([enc[1, h]["x"] for h in range(KVH)])
+    rotated = oracle.tb_attend_f64(kd, vd, ref_q, ctx)
+    expect = oracle.kvx_rotate256(rotated.reshape(-1, 256).astype(np.float32), inverse=True).reshape(M, NH, 256)
+    assert_attn_close(out, expect, "post -> encoder -> attention -> inverse rotation")
