@@ -20,95 +20,129 @@
 namespace yka {
 namespace {
 
-__device__ __forceinline__ unsigned tb_u16(const uint8_t* p) { return (unsigned)p[0] | ((unsigned)p[1] << 8); }
-__device__ __forceinline__ unsigned tb_u32(const uint8_t* p) { return tb_u16(p) | (tb_u16(p + 2) << 16); }
-__device__ __forceinline__ float tb_f32(const uint8_t* p) { return __uint_as_float(tb_u32(p)); }
-__device__ __forceinline__ float tb_h2f(unsigned h) { return __half2float(__ushort_as_half((unsigned short)h)); }
+// ---- the profile blob, read where it lies (little-endian, no alignment assumed) ----
+struct Profile {
+  const uint8_t* base;
+  __device__ unsigned half_at(unsigned off) const { return base[off] | ((unsigned)base[off + 1] << 8); }
+  __device__ unsigned word_at(unsigned off) const { return half_at(off) | (half_at(off + 2) << 16); }
+  __device__ float float_at(unsigned off) const { return __uint_as_float(word_at(off)); }
+  __device__ float f16_at(unsigned off) const { return __half2float(__ushort_as_half((unsigned short)half_at(off))); }
+  __device__ int multipliers() const { return (int)half_at(24); }
+  __device__ unsigned groups() const { return word_at(28); }
+  __device__ float multiplier(int i) const { return float_at(word_at(32) + 4u * (unsigned)i); }
+  __device__ unsigned table_record(int t) const { return word_at(word_at(36) + 4u * (unsigned)t); }
+  __device__ unsigned group_record(int g) const { return word_at(word_at(40) + 4u * (unsigned)g); }
+};
+// what a group record says; `present` is false for a group index the profile does not have
+struct GroupRec {
+  bool present; int mode, bits, table, guard, ndir; bool has_mean;
+  unsigned mean_off, dir_off;            // byte offsets of the fp16 mean row and of the first fp16 direction
+};
+__device__ __forceinline__ GroupRec read_group(const Profile& P, int g) {
+  GroupRec G{};
+  G.present = (unsigned)g < P.groups();
+  G.bits = 4;
+  if (G.present) {
+    const unsigned rec = P.group_record(g);
+    G.mode = P.base[rec]; G.bits = P.base[rec + 1]; G.table = P.base[rec + 2]; G.guard = P.base[rec + 3];
+    G.ndir = P.base[rec + 4]; G.has_mean = P.base[rec + 5] != 0;
+    G.mean_off = rec + 8; G.dir_off = G.mean_off + (G.has_mean ? 512u : 0u);
+  }
+  return G;
+}
+// table of a trellis group: value of state s = (int16 at values + 2 s) / 256 * gain, each product rounded to fp32
+struct TableRec { unsigned values; float gain; };
+__device__ __forceinline__ TableRec read_table(const Profile& P, const GroupRec& G) {
+  const unsigned rec = P.table_record(G.table);
+  return TableRec{rec + 12u, P.float_at(rec + 4u)};
+}
+__device__ __forceinline__ int table_int(const Profile& P, const TableRec& T, int state) { return (int)(short)P.half_at(T.values + 2u * (unsigned)state); }
+__device__ __forceinline__ float table_value(int ti, float gain) { return __fmul_rn(__fmul_rn((float)ti, 1.f / 256.f), gain); }
+
 // fp32 value -> nearest fp16 -> fp32.  The empty asm keeps the compiler from merging the operation that produced v with the
 // conversion into one mixed-precision instruction, which would skip the fp32 rounding the reference performs in between
-__device__ __forceinline__ float tb_f16r(float v) { asm volatile("" : "+v"(v)); return __half2float(__float2half_rn(v)); }
-__device__ __forceinline__ float tb_cdec(int ci, float gain) { return __fmul_rn(__fmul_rn((float)ci, 0.00390625f), gain); }
+__device__ __forceinline__ float round_f16(float v) { asm volatile("" : "+v"(v)); return __half2float(__float2half_rn(v)); }
 
-struct Group { int nm, mode, kk, tix, guard, m, has_mu; unsigned go, off_m, off_t; bool ok; };
-__device__ __forceinline__ Group tb_group(const uint8_t* b, int g) {
-  Group P;
-  P.nm = (int)tb_u16(b + 24); P.off_m = tb_u32(b + 32); P.off_t = tb_u32(b + 36);
-  const unsigned off_g = tb_u32(b + 40), ngrp = tb_u32(b + 28);
-  P.ok = (unsigned)g < ngrp;
-  P.go = P.ok ? tb_u32(b + off_g + 4u * (unsigned)g) : 0u;
-  P.mode = P.ok ? b[P.go] : 0; P.kk = P.ok ? b[P.go + 1] : 4; P.tix = P.ok ? b[P.go + 2] : 0; P.guard = P.ok ? b[P.go + 3] : 0;
-  P.m = P.ok ? b[P.go + 4] : 0; P.has_mu = P.ok ? b[P.go + 5] : 0;
-  return P;
+// Reduction over the 256 threads of a block in the order the reference fixes (src/kvq_fast.cuh:31-52): inside each run of
+// 32 elements the butterfly a[i] = op(a[i], a[i ^ o]), o = 16 .. 1, then the 8 run results folded in order from `start`.
+struct AddRn { __device__ static float op(float a, float b) { return __fadd_rn(a, b); } };
+struct MaxOp { __device__ static float op(float a, float b) { return fmaxf(a, b); } };
+template <class Op>
+__device__ __forceinline__ float block_fold(float* part8, float v, float start) {
+#pragma unroll
+  for (int o = 16; o; o >>= 1) v = Op::op(v, __shfl_xor(v, o, 64));         // partners stay inside a half of the wave
+  const int run = threadIdx.x >> 5;
+  if ((threadIdx.x & 31) == 0) part8[run] = v;
+  __syncthreads();
+  float acc = start;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) acc = Op::op(acc, part8[k]);
+  __syncthreads();
+  return acc;
 }
 
-// sum over the 256 threads of a block in the reference's order (tbf_sum, src/kvq_fast.cuh:31-40); red: 8 floats
-__device__ __forceinline__ float block_sum(float* red, float v) {
-#pragma unroll
-  for (int o = 16; o; o >>= 1) v = __fadd_rn(v, __shfl_xor(v, o, 64));     // stays inside each half of the wave
-  if ((threadIdx.x & 31) == 0) red[threadIdx.x >> 5] = v;
-  __syncthreads();
-  float t = 0.f;
-#pragma unroll
-  for (int w = 0; w < 8; ++w) t = __fadd_rn(t, red[w]);
-  __syncthreads();
-  return t;
-}
-__device__ __forceinline__ float block_max(float* red, float v) {
-#pragma unroll
-  for (int o = 16; o; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  if ((threadIdx.x & 31) == 0) red[threadIdx.x >> 5] = v;
-  __syncthreads();
-  float t = 0.f;
-#pragma unroll
-  for (int w = 0; w < 8; ++w) t = fmaxf(t, red[w]);
-  __syncthreads();
-  return t;
-}
-
-struct Row { float y; int g, pos; size_t out; int kind, kvh; size_t slot_off; bool ok; };
-// row rj of the launch, element d.  Probe form: rows with their own group and position.  Cache form: rj = (token, K|V, kv head)
-__device__ __forceinline__ Row tb_row(const TbEncArgs& A, int rj, int d, float* buf) {
-  Row R;
+// ---- which row a block works on ----
+struct RowRef {
+  float x;             // element threadIdx.x of the row (after the optional rotation)
+  int group, pos;      // profile group and position
+  size_t index;        // probe form: the row's index in the arrays; cache form: kv head * max_ctx + position
+  int is_v;            // cache form: 0 K row, 1 V row
+  size_t container;    // cache form, multi-stream pass: byte offset of the row's container
+  bool valid;          // multi-stream pass: false if the row names no container
+};
+// Probe form: rows with their own group and position.  Cache form: row r of the launch = (token r / (2 n_kv), K | V, kv head)
+__device__ __forceinline__ RowRef locate_row(const TbEncArgs& A, int r, float* rot_buf) {
+  const int d = threadIdx.x;
+  RowRef R{};
+  R.valid = true;
   if (A.yin) {
-    const int ri = A.row0 + rj;
-    R.g = A.grp[ri]; R.pos = A.pos[ri]; R.y = A.yin[(size_t)ri * 256 + d]; R.out = (size_t)ri; R.kind = 0; R.kvh = 0;
-    R.slot_off = 0; R.ok = true;
+    R.index = (size_t)(A.row0 + r);
+    R.group = A.grp[R.index]; R.pos = A.pos[R.index]; R.x = A.yin[R.index * 256 + d];
   } else {
-    const int tok = rj / (2 * A.n_kv), rem = rj - tok * 2 * A.n_kv;
-    R.kind = rem / A.n_kv; R.kvh = rem - R.kind * A.n_kv;
-    R.slot_off = 0; R.ok = true;
-    if (A.rows.pos) {                                                           // multi-stream pass: the row's own container and position
-      R.pos = A.rows.pos[A.tok0 + tok];
-      const int slot = A.rows.slot[A.tok0 + tok];
-      R.ok = slot >= 0 && slot < A.rows.n_slots;
-      R.slot_off = R.ok ? (size_t)slot * A.rows.slot_bytes : 0;
+    const int per_tok = 2 * A.n_kv, tok = A.tok0 + r / per_tok, within = r % per_tok;
+    R.is_v = within / A.n_kv;
+    const int kvh = within % A.n_kv;
+    if (A.rows.pos) {                                  // multi-stream pass: the row's own container and position
+      const int slot = A.rows.slot[tok];
+      R.pos = A.rows.pos[tok];
+      R.valid = slot >= 0 && slot < A.rows.n_slots;
+      R.container = R.valid ? (size_t)slot * A.rows.slot_bytes : 0;
     } else {
-      R.pos = *A.d_pos + A.tok0 + tok;
+      R.pos = *A.d_pos + tok;
     }
-    R.g = (A.layer * A.n_kv + R.kvh) * 2 + R.kind;
-    const size_t e = ((size_t)(A.tok0 + tok) * A.n_kv + R.kvh) * 256 + d;
-    R.y = A.k32 ? (R.kind ? A.v32 : A.k32)[e] : __half2float(__ushort_as_half((R.kind ? A.v16 : A.k16)[e]));
-    R.out = (size_t)R.kvh * A.max_ctx + (size_t)max(0, min(R.pos, A.max_ctx - 1));
+    R.group = (A.layer * A.n_kv + kvh) * 2 + R.is_v;
+    const size_t src = ((size_t)tok * A.n_kv + kvh) * 256 + d;
+    R.x = A.k32 ? (R.is_v ? A.v32 : A.k32)[src] : __half2float(__ushort_as_half((R.is_v ? A.v16 : A.k16)[src]));
+    R.index = (size_t)kvh * A.max_ctx + (size_t)max(0, min(R.pos, A.max_ctx - 1));
   }
-  if (A.rot) R.y = rotate256(R.y, buf, false);
+  if (A.rot) R.x = rotate256(R.x, rot_buf, false);
   return R;
 }
 
-struct Pre { float r, mud, cj0, cj1, uj0, uj1, rms; };
-__device__ __forceinline__ Pre tb_pre(float* red, const uint8_t* b, const Group& P, float y) {
-  const int d = threadIdx.x;
-  const uint8_t* mup = b + P.go + 8;
-  const uint8_t* Up = mup + (P.has_mu ? 512 : 0);
-  Pre Q; Q.mud = 0.f; Q.cj0 = Q.cj1 = Q.uj0 = Q.uj1 = 0.f;
-  float r = y;
-  if (P.has_mu) { Q.mud = tb_h2f(tb_u16(mup + 2 * d)); r = __fsub_rn(y, Q.mud); }
-  if (P.m > 0) { Q.uj0 = tb_h2f(tb_u16(Up + 2 * d));         Q.cj0 = tb_f16r(block_sum(red, __fmul_rn(r, Q.uj0))); r = __fsub_rn(r, __fmul_rn(Q.cj0, Q.uj0)); }
-  if (P.m > 1) { Q.uj1 = tb_h2f(tb_u16(Up + 2 * (256 + d))); Q.cj1 = tb_f16r(block_sum(red, __fmul_rn(r, Q.uj1))); r = __fsub_rn(r, __fmul_rn(Q.cj1, Q.uj1)); }
-  const float ssq = block_sum(red, __fmul_rn(r, r));
-  float rms = sqrtf(__fdiv_rn(ssq, 256.f));
-  if (rms == 0.f) rms = 1.f;
-  Q.r = r; Q.rms = rms;
+// ---- the step before coding (src/kvq_fast.cuh:63-76): remove the mean row, project out up to two directions with
+//      coefficients rounded to fp16, measure the rms of what is left ----
+struct Residual { float r, mean, coef[2], dir[2], rms; };
+__device__ __forceinline__ Residual residual_of(float* part8, const Profile& P, const GroupRec& G, float x) {
+  const unsigned d = threadIdx.x;
+  Residual Q{};
+  Q.r = x;
+  if (G.has_mean) { Q.mean = P.f16_at(G.mean_off + 2u * d); Q.r = __fsub_rn(x, Q.mean); }
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {                        // at most two directions; the test is uniform over the block (barriers inside)
+    if (k >= G.ndir) break;
+    Q.dir[k] = P.f16_at(G.dir_off + 512u * (unsigned)k + 2u * d);
+    Q.coef[k] = round_f16(block_fold<AddRn>(part8, __fmul_rn(Q.r, Q.dir[k]), 0.f));
+    Q.r = __fsub_rn(Q.r, __fmul_rn(Q.coef[k], Q.dir[k]));
+  }
+  const float mean_sq = __fdiv_rn(block_fold<AddRn>(part8, __fmul_rn(Q.r, Q.r), 0.f), 256.f);
+  Q.rms = sqrtf(mean_sq);                              // sqrtf is correctly rounded on this target
+  if (Q.rms == 0.f) Q.rms = 1.f;
   return Q;
+}
+// scale tried for multiplier i: rms * multiplier rounded to fp32, then to fp16; 0 -> 1
+__device__ __forceinline__ float trial_scale(const Profile& P, float rms, int i) {
+  const float s = round_f16(__fmul_rn(rms, P.multiplier(i)));
+  return s == 0.f ? 1.f : s;
 }
 
 // min over the lane pair (l, l ^ O) without an LDS round trip: a row rotation for O = 8, the gfx950 row / half swaps for
@@ -199,45 +233,38 @@ __device__ __forceinline__ void wave_chunk(const int* xi, const int (&ci4)[4], u
 // grid rows * nm, block 256: block = (row, multiplier); wave c = chunk c.  Writes the 256 states of the row under this
 // multiplier and the 8 partial error sums to scratch.
 __global__ void __launch_bounds__(256) tb_search_kernel(TbEncArgs A) {
-  __shared__ float red[8];
-  __shared__ float buf[256];
-  __shared__ int xi[256];
-  __shared__ uint8_t bp[4][64 * 32];
-  __shared__ uint8_t stv[256];
+  __shared__ float part8[8];
+  __shared__ float rot_buf[256];
+  __shared__ int target[256];
+  __shared__ uint8_t back[4][64 * 32];
+  __shared__ uint8_t chosen[256];
   const int d = threadIdx.x, wave = d >> 6, lane = d & 63;
-  const int rj = blockIdx.x / A.nm, mi = blockIdx.x - rj * A.nm;
-  const uint8_t* b = A.blob;
-  const Row R = tb_row(A, rj, d, buf);
-  const Group P = tb_group(b, R.g);
-  if (!P.ok || R.pos < P.guard || P.mode != 0) return;                     // uniform over the block
-  const Pre Q = tb_pre(red, b, P, R.y);
-  const unsigned to = tb_u32(b + P.off_t + 4u * (unsigned)P.tix);
-  const float gain = tb_f32(b + to + 4);
-  float s = tb_f16r(__fmul_rn(Q.rms, tb_f32(b + P.off_m + 4u * (unsigned)mi)));
-  if (s == 0.f) s = 1.f;
-  {
-    const float t = rintf(__fmul_rn(__fdiv_rn(Q.r, s), 256.f));
-    xi[d] = (int)fminf(fmaxf(t, -2048.f), 2048.f);
-  }
+  const int row = blockIdx.x / A.nm, mult = blockIdx.x % A.nm;
+  const Profile P{A.blob};
+  const RowRef R = locate_row(A, row, rot_buf);
+  const GroupRec G = read_group(P, R.group);
+  if (!G.present || R.pos < G.guard || G.mode != 0) return;                // uniform over the block: nothing to search
+  const Residual Q = residual_of(part8, P, G, R.x);
+  const TableRec T = read_table(P, G);
+  const float s = trial_scale(P, Q.rms, mult);
+  // integer target of element d: the residual in units of s / 256, clamped
+  target[d] = (int)fminf(fmaxf(rintf(__fmul_rn(__fdiv_rn(Q.r, s), 256.f)), -2048.f), 2048.f);
   int ci4[4];
 #pragma unroll
-  for (int k = 0; k < 4; ++k) ci4[k] = (int)(short)tb_u16(b + to + 12 + 2 * (lane + 64 * k));
+  for (int k = 0; k < 4; ++k) ci4[k] = table_int(P, T, lane + 64 * k);
   __syncthreads();
-  switch (P.kk) {
-    case 3: wave_chunk<3>(xi + 64 * wave, ci4, bp[wave], stv + 64 * wave); break;
-    case 4: wave_chunk<4>(xi + 64 * wave, ci4, bp[wave], stv + 64 * wave); break;
-    default: wave_chunk<5>(xi + 64 * wave, ci4, bp[wave], stv + 64 * wave); break;
-  }
-  // error of the chunk under this multiplier: element d of the row is lane `lane` of wave `wave`
-  const int st = stv[d];
-  const float rec = __fmul_rn(tb_cdec((int)(short)tb_u16(b + to + 12 + 2 * st), gain), s);
-  const float dd = __fsub_rn(Q.r, rec);
-  float v = __fmul_rn(dd, dd);
+  if (G.bits == 5) wave_chunk<5>(target + 64 * wave, ci4, back[wave], chosen + 64 * wave);
+  else if (G.bits == 4) wave_chunk<4>(target + 64 * wave, ci4, back[wave], chosen + 64 * wave);
+  else wave_chunk<3>(target + 64 * wave, ci4, back[wave], chosen + 64 * wave);
+  // squared error of this multiplier: element d of the row is lane `lane` of wave `wave`; summed per run of 32 elements
+  const int state = chosen[d];
+  const float miss = __fsub_rn(Q.r, __fmul_rn(table_value(table_int(P, T, state), T.gain), s));
+  float sq = __fmul_rn(miss, miss);
 #pragma unroll
-  for (int o = 16; o; o >>= 1) v = __fadd_rn(v, __shfl_xor(v, o, 64));
-  const size_t job = (size_t)rj * A.nm + mi;
-  if ((d & 31) == 0) reinterpret_cast<float*>(A.scr + A.scr_w_ofs)[job * 8 + (d >> 5)] = v;
-  A.scr[job * 256 + d] = (uint8_t)st;
+  for (int o = 16; o; o >>= 1) sq = __fadd_rn(sq, __shfl_xor(sq, o, 64));
+  const size_t job = (size_t)row * A.nm + mult;
+  if ((d & 31) == 0) reinterpret_cast<float*>(A.scr + A.scr_w_ofs)[job * 8 + (d >> 5)] = sq;
+  A.scr[job * 256 + d] = (uint8_t)state;
 }
 
 // word d of a row's MSB-first stream of KB-bit fields: the fields that overlap bits [32 d, 32 d + 32)
@@ -253,103 +280,113 @@ __device__ __forceinline__ uint32_t pack_word(const uint8_t* fld, int d) {
   return w;
 }
 
-// grid rows, block 256: keeps the best multiplier (or runs the flat row quantizer), rebuilds the row, packs the fields
-__global__ void __launch_bounds__(256) tb_select_kernel(TbEncArgs A) {
-  __shared__ float red[8];
-  __shared__ float buf[256];
-  __shared__ uint8_t fld[256];
-  const int d = threadIdx.x, nm = A.nm, rj = blockIdx.x;
-  const uint8_t* b = A.blob;
-  const Row R = tb_row(A, rj, d, buf);
-  const Group P = tb_group(b, R.g);
-  float x = R.y;
-  int field = 0, kb = 4; float psc = 1.f; unsigned pc = 0u; bool pack = false;
-  if (P.ok && R.pos >= P.guard) {
-    const Pre Q = tb_pre(red, b, P, R.y);
-    float xq = Q.r;
-    if (P.mode == 1) {
-      const float am = block_max(red, fabsf(Q.r));
-      float s7 = __fdiv_rn(am, 7.f); if (s7 == 0.f) s7 = 1.f;
-      float q = rintf(__fdiv_rn(Q.r, s7)); q = fminf(fmaxf(q, -7.f), 7.f); xq = __fmul_rn(q, s7);
-      field = (int)q + 8; psc = s7; kb = 4; pack = true;
-    } else if (P.mode == 0) {
-      const float* const W = reinterpret_cast<const float*>(A.scr + A.scr_w_ofs) + (size_t)rj * nm * 8;
-      float best_e = 0.f; int best = 0; bool have = false;
-      for (int mi = 0; mi < nm; ++mi) {
-        float e = 0.f;
+// what a row is stored as: one field per element, the field width, the row scale
+struct Coded { int field, bits; float scale, value; bool any; };
+// flat groups: symmetric int4 with scale max|r| / 7 (src/kvq_fast.cuh:194-198)
+__device__ __forceinline__ Coded code_flat(float* part8, float r) {
+  const float top = block_fold<MaxOp>(part8, fabsf(r), 0.f);
+  float step = __fdiv_rn(top, 7.f);
+  if (step == 0.f) step = 1.f;
+  const float q = fminf(fmaxf(rintf(__fdiv_rn(r, step)), -7.f), 7.f);
+  return Coded{(int)q + 8, 4, step, __fmul_rn(q, step), true};
+}
+// trellis groups: the multiplier whose search left the smallest squared error (its 8 partial sums added in order from 0;
+// the first of equal errors), the state the search chose for this element under it
+__device__ __forceinline__ Coded code_trellis(const TbEncArgs& A, const Profile& P, const GroupRec& G, const Residual& Q, int row) {
+  const float* err = reinterpret_cast<const float*>(A.scr + A.scr_w_ofs) + (size_t)row * A.nm * 8;
+  int keep = 0; float least = 0.f;
+  for (int i = 0; i < A.nm; ++i) {
+    float total = 0.f;
 #pragma unroll
-        for (int w = 0; w < 8; ++w) e = __fadd_rn(e, W[mi * 8 + w]);
-        if (!have || e < best_e) { have = true; best_e = e; best = mi; }
-      }
-      float s = tb_f16r(__fmul_rn(Q.rms, tb_f32(b + P.off_m + 4u * (unsigned)best))); if (s == 0.f) s = 1.f;
-      const unsigned to = tb_u32(b + P.off_t + 4u * (unsigned)P.tix);
-      const int st = A.scr[((size_t)rj * nm + best) * 256 + d];
-      xq = __fmul_rn(tb_cdec((int)(short)tb_u16(b + to + 12 + 2 * st), tb_f32(b + to + 4)), s);
-      field = st & ((1 << P.kk) - 1); psc = s; kb = P.kk; pack = true;
-    }
-    x = xq;
-    if (P.m > 0) x = __fadd_rn(x, __fmul_rn(Q.cj0, Q.uj0));
-    if (P.m > 1) x = __fadd_rn(x, __fmul_rn(Q.cj1, Q.uj1));
-    if (P.has_mu) x = __fadd_rn(x, Q.mud);
-    pc = (unsigned)__half_as_ushort(__float2half_rn(Q.cj0)) | ((unsigned)__half_as_ushort(__float2half_rn(Q.cj1)) << 16);
+    for (int k = 0; k < 8; ++k) total = __fadd_rn(total, err[i * 8 + k]);
+    if (i == 0 || total < least) { least = total; keep = i; }
   }
-  const bool in_range = A.yin || (R.ok && R.pos >= 0 && R.pos < A.max_ctx && (A.pos_limit == 0 || R.pos < A.pos_limit));
-  uint8_t* const payb0 = R.kind ? A.pay1 : A.pay0;
-  uint8_t* const payb = payb0 ? payb0 + R.slot_off : nullptr;
-  if (payb && in_range) {
-    uint32_t* const wrow = reinterpret_cast<uint32_t*>(payb + R.out * (size_t)A.stride);
-    fld[d] = (uint8_t)field;
-    __syncthreads();
-    const int nw = A.stride >> 2;
-    if (d < nw) {
-      uint32_t w = 0u;
-      if (pack && d < 8 * kb) w = kb == 5 ? pack_word<5>(fld, d) : kb == 4 ? pack_word<4>(fld, d) : pack_word<3>(fld, d);
-      wrow[d] = w;
-    }
-    if (d == 0) {
-      float* const scl = R.kind ? A.scl1 : A.scl0;
-      if (scl) reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(scl) + R.slot_off)[R.out] = psc;
-      if (A.side) { A.side[2 * R.out] = __float_as_uint(psc); A.side[2 * R.out + 1] = pc; }
-      if (A.coded) A.coded[R.out] = pack ? 1 : 0;
-    }
-  }
-  if (A.yout) A.yout[R.out * 256 + d] = x;
+  const float s = trial_scale(P, Q.rms, keep);
+  const TableRec T = read_table(P, G);
+  const int state = A.scr[((size_t)row * A.nm + keep) * 256 + threadIdx.x];
+  return Coded{state & ((1 << G.bits) - 1), G.bits, s, __fmul_rn(table_value(table_int(P, T, state), T.gain), s), true};
 }
 
-// decoder (tba_unpack_kernel, src/kvq_attn.cuh:46-75): grid rows, block 256
-__device__ __forceinline__ unsigned stream_bits(const uint32_t* wp, int nwords, int pos, int n) {
-  const int wi = pos >> 5, o = pos & 31;
-  const unsigned long long Z = ((unsigned long long)wp[wi] << 32) | (unsigned long long)((wi + 1 < nwords) ? wp[wi + 1] : 0u);
-  return (unsigned)((Z >> (64 - o - n)) & ((1ull << n) - 1ull));
+// grid rows, block 256: codes the row (best multiplier of the search, or the flat quantizer), rebuilds what it decodes to,
+// packs the fields, stores payload / scale / projection coefficients
+__global__ void __launch_bounds__(256) tb_select_kernel(TbEncArgs A) {
+  __shared__ float part8[8];
+  __shared__ float rot_buf[256];
+  __shared__ uint8_t fld[256];
+  const int d = threadIdx.x, row = blockIdx.x;
+  const Profile P{A.blob};
+  const RowRef R = locate_row(A, row, rot_buf);
+  const GroupRec G = read_group(P, R.group);
+  Coded C{0, 4, 1.f, R.x, false};
+  float rebuilt = R.x;                                   // rows that stay uncoded come back as they are
+  unsigned coef_bits = 0u;
+  if (G.present && R.pos >= G.guard) {
+    const Residual Q = residual_of(part8, P, G, R.x);
+    if (G.mode == 1) C = code_flat(part8, Q.r);
+    else if (G.mode == 0) C = code_trellis(A, P, G, Q, row);
+    else C.value = Q.r;
+    rebuilt = C.value;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) if (k < G.ndir) rebuilt = __fadd_rn(rebuilt, __fmul_rn(Q.coef[k], Q.dir[k]));
+    if (G.has_mean) rebuilt = __fadd_rn(rebuilt, Q.mean);
+    coef_bits = (unsigned)__half_as_ushort(__float2half_rn(Q.coef[0])) | ((unsigned)__half_as_ushort(__float2half_rn(Q.coef[1])) << 16);
+  }
+  const bool storable = A.yin || (R.valid && R.pos >= 0 && R.pos < A.max_ctx && (A.pos_limit == 0 || R.pos < A.pos_limit));
+  uint8_t* const plane = R.is_v ? A.pay1 : A.pay0;
+  if (plane && storable) {
+    uint32_t* const words = reinterpret_cast<uint32_t*>(plane + R.container + R.index * (size_t)A.stride);
+    fld[d] = (uint8_t)C.field;
+    __syncthreads();
+    if (d < (A.stride >> 2)) {
+      uint32_t w = 0u;
+      if (C.any && d < 8 * C.bits) w = C.bits == 5 ? pack_word<5>(fld, d) : C.bits == 4 ? pack_word<4>(fld, d) : pack_word<3>(fld, d);
+      words[d] = w;
+    }
+    if (d == 0) {
+      float* const scales = R.is_v ? A.scl1 : A.scl0;
+      if (scales) reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(scales) + R.container)[R.index] = C.scale;
+      if (A.side) { A.side[2 * R.index] = __float_as_uint(C.scale); A.side[2 * R.index + 1] = coef_bits; }
+      if (A.coded) A.coded[R.index] = C.any ? 1 : 0;
+    }
+  }
+  if (A.yout) A.yout[R.index * 256 + d] = rebuilt;
 }
+
+// n <= 13 bits that start at bit `first` of an MSB-first stream of words (bits past the last word read as zero)
+__device__ __forceinline__ unsigned stream_field(const uint32_t* words, int nwords, int first, int n) {
+  const int w = first >> 5, used = first & 31;
+  const uint32_t hi = words[w], lo = w + 1 < nwords ? words[w + 1] : 0u;
+  const uint32_t window = used ? (hi << used) | (lo >> (32 - used)) : hi;   // the 32 bits that start at `first`
+  return window >> (32 - n);
+}
+// decoder (src/kvq_attn.cuh:46-75): grid rows, block 256.  The state of element d is the last 8 bits of the stream up to
+// the end of its field, cut at the start of its chunk of 64 elements.
 __global__ void __launch_bounds__(256) tb_unpack_kernel(const uint8_t* blob, const int* grp, const int* pos, const uint8_t* pay, const uint32_t* side,
                                                         int stride, const float* yin, float* y) {
-  __shared__ float tab[256];
+  __shared__ float values[256];
   const int row = blockIdx.x, d = threadIdx.x;
-  const int g = grp[row];
+  const Profile P{blob};
+  const GroupRec G = read_group(P, grp[row]);
   float out = yin ? yin[(size_t)row * 256 + d] : 0.f;
-  if ((unsigned)g < tb_u32(blob + 28)) {
-    const Group P = tb_group(blob, g);
-    if (pos[row] >= P.guard && P.mode <= 1) {
-      const uint32_t* wp = reinterpret_cast<const uint32_t*>(pay + (size_t)row * stride);
-      const float s = __uint_as_float(side[2 * (size_t)row]); const unsigned pc = side[2 * (size_t)row + 1];
-      const int kb = P.mode == 1 ? 4 : P.kk, nw = 8 * kb;
-      float xq;
-      if (P.mode == 1) xq = __fmul_rn((float)((int)stream_bits(wp, nw, 4 * d, 4) - 8), s);
-      else {
-        const unsigned to = tb_u32(blob + P.off_t + 4u * (unsigned)P.tix);
-        tab[d] = tb_cdec((int)(short)tb_u16(blob + to + 12 + 2 * d), tb_f32(blob + to + 4));
-        __syncthreads();
-        const int endb = kb * (d + 1), first = kb * (d & ~63), lo = max(endb - 8, first);
-        xq = __fmul_rn(tab[stream_bits(wp, nw, lo, endb - lo)], s);
-      }
-      float x = xq;
-      const uint8_t* mup = blob + P.go + 8; const uint8_t* Up = mup + (P.has_mu ? 512 : 0);
-      if (P.m > 0) x = __fadd_rn(x, __fmul_rn(tb_h2f(pc & 0xffffu), tb_h2f(tb_u16(Up + 2 * d))));
-      if (P.m > 1) x = __fadd_rn(x, __fmul_rn(tb_h2f(pc >> 16), tb_h2f(tb_u16(Up + 2 * (256 + d)))));
-      if (P.has_mu) x = __fadd_rn(x, tb_h2f(tb_u16(mup + 2 * d)));
-      out = x;
+  if (G.present && pos[row] >= G.guard && G.mode <= 1) {                    // uniform over the block
+    const uint32_t* words = reinterpret_cast<const uint32_t*>(pay + (size_t)row * stride);
+    const float s = __uint_as_float(side[2 * (size_t)row]);
+    const unsigned coef_bits = side[2 * (size_t)row + 1];
+    float v;
+    if (G.mode == 1) {
+      v = __fmul_rn((float)((int)stream_field(words, 32, 4 * d, 4) - 8), s);
+    } else {
+      const TableRec T = read_table(P, G);
+      values[d] = table_value(table_int(P, T, d), T.gain);
+      __syncthreads();
+      const int end = G.bits * (d + 1), chunk_start = G.bits * (d & ~63), begin = max(end - 8, chunk_start);
+      v = __fmul_rn(values[stream_field(words, 8 * G.bits, begin, end - begin)], s);
     }
+    const float coef[2] = {__half2float(__ushort_as_half((unsigned short)(coef_bits & 0xffffu))), __half2float(__ushort_as_half((unsigned short)(coef_bits >> 16)))};
+#pragma unroll
+    for (int k = 0; k < 2; ++k) if (k < G.ndir) v = __fadd_rn(v, __fmul_rn(coef[k], P.f16_at(G.dir_off + 512u * (unsigned)k + 2u * (unsigned)d)));
+    if (G.has_mean) v = __fadd_rn(v, P.f16_at(G.mean_off + 2u * (unsigned)d));
+    out = v;
   }
   y[(size_t)row * 256 + d] = out;
 }
