@@ -11,9 +11,11 @@
 
 /* src/kvx_codec.cuh:28-32: sign of channel d from an integer hash of d+1 */
 float yko_kvx_sign(int d) {
-  uint32_t x = (uint32_t)d + 1u;
-  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
-  return (x & 1u) ? -1.f : 1.f;
+  uint32_t h = (uint32_t)d + 1u;
+  h = (h ^ (h >> 16)) * 0x7feb352du;
+  h = (h ^ (h >> 15)) * 0x846ca68bu;
+  h ^= h >> 16;
+  return (h & 1u) != 0u ? -1.f : 1.f;
 }
 
 /* src/kvx_codec.cuh:35-49: forward = signs, then 8 butterfly stages (h = 1..128; the element whose index has bit h set

@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <stdexcept>
 #include <string>
@@ -515,27 +516,43 @@ int yka_kvx256_probe(const float* x, int rows, int mode, int rot, int8_t* q8, ui
 namespace {
 struct TbInfo { int nm = 0, ngrp = 0, layers = 0, kv_heads = 0; bool has_trellis = false; };
 // the checks of the reference's loaders (src/engine35.cpp:48-52, src/kvq_fast.hpp:52-76) plus bounds on every record
+// Little-endian view of a profile blob: a 100-byte header, then three offset arrays (multipliers, tables, groups).
+struct BlobView {
+  const uint8_t* p; size_t n;
+  unsigned half(size_t at) const { return (unsigned)p[at] + 256u * (unsigned)p[at + 1]; }
+  uint32_t word(size_t at) const { return (uint32_t)half(at) + 65536u * (uint32_t)half(at + 2); }
+  int table_int(size_t rec, int state) const { return (int)(int16_t)half(rec + 12 + 2 * (size_t)state); }
+  size_t multipliers() const { return word(32); }
+  size_t table_record(unsigned t) const { return word((size_t)word(36) + 4 * (size_t)t); }
+  size_t group_record(int g) const { return word((size_t)word(40) + 4 * (size_t)g); }
+};
 TbInfo tb_check_blob(const uint8_t* b, size_t n) {
-  auto u16 = [&](size_t o) { return (unsigned)b[o] | ((unsigned)b[o + 1] << 8); };
-  auto u32 = [&](size_t o) { return u16(o) | (u16(o + 2) << 16); };
-  if (!b || n < 100 || std::memcmp(b, "KVQP", 4) != 0 || u16(4) != 1 || u32(8) != n) throw std::runtime_error("not a KVQP v1 profile blob");
-  if (u16(16) != 256) throw std::runtime_error("profile blob: rows must have 256 elements");
-  TbInfo I; I.layers = (int)u16(18); I.kv_heads = (int)u16(20); I.nm = (int)u16(24); I.ngrp = (int)u32(28);
-  const unsigned nt = u16(22);
-  const size_t off_m = u32(32), off_t = u32(36), off_g = u32(40);
-  if (I.nm < 1 || I.nm > 16) throw std::runtime_error("profile blob: bad scale-multiplier count");
-  if (off_m + 4 * (size_t)I.nm > n || off_t + 4 * (size_t)nt > n || off_g + 4 * (size_t)I.ngrp > n) throw std::runtime_error("profile blob: offsets outside the blob");
-  for (unsigned t = 0; t < nt; ++t) {
-    const size_t to = u32(off_t + 4 * t);
-    if (to + 12 + 512 > n || b[to] != 8 || b[to + 2] != 64 || b[to + 3] != 8) throw std::runtime_error("profile blob: tables must have 8 state bits, chunks of 64");
-    for (int s = 0; s < 256; ++s) { const int c = (int)(short)u16(to + 12 + 2 * (size_t)s); if (c > 1100 || c < -1100) throw std::runtime_error("profile blob: table value out of range"); }
+  auto bad = [](const char* what) { throw std::runtime_error(what); };
+  if (!b || n < 100 || std::memcmp(b, "KVQP", 4) != 0) bad("not a KVQP v1 profile blob");
+  const BlobView V{b, n};
+  if (V.half(4) != 1 || V.word(8) != n) bad("not a KVQP v1 profile blob");
+  if (V.half(16) != 256) bad("profile blob: rows must have 256 elements");
+  TbInfo I;
+  I.layers = (int)V.half(18); I.kv_heads = (int)V.half(20); I.nm = (int)V.half(24); I.ngrp = (int)V.word(28);
+  const unsigned n_tab = V.half(22);
+  if (I.nm < 1 || I.nm > 16) bad("profile blob: bad scale-multiplier count");
+  if (V.multipliers() + 4 * (size_t)I.nm > n || (size_t)V.word(36) + 4 * (size_t)n_tab > n || (size_t)V.word(40) + 4 * (size_t)I.ngrp > n)
+    bad("profile blob: offsets outside the blob");
+  for (unsigned t = 0; t < n_tab; ++t) {
+    const size_t rec = V.table_record(t);
+    if (rec + 12 + 512 > n || b[rec] != 8 || b[rec + 2] != 64 || b[rec + 3] != 8) bad("profile blob: tables must have 8 state bits, chunks of 64");
+    for (int st = 0; st < 256; ++st)
+      if (std::abs(V.table_int(rec, st)) > 1100) bad("profile blob: table value out of range");
   }
   for (int g = 0; g < I.ngrp; ++g) {
-    const size_t go = u32(off_g + 4 * (size_t)g);
-    if (go + 8 > n) throw std::runtime_error("profile blob: group record outside the blob");
-    const int mode = b[go], kk = b[go + 1], tix = b[go + 2], m = b[go + 4], has_mu = b[go + 5];
-    if (mode > 1 || m > 2 || go + 8 + (has_mu ? 512 : 0) + 512 * (size_t)m > n) throw std::runtime_error("profile blob: bad group record");
-    if (mode == 0) { if (kk < 3 || kk > 5 || (unsigned)tix >= nt) throw std::runtime_error("profile blob: trellis groups need 3..5 bits and a table"); I.has_trellis = true; }
+    const size_t rec = V.group_record(g);
+    if (rec + 8 > n) bad("profile blob: group record outside the blob");
+    const unsigned mode = b[rec], bits = b[rec + 1], table = b[rec + 2], ndir = b[rec + 4];
+    const size_t tail = (b[rec + 5] ? 512u : 0u) + 512u * (size_t)ndir;
+    if (mode > 1 || ndir > 2 || rec + 8 + tail > n) bad("profile blob: bad group record");
+    if (mode != 0) continue;
+    if (bits < 3 || bits > 5 || table >= n_tab) bad("profile blob: trellis groups need 3..5 bits and a table");
+    I.has_trellis = true;
   }
   return I;
 }
@@ -596,33 +613,32 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
   const int n_kv = kv->cfg.n_kv_heads;
   if (I.kv_heads != n_kv || I.ngrp < n_kv * 2) throw std::runtime_error("the profile does not cover the kv heads of the handle");
   const int need = (I.ngrp / (n_kv * 2)) * n_kv * 2;
-  auto u16 = [&](size_t o) { return (unsigned)blob[o] | ((unsigned)blob[o + 1] << 8); };
-  auto u32 = [&](size_t o) { return u16(o) | (u16(o + 2) << 16); };
-  const size_t off_t = u32(36), off_g = u32(40);
+  const BlobView V{blob, blob_len};
   // what the reference asks of a layer before it keeps packed rows for it (kvqaxpk_packable, src/kvq_atxpk.hpp:61-72)
   int kb = 0; bool has_mu = false;
   std::vector<uint16_t> tabs((size_t)need * 256); std::vector<float> gfac(need), mu((size_t)need * 256, 0.f);
   std::vector<uint32_t> pairs;
   for (int g = 0; g < need; ++g) {
-    const size_t go = u32(off_g + 4 * (size_t)g);
-    const int mode = blob[go], kk = blob[go + 1], tix = blob[go + 2], guard = blob[go + 3], m = blob[go + 4];
-    if (mode != 0 || (kk != 4 && kk != 5) || guard != 0 || m != 0)
+    const size_t rec = V.group_record(g);
+    const int bits = blob[rec + 1];
+    const bool plain_trellis = blob[rec] == 0 && blob[rec + 3] == 0 && blob[rec + 4] == 0;   // mode, guard, directions
+    if (!plain_trellis || (bits != 4 && bits != 5))
       throw std::runtime_error("packed rows need every group trellis-coded with 4 or 5 bits, no guard position and no projected directions");
-    if (kb && kk != kb) throw std::runtime_error("packed rows need the same bits per element in every group");
-    kb = kk;
-    const size_t to = u32(off_t + 4 * (size_t)tix);
-    float gain; std::memcpy(&gain, blob + to + 4, 4);
+    if (kb != 0 && bits != kb) throw std::runtime_error("packed rows need the same bits per element in every group");
+    kb = bits;
+    const size_t trec = V.table_record(blob[rec + 2]);
+    float gain; std::memcpy(&gain, blob + trec + 4, 4);
     if (!(gain > 0.f) || gain > 1e6f) throw std::runtime_error("profile blob: table gain must be positive and finite");
     gfac[g] = 0.00390625f * gain;
-    for (int st = 0; st < 256; ++st) tabs[(size_t)g * 256 + st] = int_to_f16_bits((int)(short)u16(to + 12 + 2 * (size_t)st));
-    if (blob[go + 5]) {
-      has_mu = true;
-      for (int d = 0; d < 256; ++d) {
-        const unsigned h = u16(go + 8 + 2 * (size_t)d), sg = h >> 15, e = (h >> 10) & 31u, mm = h & 1023u;
-        float v = e == 0 ? std::ldexp((float)mm, -24) : std::ldexp((float)(mm | 1024u), (int)e - 25);
-        if (e == 31) throw std::runtime_error("profile blob: mean row is not finite");
-        mu[(size_t)g * 256 + d] = sg ? -v : v;
-      }
+    uint16_t* row = &tabs[(size_t)g * 256];
+    for (int st = 0; st < 256; ++st) row[st] = int_to_f16_bits(V.table_int(trec, st));
+    if (blob[rec + 5] == 0) continue;
+    has_mu = true;
+    for (int d = 0; d < 256; ++d) {                    // fp16 mean row, widened by hand (host code, no half type needed)
+      const unsigned h = V.half(rec + 8 + 2 * (size_t)d), expo = (h >> 10) & 31u, frac = h & 1023u;
+      if (expo == 31) throw std::runtime_error("profile blob: mean row is not finite");
+      const float mag = expo == 0 ? std::ldexp((float)frac, -24) : std::ldexp((float)(frac + 1024u), (int)expo - 25);
+      mu[(size_t)g * 256 + d] = (h & 0x8000u) ? -mag : mag;
     }
   }
   // pair tables: entry i decodes two consecutive elements from the 8 + kb stream bits that end with the second one

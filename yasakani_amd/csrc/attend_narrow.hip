@@ -26,6 +26,7 @@
 //     before it loads the tile.  The split merge stays a second launch: the 8 XCDs keep separate L2s, so merging in
 //     the last workgroup needs a device-scope release (an L2 write-back) in every workgroup, measured 4x slower.
 #include "codec_device.h"
+#include "sign_device.h"
 
 namespace yka {
 
@@ -422,9 +423,7 @@ __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
     if (tid < kD) {
       const float b = s_w[tid ^ 64];
       y = (tid & 64) ? b - y : y + b;
-      uint32_t x = (uint32_t)tid + 1u;             // sign of channel tid (src/kvx_codec.cuh:28-32)
-      x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
-      y = y * 0.0625f * ((x & 1u) ? -1.f : 1.f);
+      y = y * 0.0625f * channel_sign(tid);         // signs last on the way back (src/kvx_codec.cuh:28-32)
     }
   }
   if (tid < kD) A.out16[((size_t)tok * A.n_heads + head) * kD + tid] = __half_as_ushort(__float2half_rn(y));

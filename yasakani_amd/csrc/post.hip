@@ -9,15 +9,11 @@
 //   rotation: signs (src/kvx_codec.cuh:28-32), 7 butterfly stages (src/kvx_codec.cuh:40-45), x 1/8 for K and V,
 //   x 1/16 for Q (and for the inverse applied to attention outputs): (1/8)(1/16) 128 = 1.
 #include "codec_device.h"
+#include "sign_device.h"
 
 namespace yka {
 namespace {
 
-__device__ __forceinline__ float sign128(int d) {
-  uint32_t x = (uint32_t)d + 1u;
-  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
-  return (x & 1u) ? -1.f : 1.f;
-}
 // Round an fp32 value to fp16 and back.  The empty asm keeps the value's producer (an fp32 multiply) from being merged
 // with the conversion into one mixed-precision instruction that rounds the exact product once: the arithmetic here is
 // defined as two roundings (fp32, then fp16), and the two differ when the fp32 product lands on an fp16 tie.
@@ -26,7 +22,7 @@ __device__ __forceinline__ float f16r(float x) { asm volatile("" : "+v"(x)); ret
 // forward rotation of one 128-channel row held one channel per thread (2 waves); buf: 128 floats of LDS
 __device__ __forceinline__ float rotate128_fwd(float x, float* buf, float factor) {
   const int d = threadIdx.x;
-  float a = __fmul_rn(x, sign128(d));
+  float a = __fmul_rn(x, channel_sign(d));
 #pragma unroll
   for (int h = 1; h < 64; h *= 2) {
     const float b = __shfl_xor(a, h, 64);

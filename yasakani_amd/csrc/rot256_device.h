@@ -4,20 +4,15 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include "sign_device.h"
 
 namespace yka {
-
-__device__ __forceinline__ float kvx_sign(int d) {
-  uint32_t x = (uint32_t)d + 1u;
-  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
-  return (x & 1u) ? -1.f : 1.f;
-}
 
 // The butterfly stages are element-wise, so where the partner lives does not change a bit of the result: partners at
 // distance 1..32 are in the same wave (cross-lane exchange), 64 and 128 go through LDS.
 __device__ __forceinline__ float rotate256(float x, float* buf, bool inverse) {
   const int d = threadIdx.x;
-  float a = inverse ? x : __fmul_rn(x, kvx_sign(d));
+  float a = inverse ? x : __fmul_rn(x, channel_sign(d));
 #pragma unroll
   for (int h = 1; h < 64; h *= 2) {
     const float b = __shfl_xor(a, h, 64);
@@ -32,7 +27,7 @@ __device__ __forceinline__ float rotate256(float x, float* buf, bool inverse) {
     a = (d & h) ? __fsub_rn(b, a) : __fadd_rn(a, b);
   }
   float y = __fmul_rn(a, 0.0625f);
-  if (inverse) y = __fmul_rn(y, kvx_sign(d));
+  if (inverse) y = __fmul_rn(y, channel_sign(d));
   return y;
 }
 
