@@ -162,72 +162,199 @@ __device__ __forceinline__ int group_min(int v) {       // min over the lanes co
   return pair_min<32>(v);
 }
 
-// One chunk in one wave.  xi: the chunk's 64 integer targets (LDS), ci4: table values of the lane's four states,
-// bp: 64 x 32 bytes of LDS private to the wave, st_out: 64 bytes of LDS private to the wave.
-template <int KK>
-__device__ __forceinline__ void wave_chunk(const int* xi, const int (&ci4)[4], uint8_t* bp, uint8_t* st_out) {
-  constexpr int U = 256 >> KK, PER = 64 / U;          // PER = predecessor indices j a lane step covers: j = l / U + PER * k
-  const int lane = threadIdx.x & 63;
-  const int xreg = xi[lane];                           // target t lives in lane t
-  // Costs are kept relative to a common offset (only differences decide) and, for 4- and 5-bit fields, carried as
-  // cost * 2^KK + j with j the state's index among the predecessors of its group: ONE minimum then yields the smallest
-  // cost and, among equal costs, the smallest predecessor.  At any step two states differ by at most two (three at 3
-  // bits) steps' worth of squared error, < 2 * 3148^2, so the packed value fits 32 bits once the offset - the minimum of
-  // group 0 - is subtracted at every step.  States that cannot be reached yet start 40,000,000 above state 0: more than
-  // any path costs before every state is reachable, like the reference's 2^30, and small enough to be packed.
-  constexpr bool kPacked = KK >= 4;
-  constexpr int kFar = kPacked ? 40000000 : 0x40000000;
-  int cost[4];
-#pragma unroll
-  for (int k = 0; k < 4; ++k) cost[k] = (lane == 0 && k == 0) ? 0 : kFar;
-#pragma unroll 1
-  for (int t = 0; t < 64; ++t) {
-    int mn, jb;
-    if constexpr (kPacked) {
-      int key[4];
-#pragma unroll
-      for (int k = 0; k < 4; ++k) key[k] = (cost[k] << KK) | (lane / U + PER * k);
-      const int km = group_min<U>(min(min(key[0], key[1]), min(key[2], key[3])));
-      jb = km & ((1 << KK) - 1);
-      mn = km >> KK;
-      mn -= __builtin_amdgcn_readlane(mn, 0);           // the common offset: group 0's minimum
-    } else {
-      mn = group_min<U>(min(min(cost[0], cost[1]), min(cost[2], cost[3])));
-      jb = 255;
-#pragma unroll
-      for (int k = 3; k >= 0; --k) jb = cost[k] == mn ? lane / U + PER * k : jb;
-      jb = group_min<U>(jb);
-    }
-    if (lane < U) bp[t * 32 + lane] = (uint8_t)jb;
-    const int x = __builtin_amdgcn_readlane(xreg, t);
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-      // the group this state continues is u = (lane + 64 k) >> KK; lane u holds its minimum (reading the minima into
-      // scalar registers and selecting per lane was measured slower than this gather)
-      const int m = __shfl(mn, (lane + 64 * k) >> KK, 64);
-      const int dx = x - ci4[k];
-      cost[k] = dx * dx + m;
+// min(v, v of the lane a DPP control names) as ONE instruction.  The compiler's own form is copy + move-with-control +
+// min; the two idle cycles a lane-crossing read needs after its source was written are part of the statement.
+#define YKA_DPP_MIN(NAME, CTRL)                                                                                  \
+  __device__ __forceinline__ int NAME(int v) {                                                                   \
+    int r;                                                                                                       \
+    asm("s_nop 1\n\tv_min_i32_dpp %0, %1, %1 " CTRL " row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(v));          \
+    return r;                                                                                                    \
+  }
+YKA_DPP_MIN(min_xor1, "quad_perm:[1,0,3,2]")            // with the neighbour in the pair
+YKA_DPP_MIN(min_xor2, "quad_perm:[2,3,0,1]")            // with the other pair of the quad
+YKA_DPP_MIN(min_oct, "row_half_mirror")                 // with the mirrored lane of 8: the other quad
+YKA_DPP_MIN(min_ror4, "row_ror:4")                      // with the lane four further in the row of 16
+YKA_DPP_MIN(min_ror8, "row_ror:8")
+#undef YKA_DPP_MIN
+// v + (w of the lane the control names), one instruction
+#define YKA_DPP_ADD(NAME, CTRL)                                                                                  \
+  __device__ __forceinline__ int NAME(int w, int v) {                                                            \
+    int r;                                                                                                       \
+    asm("s_nop 1\n\tv_add_u32_dpp %0, %1, %2 " CTRL " row_mask:0xf bank_mask:0xf" : "=v"(r) : "v"(w), "v"(v));  \
+    return r;                                                                                                    \
+  }
+YKA_DPP_ADD(add_rot1, "quad_perm:[1,2,3,0]")            // w of the next lane of the quad (cyclic)
+YKA_DPP_ADD(add_rot2, "quad_perm:[2,3,0,1]")
+YKA_DPP_ADD(add_rot3, "quad_perm:[3,0,1,2]")
+YKA_DPP_ADD(add_pos0, "quad_perm:[0,0,0,0]")            // w of lane 0 / 1 / 2 / 3 of the quad
+YKA_DPP_ADD(add_pos1, "quad_perm:[1,1,1,1]")
+YKA_DPP_ADD(add_pos2, "quad_perm:[2,2,2,2]")
+YKA_DPP_ADD(add_pos3, "quad_perm:[3,3,3,3]")
+#undef YKA_DPP_ADD
+
+// Where the 256 states sit in a wave: 64 lanes x 4 slots, in one of two arrangements between which the costs alternate
+// from step to step.  A state s is a member of group s & (U - 1) (U = 256 >> KK groups of 2^KK members: the states that
+// can precede the same successors) and continues group s >> KK.  Write a lane as (r, q, i) = 16 r + 4 q + i.
+//   5 bits, arrangement 0: lane = 8 (s >> 5) + (s & 7), slot = bits 3-4 of s.  A group's members are the lanes congruent
+//     modulo 8; after the reduction (row rotation, row swap, half swap) all of them hold its minimum.  Arrangement 1:
+//     lane = 8 (s & 7) + (s >> 5): exactly those lanes hold the states that continue that group, and a group's members
+//     are now 8 adjacent lanes (three quad / half-mirror steps), which are the lanes of its successors in arrangement 0.
+//   4 bits, arrangement 0: s = 16 (4 r + slot) + (lane & 15).  Members: lanes congruent modulo 16 (row swap, half swap); the minimum of
+//     group 4 q + i then sits in lane (., q, i) of every row.  Arrangement 1: group (s & 15) = 4 r + i, continued group
+//     (s >> 4) = 4 q + ((i + slot) & 3): a lane finds the four minima it needs in its own quad, rotated by the slot,
+//     and a group's members are the four lanes (r, ., i) of a row (two row rotations).  Back in arrangement 0 the states
+//     of lane (r, q, i), slot n continue group 4 r + n, whose minimum is in position n of the lane's own quad.
+// No minimum is ever fetched through LDS.
+template <int KK, int ARR>
+__device__ __forceinline__ int state_at(int lane, int n) {
+  const int r = lane >> 4, q = (lane >> 2) & 3, i = lane & 3;
+  if constexpr (KK == 5) return ARR ? ((lane & 7) << 5) | (n << 3) | (lane >> 3) : ((lane >> 3) << 5) | (n << 3) | (lane & 7);
+  else if constexpr (KK == 4) return ARR ? ((4 * q + ((i + n) & 3)) << 4) | (4 * r + i) : ((4 * r + n) << 4) | (lane & 15);
+  else return (n << 6) | lane;
+}
+// the lane that holds the minimum of group g after the reduction in BOTH arrangements
+template <int KK> __device__ __forceinline__ int keeper_lane(int g) { return KK == 5 ? 9 * g : 20 * (g >> 2) + (g & 3); }
+
+// lane 0 walks the chosen path back from the best final state.  WORDS: word (t / 4) * 32 + u of bp holds, in byte t % 4,
+// the predecessor index chosen at step t for the states that continue group u; otherwise byte t * 32 + u does.
+template <int KK, bool WORDS>
+__device__ __forceinline__ void walk_back(int best_state, const uint8_t* bp, uint8_t* st_out) {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  if ((threadIdx.x & 63) == 0) {
+    int st = best_state;
+    for (int t = 63; t >= 0; --t) {
+      st_out[t] = (uint8_t)st;
+      const int u = st >> KK;
+      const int j = WORDS ? (int)((reinterpret_cast<const uint32_t*>(bp)[(t >> 2) * 32 + u] >> (8 * (t & 3))) & 255u) : (int)bp[t * 32 + u];
+      st = (j << (8 - KK)) | u;
     }
   }
-  // smallest cost, then smallest state
-  int bc = cost[0], bs = lane;
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+// smallest cost over the wave's 256 states, the smallest state among equal costs; sid[k] ascending in k
+__device__ __forceinline__ int best_final(const int (&cost)[4], const int (&sid)[4]) {
+  int bc = cost[0], bs = sid[0];
 #pragma unroll
-  for (int k = 1; k < 4; ++k) if (cost[k] < bc) { bc = cost[k]; bs = lane + 64 * k; }
+  for (int k = 1; k < 4; ++k) if (cost[k] < bc) { bc = cost[k]; bs = sid[k]; }
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
     const int oc = __shfl_xor(bc, o, 64), os = __shfl_xor(bs, o, 64);
     if (oc < bc || (oc == bc && os < bs)) { bc = oc; bs = os; }
   }
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  if (lane == 0) {
-    int st = bs;
-    for (int t = 63; t >= 0; --t) {
-      st_out[t] = (uint8_t)st;
-      const int j = bp[t * 32 + (st >> KK)];
-      st = (j << (8 - KK)) | (st >> KK);
+  return bs;
+}
+
+// One chunk in one wave, 4- or 5-bit fields.  xi: the chunk's 64 integer targets (LDS), tab(s): table value of state s,
+// bp: 64 x 32 bytes of LDS private to the wave, st_out: 64 bytes of LDS private to the wave.
+// A state's cost is carried as key = cost * 2^KK + j with j the state's index among the members of its group, relative to
+// a common offset (only differences decide): ONE minimum then yields the smallest cost and, among equal costs, the
+// smallest predecessor.  At any step two states differ by at most two steps' worth of squared error, < 2 * 3148^2, so the
+// key fits 32 bits once the offset - the minimum of group 0 - is subtracted at every step.  States that cannot be
+// reached yet start 40,000,000 above state 0: more than any path costs before every state is reachable, like the
+// reference's 2^30, and small enough for the key.
+// a + x * b for |x|, |b| < 2^23, one full-rate instruction (x wave-uniform)
+__device__ __forceinline__ int mad24(int x, int b, int a) {
+  int r;
+  asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(r) : "s"(x), "v"(b), "v"(a));
+  return r;
+}
+template <int KK, class Tab>
+__device__ __forceinline__ void wave_chunk(const int* xi, Tab tab, uint8_t* bp, uint8_t* st_out) {
+  static_assert(KK == 4 || KK == 5, "packed search: 4 or 5 bits");
+  constexpr int U = 256 >> KK, kFar = 40000000, kLow = (1 << KK) - 1;
+  const int lane = threadIdx.x & 63;
+  const int xreg = xi[lane];                           // target t lives in lane t
+  // (x - c)^2 = x^2 - 2 x c + c^2, and x^2 is common to all states of a step: a state's step cost in key units is
+  // a - x b with a = c^2 * 2^KK + j and b = 2 c * 2^KK, constants of the (lane, slot) in each arrangement
+  int a0[4], a1[4], b0[4], b1[4], sid[4], key[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    sid[k] = state_at<KK, 0>(lane, k);
+    const int s1 = state_at<KK, 1>(lane, k), c0 = tab(sid[k]), c1 = tab(s1);
+    a0[k] = ((c0 * c0) << KK) | (sid[k] >> (8 - KK)); b0[k] = (2 * c0) << KK;
+    a1[k] = ((c1 * c1) << KK) | (s1 >> (8 - KK));     b1[k] = (2 * c1) << KK;
+    key[k] = ((sid[k] == 0 ? 0 : kFar) << KK) | (sid[k] >> (8 - KK));
+  }
+  // is this lane the keeper of a group, and of which: its record of chosen predecessors goes to LDS every four steps
+  int kept = -1;
+#pragma unroll
+  for (int g = 0; g < U; ++g) kept = lane == keeper_lane<KK>(g) ? g : kept;
+  uint32_t* const rec = reinterpret_cast<uint32_t*>(bp) + (kept < 0 ? 0 : kept);
+#pragma unroll 1
+  for (int t = 0; t < 64; t += 4) {
+    uint32_t chosen4 = 0u;
+#pragma unroll
+    for (int h = 0; h < 4; h += 2) {
+      {                                                // arrangement 0 -> 1
+        int km = min(min(key[0], key[1]), min(key[2], key[3]));
+        if constexpr (KK == 5) km = min_ror8(km);
+        km = pair_min<32>(pair_min<16>(km));
+        chosen4 |= (uint32_t)(km & kLow) << (8 * h);
+        int m = km & ~kLow;                            // cost * 2^KK
+        m -= __builtin_amdgcn_readlane(m, 0);          // the common offset: group 0's minimum
+        const int nx = -__builtin_amdgcn_readlane(xreg, t + h);
+        if constexpr (KK == 5) {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) key[k] = mad24(nx, b1[k], a1[k]) + m;
+        } else {
+          key[0] = mad24(nx, b1[0], a1[0]) + m;
+          key[1] = add_rot1(m, mad24(nx, b1[1], a1[1]));
+          key[2] = add_rot2(m, mad24(nx, b1[2], a1[2]));
+          key[3] = add_rot3(m, mad24(nx, b1[3], a1[3]));
+        }
+      }
+      {                                                // arrangement 1 -> 0
+        int km = min(min(key[0], key[1]), min(key[2], key[3]));
+        if constexpr (KK == 5) km = min_oct(min_xor2(min_xor1(km)));
+        else km = min_ror8(min_ror4(km));
+        chosen4 |= (uint32_t)(km & kLow) << (8 * h + 8);
+        int m = km & ~kLow;
+        m -= __builtin_amdgcn_readlane(m, 0);
+        const int nx = -__builtin_amdgcn_readlane(xreg, t + h + 1);
+        if constexpr (KK == 5) {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) key[k] = mad24(nx, b0[k], a0[k]) + m;
+        } else {
+          key[0] = add_pos0(m, mad24(nx, b0[0], a0[0]));
+          key[1] = add_pos1(m, mad24(nx, b0[1], a0[1]));
+          key[2] = add_pos2(m, mad24(nx, b0[2], a0[2]));
+          key[3] = add_pos3(m, mad24(nx, b0[3], a0[3]));
+        }
+      }
+    }
+    if (kept >= 0) rec[(t >> 2) * 32] = chosen4;
+  }
+  int cost[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) cost[k] = key[k] >> KK;
+  walk_back<KK, true>(best_final(cost, sid), bp, st_out);
+}
+
+// One chunk in one wave, 3-bit fields (32 groups of 8): unpacked costs, the group minima gathered across lanes.
+__device__ __forceinline__ void wave_chunk3(const int* xi, const int (&ci4)[4], uint8_t* bp, uint8_t* st_out) {
+  constexpr int KK = 3, U = 32, PER = 2;               // PER = predecessor indices j a lane step covers: j = l / U + PER * k
+  const int lane = threadIdx.x & 63;
+  const int xreg = xi[lane];
+  int cost[4], sid[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) { sid[k] = lane + 64 * k; cost[k] = sid[k] == 0 ? 0 : 0x40000000; }
+#pragma unroll 1
+  for (int t = 0; t < 64; ++t) {
+    const int mn = group_min<U>(min(min(cost[0], cost[1]), min(cost[2], cost[3])));
+    int jb = 255;
+#pragma unroll
+    for (int k = 3; k >= 0; --k) jb = cost[k] == mn ? lane / U + PER * k : jb;
+    jb = group_min<U>(jb);
+    if (lane < U) bp[t * 32 + lane] = (uint8_t)jb;
+    const int x = __builtin_amdgcn_readlane(xreg, t);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int m = __shfl(mn, (lane + 64 * k) >> KK, 64);   // lane u holds the minimum of group u
+      const int dx = x - ci4[k];
+      cost[k] = dx * dx + m;
     }
   }
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  walk_back<KK, false>(best_final(cost, sid), bp, st_out);
 }
 
 // grid rows * nm, block 256: block = (row, multiplier); wave c = chunk c.  Writes the 256 states of the row under this
@@ -236,7 +363,7 @@ __global__ void __launch_bounds__(256) tb_search_kernel(TbEncArgs A) {
   __shared__ float part8[8];
   __shared__ float rot_buf[256];
   __shared__ int target[256];
-  __shared__ uint8_t back[4][64 * 32];
+  __shared__ __align__(16) uint8_t back[4][64 * 32];
   __shared__ uint8_t chosen[256];
   const int d = threadIdx.x, wave = d >> 6, lane = d & 63;
   const int row = blockIdx.x / A.nm, mult = blockIdx.x % A.nm;
@@ -249,13 +376,16 @@ __global__ void __launch_bounds__(256) tb_search_kernel(TbEncArgs A) {
   const float s = trial_scale(P, Q.rms, mult);
   // integer target of element d: the residual in units of s / 256, clamped
   target[d] = (int)fminf(fmaxf(rintf(__fmul_rn(__fdiv_rn(Q.r, s), 256.f)), -2048.f), 2048.f);
-  int ci4[4];
-#pragma unroll
-  for (int k = 0; k < 4; ++k) ci4[k] = table_int(P, T, lane + 64 * k);
   __syncthreads();
-  if (G.bits == 5) wave_chunk<5>(target + 64 * wave, ci4, back[wave], chosen + 64 * wave);
-  else if (G.bits == 4) wave_chunk<4>(target + 64 * wave, ci4, back[wave], chosen + 64 * wave);
-  else wave_chunk<3>(target + 64 * wave, ci4, back[wave], chosen + 64 * wave);
+  const auto tab = [&](int state) { return table_int(P, T, state); };
+  if (G.bits == 5) wave_chunk<5>(target + 64 * wave, tab, back[wave], chosen + 64 * wave);
+  else if (G.bits == 4) wave_chunk<4>(target + 64 * wave, tab, back[wave], chosen + 64 * wave);
+  else {
+    int ci4[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) ci4[k] = tab(lane + 64 * k);
+    wave_chunk3(target + 64 * wave, ci4, back[wave], chosen + 64 * wave);
+  }
   // squared error of this multiplier: element d of the row is lane `lane` of wave `wave`; summed per run of 32 elements
   const int state = chosen[d];
   const float miss = __fsub_rn(Q.r, __fmul_rn(table_value(table_int(P, T, state), T.gain), s));
