@@ -231,6 +231,40 @@ __device__ __forceinline__ void walk_back(int best_state, const uint8_t* bp, uin
   }
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
+// The same walk for 4- and 5-bit fields, in parallel.  The step t -> t - 1 depends on the state only through the group
+// u = state >> KK it continues (U = 256 >> KK values): state(t - 1) = (chosen[t][u] << (8 - KK)) | u.  The 64 steps are cut
+// into 64 / U blocks of U steps; lane (block, u0) walks its block assuming it is entered in group u0 and keeps the
+// states it passes.  A chain of 64 / U lane reads then finds, from the best final state downwards, the group in which
+// every block really is entered, and the lanes that assumed right write their states.  bp in the word layout above.
+template <int KK>
+__device__ __forceinline__ void walk_back_blocks(int best_state, const uint8_t* bp, uint8_t* st_out) {
+  constexpr int U = 256 >> KK, NB = 64 / U;            // steps per block, blocks
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  const int lane = threadIdx.x & 63, blk = lane / U, u0 = lane % U;
+  const uint32_t* const words = reinterpret_cast<const uint32_t*>(bp) + (U / 4) * 32 * blk;
+  int passed[U], u = u0;
+#pragma unroll
+  for (int i = 0; i < U; ++i) {                        // step t = U blk + U - 1 - i
+    const int j = (int)((words[((U - 1 - i) >> 2) * 32 + u] >> (8 * ((U - 1 - i) & 3))) & 255u);
+    passed[i] = (j << (8 - KK)) | u;                   // state(t - 1)
+    u = passed[i] >> KK;
+  }
+  int entered = best_state >> KK, mine = 0;            // group in which the top block is entered
+#pragma unroll
+  for (int b = NB - 1; b >= 0; --b) {
+    mine = blk == b ? entered : mine;
+    entered = __builtin_amdgcn_readlane(u, __builtin_amdgcn_readfirstlane(U * b + entered));
+  }
+  if (lane == 0) st_out[63] = (uint8_t)best_state;
+  if (u0 == mine) {
+#pragma unroll
+    for (int i = 0; i < U; ++i) {
+      const int t1 = U * blk + U - 2 - i;              // t - 1
+      if (t1 >= 0) st_out[t1] = (uint8_t)passed[i];
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 // smallest cost over the wave's 256 states, the smallest state among equal costs; sid[k] ascending in k
 __device__ __forceinline__ int best_final(const int (&cost)[4], const int (&sid)[4]) {
   int bc = cost[0], bs = sid[0];
@@ -248,10 +282,11 @@ __device__ __forceinline__ int best_final(const int (&cost)[4], const int (&sid)
 // bp: 64 x 32 bytes of LDS private to the wave, st_out: 64 bytes of LDS private to the wave.
 // A state's cost is carried as key = cost * 2^KK + j with j the state's index among the members of its group, relative to
 // a common offset (only differences decide): ONE minimum then yields the smallest cost and, among equal costs, the
-// smallest predecessor.  At any step two states differ by at most two steps' worth of squared error, < 2 * 3148^2, so the
-// key fits 32 bits once the offset - the minimum of group 0 - is subtracted at every step.  States that cannot be
-// reached yet start 40,000,000 above state 0: more than any path costs before every state is reachable, like the
-// reference's 2^30, and small enough for the key.
+// smallest predecessor.  At any step two states differ by at most two steps' worth of squared error, < 2 * 3148^2 (634 M
+// in key units at 5 bits), and a step moves every key by -144 M ... +182 M, so the key fits 32 bits when the offset - the
+// minimum of group 0 - is subtracted every fourth step.  States that cannot be reached yet start 40,000,000 above state
+// 0: more than any path costs before every state is reachable (after two steps), like the reference's 2^30, and small
+// enough for the key.
 // a + x * b for |x|, |b| < 2^23, one full-rate instruction (x wave-uniform)
 __device__ __forceinline__ int mad24(int x, int b, int a) {
   int r;
@@ -289,9 +324,9 @@ __device__ __forceinline__ void wave_chunk(const int* xi, Tab tab, uint8_t* bp, 
         int km = min(min(key[0], key[1]), min(key[2], key[3]));
         if constexpr (KK == 5) km = min_ror8(km);
         km = pair_min<32>(pair_min<16>(km));
-        chosen4 |= (uint32_t)(km & kLow) << (8 * h);
+        chosen4 = __builtin_amdgcn_alignbit((uint32_t)km, chosen4, 8);   // low byte of km enters at the top
         int m = km & ~kLow;                            // cost * 2^KK
-        m -= __builtin_amdgcn_readlane(m, 0);          // the common offset: group 0's minimum
+        if (h == 0) m -= __builtin_amdgcn_readlane(m, 0);   // the common offset: group 0's minimum, once per four steps
         const int nx = -__builtin_amdgcn_readlane(xreg, t + h);
         if constexpr (KK == 5) {
 #pragma unroll
@@ -307,9 +342,8 @@ __device__ __forceinline__ void wave_chunk(const int* xi, Tab tab, uint8_t* bp, 
         int km = min(min(key[0], key[1]), min(key[2], key[3]));
         if constexpr (KK == 5) km = min_oct(min_xor2(min_xor1(km)));
         else km = min_ror8(min_ror4(km));
-        chosen4 |= (uint32_t)(km & kLow) << (8 * h + 8);
-        int m = km & ~kLow;
-        m -= __builtin_amdgcn_readlane(m, 0);
+        chosen4 = __builtin_amdgcn_alignbit((uint32_t)km, chosen4, 8);
+        const int m = km & ~kLow;
         const int nx = -__builtin_amdgcn_readlane(xreg, t + h + 1);
         if constexpr (KK == 5) {
 #pragma unroll
@@ -322,12 +356,12 @@ __device__ __forceinline__ void wave_chunk(const int* xi, Tab tab, uint8_t* bp, 
         }
       }
     }
-    if (kept >= 0) rec[(t >> 2) * 32] = chosen4;
+    if (kept >= 0) rec[(t >> 2) * 32] = chosen4 & (0x01010101u * (uint32_t)kLow);
   }
   int cost[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) cost[k] = key[k] >> KK;
-  walk_back<KK, true>(best_final(cost, sid), bp, st_out);
+  walk_back_blocks<KK>(best_final(cost, sid), bp, st_out);
 }
 
 // One chunk in one wave, 3-bit fields (32 groups of 8): unpacked costs, the group minima gathered across lanes.
