@@ -37,7 +37,7 @@ struct yka_kv {
   // [K payload n_kv * max_ctx * stride][V payload][K scales n_kv * max_ctx fp32][V scales]
   struct Tb {
     int kb = 0, stride = 0, nm = 0, layers = 0; bool has_mu = false;   // layers: layers the profile has groups for
-    uint8_t* blob = nullptr; uint32_t* pairs = nullptr; float* gfac = nullptr; float* mu = nullptr;
+    uint8_t* blob = nullptr; uint32_t* desc = nullptr; int ngrp = 0; unsigned mult_off = 0; uint32_t* pairs = nullptr; float* gfac = nullptr; float* mu = nullptr;
     uint8_t* pool = nullptr; size_t layer_bytes = 0, pay_bytes = 0, scl_bytes = 0;
     uint8_t* scr = nullptr; size_t scr_w_ofs = 0;
     float* stage = nullptr;          // fp32 K rows then V rows of one pass ([max_rows][n_kv][256] each): yka_attn_post -> encoder
@@ -122,7 +122,7 @@ void tb_append(yka_kv* kv, int layer, const float* k32, const float* v32, const 
   check_tb_layer(kv, layer);
   for (int t0 = 0; t0 < M; t0 += kTbTileTok) {
     TbEncArgs A{};
-    A.blob = T.blob; A.nm = T.nm; A.has_trellis = 1;
+    A.blob = T.blob; A.nm = T.nm; A.has_trellis = 1; A.desc = T.desc; A.ngrp = T.ngrp; A.mult_off = T.mult_off;
     A.k32 = k32; A.v32 = v32; A.k16 = k16; A.v16 = v16; A.d_pos = d_pos; A.layer = layer; A.tok0 = t0; A.n_kv = kv->cfg.n_kv_heads;
     A.max_ctx = kv->cfg.max_ctx; A.rot = rot; A.pos_limit = pos_limit;
     A.nrow = std::min(kTbTileTok, M - t0) * 2 * kv->cfg.n_kv_heads;
@@ -327,7 +327,7 @@ void yka_kv_close(yka_kv* kv) {
   (void)hipDeviceSynchronize();
   if (kv->stream) (void)hipStreamDestroy(kv->stream);
   if (kv->tb) {
-    (void)hipFree(kv->tb->blob); (void)hipFree(kv->tb->pairs); (void)hipFree(kv->tb->gfac); (void)hipFree(kv->tb->mu); (void)hipFree(kv->tb->pool);
+    (void)hipFree(kv->tb->blob); (void)hipFree(kv->tb->desc); (void)hipFree(kv->tb->pairs); (void)hipFree(kv->tb->gfac); (void)hipFree(kv->tb->mu); (void)hipFree(kv->tb->pool);
     (void)hipFree(kv->tb->scr); (void)hipFree(kv->tb->stage);
     delete kv->tb;
   }
@@ -514,7 +514,7 @@ int yka_kvx256_probe(const float* x, int rows, int mode, int rot, int8_t* q8, ui
 // ---- trellis-coded rows ----
 }  // extern "C"
 namespace {
-struct TbInfo { int nm = 0, ngrp = 0, layers = 0, kv_heads = 0; bool has_trellis = false; };
+struct TbInfo { int nm = 0, ngrp = 0, layers = 0, kv_heads = 0, tables = 0; bool has_trellis = false; };
 // the checks of the reference's loaders (src/engine35.cpp:48-52, src/kvq_fast.hpp:52-76) plus bounds on every record
 // Little-endian view of a profile blob: a 100-byte header, then three offset arrays (multipliers, tables, groups).
 struct BlobView {
@@ -535,6 +535,7 @@ TbInfo tb_check_blob(const uint8_t* b, size_t n) {
   TbInfo I;
   I.layers = (int)V.half(18); I.kv_heads = (int)V.half(20); I.nm = (int)V.half(24); I.ngrp = (int)V.word(28);
   const unsigned n_tab = V.half(22);
+  I.tables = (int)n_tab;
   if (I.nm < 1 || I.nm > 16) bad("profile blob: bad scale-multiplier count");
   if (V.multipliers() + 4 * (size_t)I.nm > n || (size_t)V.word(36) + 4 * (size_t)n_tab > n || (size_t)V.word(40) + 4 * (size_t)I.ngrp > n)
     bad("profile blob: offsets outside the blob");
@@ -556,6 +557,32 @@ TbInfo tb_check_blob(const uint8_t* b, size_t n) {
   }
   return I;
 }
+// What the encoder kernels would otherwise look up in the blob by four dependent loads (layout: TbEncArgs::desc): a
+// record per group, then every table as aligned int16.  The blob has passed tb_check_blob.
+std::vector<uint32_t> tb_descriptors(const uint8_t* b, size_t n, const TbInfo& I) {
+  const BlobView V{b, n};
+  const size_t rec_words = 8 * (size_t)I.ngrp;
+  std::vector<uint32_t> D(rec_words + 128 * (size_t)I.tables, 0u);
+  for (int t = 0; t < I.tables; ++t) {
+    const size_t rec = V.table_record((unsigned)t);
+    for (int st = 0; st < 256; st += 2)
+      D[rec_words + 128 * (size_t)t + st / 2] = (uint32_t)(uint16_t)V.table_int(rec, st) | ((uint32_t)(uint16_t)V.table_int(rec, st + 1) << 16);
+  }
+  for (int g = 0; g < I.ngrp; ++g) {
+    const size_t rec = V.group_record(g);
+    uint32_t* d = &D[8 * (size_t)g];
+    const bool has_mean = b[rec + 5] != 0, trellis = b[rec] == 0;
+    d[0] = (uint32_t)b[rec] | ((uint32_t)b[rec + 1] << 8) | ((uint32_t)b[rec + 2] << 16) | ((uint32_t)b[rec + 3] << 24);
+    d[1] = (uint32_t)b[rec + 4] | ((uint32_t)has_mean << 8);
+    d[2] = (uint32_t)(rec + 8);
+    d[3] = (uint32_t)(rec + 8 + (has_mean ? 512 : 0));
+    if (trellis) {
+      d[4] = (uint32_t)(2 * (rec_words + 128 * (size_t)b[rec + 2]));            // in int16 units from the start of D
+      std::memcpy(&d[5], b + V.table_record(b[rec + 2]) + 4, 4);                 // gain
+    }
+  }
+  return D;
+}
 }  // namespace
 extern "C" {
 
@@ -570,12 +597,16 @@ int yka_tb_pack_unpack(const uint8_t* blob, size_t blob_len, const float* x, con
   DevBuf db(blob_len), dx(nx * 4), dg((size_t)rows * 4), dp((size_t)rows * 4), dy(nx * 4), dpay((size_t)rows * stride), dside((size_t)rows * 8),
          dd(nx * 4), scr(w_ofs + (size_t)kTile * I.nm * 32);
   HIPCHK(hipMemcpy(db.p, blob, blob_len, hipMemcpyHostToDevice));
+  const std::vector<uint32_t> desc = tb_descriptors(blob, blob_len, I);
+  DevBuf dd_desc(desc.size() * 4);
+  HIPCHK(hipMemcpy(dd_desc.p, desc.data(), desc.size() * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dx.p, x, nx * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dg.p, grp, (size_t)rows * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dp.p, pos, (size_t)rows * 4, hipMemcpyHostToDevice));
   for (int r0 = 0; r0 < rows; r0 += kTile) {
     TbEncArgs A{};
     A.blob = db.as<uint8_t>(); A.nm = I.nm; A.has_trellis = I.has_trellis;
+    A.desc = dd_desc.as<uint32_t>(); A.ngrp = I.ngrp; A.mult_off = BlobView{blob, blob_len}.word(32);
     A.yin = dx.as<float>(); A.grp = dg.as<int>(); A.pos = dp.as<int>(); A.row0 = r0; A.nrow = std::min(kTile, rows - r0);
     A.yout = dy.as<float>(); A.side = dside.as<uint32_t>(); A.scr = scr.as<uint8_t>(); A.scr_w_ofs = w_ofs;
     A.pay0 = dpay.as<uint8_t>(); A.stride = stride;
@@ -652,7 +683,7 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
     ~TbGuard() {
       if (done || !kv->tb) return;
       yka_kv::Tb* t = kv->tb;
-      (void)hipFree(t->blob); (void)hipFree(t->pairs); (void)hipFree(t->gfac); (void)hipFree(t->mu); (void)hipFree(t->pool); (void)hipFree(t->scr); (void)hipFree(t->stage);
+      (void)hipFree(t->blob); (void)hipFree(t->desc); (void)hipFree(t->pairs); (void)hipFree(t->gfac); (void)hipFree(t->mu); (void)hipFree(t->pool); (void)hipFree(t->scr); (void)hipFree(t->stage);
       delete t; kv->tb = nullptr;
     }
   } guard{kv};
@@ -664,6 +695,9 @@ int yka_kv_set_profile(yka_kv* kv, const uint8_t* blob, size_t blob_len) {
   const size_t jobs = (size_t)kTbTileTok * 2 * n_kv * I.nm;
   T->scr_w_ofs = jobs * 256;
   HIPCHK(hipMalloc((void**)&T->blob, blob_len)); HIPCHK(hipMemcpy(T->blob, blob, blob_len, hipMemcpyHostToDevice));
+  const std::vector<uint32_t> desc = tb_descriptors(blob, blob_len, I);
+  T->ngrp = I.ngrp; T->mult_off = V.word(32);
+  HIPCHK(hipMalloc((void**)&T->desc, desc.size() * 4)); HIPCHK(hipMemcpy(T->desc, desc.data(), desc.size() * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMalloc((void**)&T->pairs, pairs.size() * 4)); HIPCHK(hipMemcpy(T->pairs, pairs.data(), pairs.size() * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMalloc((void**)&T->gfac, gfac.size() * 4)); HIPCHK(hipMemcpy(T->gfac, gfac.data(), gfac.size() * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMalloc((void**)&T->mu, mu.size() * 4)); HIPCHK(hipMemcpy(T->mu, mu.data(), mu.size() * 4, hipMemcpyHostToDevice));

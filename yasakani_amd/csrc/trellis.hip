@@ -6,13 +6,15 @@
 // added in order), and the path search works on integers with the reference's tie rules, so rows are bit-identical.
 //
 // How the search is laid out is specific to wave64: a chunk of 64 elements is one path through 256 states and belongs to
-// ONE wave; lane l holds the costs of states l, l + 64, l + 128, l + 192.  The predecessors of state d are the states
-// p with p mod U == d >> kk (U = 256 >> kk), and 64 is a multiple of U, so all four states of a lane feed the same
-// group u = l mod U: the minimum of a group is a per-lane minimum of 4 followed by a butterfly over the lane bits above
-// log2(U) - 3 exchanges for 5-bit fields, 2 for 4-bit fields, done with a row rotation and the row / half swap
-// instructions of gfx950 - with no barrier, no cost array in LDS and no LDS round trip.  The smallest predecessor among
-// equal costs is found by a second butterfly on the candidate indices.  Back-pointers (one per group
-// and step) go to a 2 KB LDS block private to the wave; one lane walks them back.
+// ONE wave, four states per lane.  The states that can precede state d are the group { p : p mod U == d >> kk } (U =
+// 256 >> kk), so a step is "minimum of every group, then add each state's own step cost".  For 4- and 5-bit fields the
+// costs alternate between two lane arrangements chosen so that a group's minimum, found by lane-crossing minimum
+// instructions (quad permutations, row rotations, the row / half swaps of gfx950), already sits in the lanes whose states
+// continue that group: no barrier, no cost array in LDS, no LDS round trip.  Cost and predecessor index travel in one
+// 32-bit key, so one reduction yields both and the reference's tie rule (smallest predecessor); the step cost
+// (x - c)^2 loses the x^2 common to all states and becomes one 24-bit multiply-add.  The chosen predecessors (one per
+// group and step) go to a 2 KB LDS block private to the wave, a word per four steps, and are walked back in parallel
+// blocks.  3-bit fields keep a plainer form (group minima gathered through LDS, one lane walks back).
 #include "yka_internal.h"
 #include "rot256_device.h"
 #include <hip/hip_fp16.h>
@@ -21,15 +23,18 @@ namespace yka {
 namespace {
 
 // ---- the profile blob, read where it lies (little-endian, no alignment assumed) ----
+// The encoder kernels also get what the host has already looked up in the blob (`desc`, see TbEncArgs): one aligned
+// 32-byte record per group and the tables as aligned int16, so that a block reaches its table after ONE dependent load
+// instead of four (header -> offset of the group record -> record -> offset of the table record -> table).
 struct Profile {
   const uint8_t* base;
+  const uint32_t* desc = nullptr; int n_groups = 0; unsigned mult_off = 0;
   __device__ unsigned half_at(unsigned off) const { return base[off] | ((unsigned)base[off + 1] << 8); }
   __device__ unsigned word_at(unsigned off) const { return half_at(off) | (half_at(off + 2) << 16); }
   __device__ float float_at(unsigned off) const { return __uint_as_float(word_at(off)); }
   __device__ float f16_at(unsigned off) const { return __half2float(__ushort_as_half((unsigned short)half_at(off))); }
-  __device__ int multipliers() const { return (int)half_at(24); }
-  __device__ unsigned groups() const { return word_at(28); }
-  __device__ float multiplier(int i) const { return float_at(word_at(32) + 4u * (unsigned)i); }
+  __device__ unsigned groups() const { return desc ? (unsigned)n_groups : word_at(28); }
+  __device__ float multiplier(int i) const { return float_at((desc ? mult_off : word_at(32)) + 4u * (unsigned)i); }
   __device__ unsigned table_record(int t) const { return word_at(word_at(36) + 4u * (unsigned)t); }
   __device__ unsigned group_record(int g) const { return word_at(word_at(40) + 4u * (unsigned)g); }
 };
@@ -37,26 +42,38 @@ struct Profile {
 struct GroupRec {
   bool present; int mode, bits, table, guard, ndir; bool has_mean;
   unsigned mean_off, dir_off;            // byte offsets of the fp16 mean row and of the first fp16 direction
+  const int16_t* ints; float gain;       // descriptor form: the group's table
 };
 __device__ __forceinline__ GroupRec read_group(const Profile& P, int g) {
   GroupRec G{};
   G.present = (unsigned)g < P.groups();
   G.bits = 4;
-  if (G.present) {
-    const unsigned rec = P.group_record(g);
-    G.mode = P.base[rec]; G.bits = P.base[rec + 1]; G.table = P.base[rec + 2]; G.guard = P.base[rec + 3];
-    G.ndir = P.base[rec + 4]; G.has_mean = P.base[rec + 5] != 0;
-    G.mean_off = rec + 8; G.dir_off = G.mean_off + (G.has_mean ? 512u : 0u);
+  if (!G.present) return G;
+  if (P.desc) {
+    const uint4 lo = *reinterpret_cast<const uint4*>(P.desc + 8 * (size_t)g);
+    const uint2 hi = *reinterpret_cast<const uint2*>(P.desc + 8 * (size_t)g + 4);
+    G.mode = lo.x & 255u; G.bits = (lo.x >> 8) & 255u; G.table = (lo.x >> 16) & 255u; G.guard = lo.x >> 24;
+    G.ndir = lo.y & 255u; G.has_mean = (lo.y >> 8) != 0u;
+    G.mean_off = lo.z; G.dir_off = lo.w;
+    G.ints = reinterpret_cast<const int16_t*>(P.desc) + hi.x; G.gain = __uint_as_float(hi.y);
+    return G;
   }
+  const unsigned rec = P.group_record(g);
+  G.mode = P.base[rec]; G.bits = P.base[rec + 1]; G.table = P.base[rec + 2]; G.guard = P.base[rec + 3];
+  G.ndir = P.base[rec + 4]; G.has_mean = P.base[rec + 5] != 0;
+  G.mean_off = rec + 8; G.dir_off = G.mean_off + (G.has_mean ? 512u : 0u);
   return G;
 }
 // table of a trellis group: value of state s = (int16 at values + 2 s) / 256 * gain, each product rounded to fp32
-struct TableRec { unsigned values; float gain; };
+struct TableRec { unsigned values; float gain; const int16_t* ints; };
 __device__ __forceinline__ TableRec read_table(const Profile& P, const GroupRec& G) {
+  if (G.ints) return TableRec{0u, G.gain, G.ints};
   const unsigned rec = P.table_record(G.table);
-  return TableRec{rec + 12u, P.float_at(rec + 4u)};
+  return TableRec{rec + 12u, P.float_at(rec + 4u), nullptr};
 }
-__device__ __forceinline__ int table_int(const Profile& P, const TableRec& T, int state) { return (int)(short)P.half_at(T.values + 2u * (unsigned)state); }
+__device__ __forceinline__ int table_int(const Profile& P, const TableRec& T, int state) {
+  return T.ints ? (int)T.ints[state] : (int)(short)P.half_at(T.values + 2u * (unsigned)state);
+}
 __device__ __forceinline__ float table_value(int ti, float gain) { return __fmul_rn(__fmul_rn((float)ti, 1.f / 256.f), gain); }
 
 // fp32 value -> nearest fp16 -> fp32.  The empty asm keeps the compiler from merging the operation that produced v with the
@@ -401,7 +418,7 @@ __global__ void __launch_bounds__(256) tb_search_kernel(TbEncArgs A) {
   __shared__ uint8_t chosen[256];
   const int d = threadIdx.x, wave = d >> 6, lane = d & 63;
   const int row = blockIdx.x / A.nm, mult = blockIdx.x % A.nm;
-  const Profile P{A.blob};
+  const Profile P{A.blob, A.desc, A.ngrp, A.mult_off};
   const RowRef R = locate_row(A, row, rot_buf);
   const GroupRec G = read_group(P, R.group);
   if (!G.present || R.pos < G.guard || G.mode != 0) return;                // uniform over the block: nothing to search
@@ -478,7 +495,7 @@ __global__ void __launch_bounds__(256) tb_select_kernel(TbEncArgs A) {
   __shared__ float rot_buf[256];
   __shared__ uint8_t fld[256];
   const int d = threadIdx.x, row = blockIdx.x;
-  const Profile P{A.blob};
+  const Profile P{A.blob, A.desc, A.ngrp, A.mult_off};
   const RowRef R = locate_row(A, row, rot_buf);
   const GroupRec G = read_group(P, R.group);
   Coded C{0, 4, 1.f, R.x, false};

@@ -86,6 +86,11 @@ struct PostArgs {
 // pay0 (K) / pay1 (V) + (kvh * max_ctx + pos) * stride and its scale to scl0 / scl1 [kvh * max_ctx + pos].
 struct TbEncArgs {
   const uint8_t* blob; int nm; int has_trellis;
+  // what the host looked up in the blob (see tb_descriptors in abi.hip): [ngrp][8] words
+  //   { mode | bits << 8 | table << 16 | guard << 24, directions | has_mean << 8, byte offset of the mean row, of the
+  //     first direction, index (in int16 units, from desc) of the group's table as aligned int16, gain bits, 0, 0 }
+  // followed by the tables; mult_off: byte offset of the scale multipliers in the blob
+  const uint32_t* desc; int ngrp; unsigned mult_off;
   const float* k32; const float* v32; const uint16_t* k16; const uint16_t* v16;   // cache form: fp32 rows, or fp16 rows if k32 == nullptr
   const int* d_pos; int layer, tok0, n_kv, max_ctx, rot;
   const float* yin; const int* grp; const int* pos; int row0;
