@@ -472,20 +472,38 @@ __device__ __forceinline__ Coded code_flat(float* part8, float r) {
   return Coded{(int)q + 8, 4, step, __fmul_rn(q, step), true};
 }
 // trellis groups: the multiplier whose search left the smallest squared error (its 8 partial sums added in order from 0;
-// the first of equal errors), the state the search chose for this element under it
-__device__ __forceinline__ Coded code_trellis(const TbEncArgs& A, const Profile& P, const GroupRec& G, const Residual& Q, int row) {
-  const float* err = reinterpret_cast<const float*>(A.scr + A.scr_w_ofs) + (size_t)row * A.nm * 8;
-  int keep = 0; float least = 0.f;
-  for (int i = 0; i < A.nm; ++i) {
+// the first of equal errors), the state the search chose for this element under it.  What that needs from memory is
+// requested before the residual is computed, for all multipliers at once (the choice then costs no further round trip):
+// the states of this element, and - by thread i < multipliers - multiplier i and the error total of its search.
+constexpr int kMaxMult = 16;
+struct SearchResults { int state[kMaxMult]; };
+__device__ __forceinline__ SearchResults fetch_search_results(const TbEncArgs& A, const Profile& P, int row, float* totals, float* mults) {
+  SearchResults S;
+  const int d = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < kMaxMult; ++i) S.state[i] = i < A.nm ? (int)A.scr[((size_t)row * A.nm + i) * 256 + d] : 0;
+  if (d < A.nm) {
+    const float* err = reinterpret_cast<const float*>(A.scr + A.scr_w_ofs) + ((size_t)row * A.nm + d) * 8;
     float total = 0.f;
 #pragma unroll
-    for (int k = 0; k < 8; ++k) total = __fadd_rn(total, err[i * 8 + k]);
-    if (i == 0 || total < least) { least = total; keep = i; }
+    for (int k = 0; k < 8; ++k) total = __fadd_rn(total, err[k]);
+    totals[d] = total;
+    mults[d] = P.multiplier(d);
   }
-  const float s = trial_scale(P, Q.rms, keep);
-  const TableRec T = read_table(P, G);
-  const int state = A.scr[((size_t)row * A.nm + keep) * 256 + threadIdx.x];
-  return Coded{state & ((1 << G.bits) - 1), G.bits, s, __fmul_rn(table_value(table_int(P, T, state), T.gain), s), true};
+  return S;                                              // totals / mults: visible after the next barrier
+}
+__device__ __forceinline__ Coded code_trellis(const TbEncArgs& A, const Profile& P, const GroupRec& G, const Residual& Q, const SearchResults& S,
+                                              const float* totals, const float* mults) {
+  int keep = 0; float least = totals[0];
+  for (int i = 1; i < A.nm; ++i) { const float total = totals[i]; if (total < least) { least = total; keep = i; } }
+  float s = round_f16(__fmul_rn(Q.rms, mults[keep]));
+  if (s == 0.f) s = 1.f;
+  int state = 0;
+#pragma unroll
+  for (int i = 0; i < kMaxMult; ++i) state = i == keep ? S.state[i] : state;
+  float value = 0.f;
+  if (A.yout) { const TableRec T = read_table(P, G); value = __fmul_rn(table_value(table_int(P, T, state), T.gain), s); }
+  return Coded{state & ((1 << G.bits) - 1), G.bits, s, value, true};
 }
 
 // grid rows, block 256: codes the row (best multiplier of the search, or the flat quantizer), rebuilds what it decodes to,
@@ -494,6 +512,7 @@ __global__ void __launch_bounds__(256) tb_select_kernel(TbEncArgs A) {
   __shared__ float part8[8];
   __shared__ float rot_buf[256];
   __shared__ uint8_t fld[256];
+  __shared__ float totals[kMaxMult], mults[kMaxMult];
   const int d = threadIdx.x, row = blockIdx.x;
   const Profile P{A.blob, A.desc, A.ngrp, A.mult_off};
   const RowRef R = locate_row(A, row, rot_buf);
@@ -502,9 +521,11 @@ __global__ void __launch_bounds__(256) tb_select_kernel(TbEncArgs A) {
   float rebuilt = R.x;                                   // rows that stay uncoded come back as they are
   unsigned coef_bits = 0u;
   if (G.present && R.pos >= G.guard) {
-    const Residual Q = residual_of(part8, P, G, R.x);
+    SearchResults S{};
+    if (G.mode == 0) S = fetch_search_results(A, P, row, totals, mults);
+    const Residual Q = residual_of(part8, P, G, R.x);   // its barriers publish totals / mults
     if (G.mode == 1) C = code_flat(part8, Q.r);
-    else if (G.mode == 0) C = code_trellis(A, P, G, Q, row);
+    else if (G.mode == 0) C = code_trellis(A, P, G, Q, S, totals, mults);
     else C.value = Q.r;
     rebuilt = C.value;
 #pragma unroll
