@@ -38,6 +38,29 @@ def test_rows_bit_exact(native, oracle, kk, mu, dirs, flat):
     assert _same(got["dec"], oracle.tb_decode_rows(blob, grp, ref["words"], ref["scale"], ref["pc"]))
 
 
+@pytest.mark.parametrize("kk", [3, 4, 5])
+def test_rows_bit_exact_when_paths_tie(native, oracle, kk):
+    """Tables with few distinct values and rows of few distinct values: many paths cost the same, so the rows depend on the
+    tie rules (smallest predecessor among equal costs, smallest final state) and on the clamp of the targets."""
+    rng = np.random.default_rng(100 + kk)
+    coarse = (rng.integers(-3, 4, 256) * 256).astype(np.int16)      # 7 distinct table values
+    two = np.where(rng.random(256) < 0.5, -512, 512).astype(np.int16)
+    groups = [dict(mode=0, kk=kk, table=g & 1, guard=0, mu=None, dirs=[]) for g in range(8)]
+    blob = kvqp.build(1, 4, np.array([0.5, 1.0, 1.0, 2.0], np.float32), [(1.0, coarse), (1.0, two)], groups)
+    n = 64
+    y = rng.integers(-2, 3, (n, 256)).astype(np.float32)            # values in {-2..2}
+    y[0] = 0
+    y[1] = 1
+    y[2, ::2] = 40; y[2, 1::2] = -40                                # targets far outside the table: clamped
+    y[3] = np.where(np.arange(256) % 64 < 32, 3.0, -3.0)
+    grp = np.arange(n) % 8
+    pos = np.arange(n)
+    ref = oracle.tb_encode_rows(blob, grp, pos, y, stride_words=40)
+    got = native.tb_pack_unpack(blob, y, grp, pos, stride=160)
+    assert np.array_equal(got["words"], ref["words"])
+    assert _same(got["scale"], ref["scale"]) and _same(got["x"], ref["x"]) and _same(got["dec"], ref["x"])
+
+
 def test_guard_rows_and_missing_groups_pass_through(native, oracle):
     blob = kvqp.synthetic(layers=1, kk=5, seed=4, guard=7)
     y = _rows(9, 24)
