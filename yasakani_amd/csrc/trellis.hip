@@ -156,9 +156,9 @@ __device__ __forceinline__ Residual residual_of(float* part8, const Profile& P, 
   if (Q.rms == 0.f) Q.rms = 1.f;
   return Q;
 }
-// scale tried for multiplier i: rms * multiplier rounded to fp32, then to fp16; 0 -> 1
-__device__ __forceinline__ float trial_scale(const Profile& P, float rms, int i) {
-  const float s = round_f16(__fmul_rn(rms, P.multiplier(i)));
+// scale tried for a multiplier: rms * multiplier rounded to fp32, then to fp16; 0 -> 1
+__device__ __forceinline__ float trial_scale(float rms, float multiplier) {
+  const float s = round_f16(__fmul_rn(rms, multiplier));
   return s == 0.f ? 1.f : s;
 }
 
@@ -310,21 +310,32 @@ __device__ __forceinline__ int mad24(int x, int b, int a) {
   asm("v_mad_i32_i24 %0, %1, %2, %3" : "=v"(r) : "s"(x), "v"(b), "v"(a));
   return r;
 }
+// (x - c)^2 = x^2 - 2 x c + c^2, and x^2 is common to all states of a step: a state's step cost in key units is
+// a - x b with a = c^2 * 2^KK + j and b = 2 c * 2^KK, constants of the (lane, slot) in each arrangement
+struct StepConsts { int a0[4], a1[4], b0[4], b1[4]; };
 template <int KK, class Tab>
-__device__ __forceinline__ void wave_chunk(const int* xi, Tab tab, uint8_t* bp, uint8_t* st_out) {
+__device__ __forceinline__ StepConsts step_consts(Tab tab) {
+  const int lane = threadIdx.x & 63;
+  StepConsts C;
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const int s0 = state_at<KK, 0>(lane, k), s1 = state_at<KK, 1>(lane, k), c0 = tab(s0), c1 = tab(s1);
+    C.a0[k] = ((c0 * c0) << KK) | (s0 >> (8 - KK)); C.b0[k] = (2 * c0) << KK;
+    C.a1[k] = ((c1 * c1) << KK) | (s1 >> (8 - KK)); C.b1[k] = (2 * c1) << KK;
+  }
+  return C;
+}
+template <int KK>
+__device__ __forceinline__ void wave_chunk(const int* xi, const StepConsts& C, uint8_t* bp, uint8_t* st_out) {
   static_assert(KK == 4 || KK == 5, "packed search: 4 or 5 bits");
   constexpr int U = 256 >> KK, kFar = 40000000, kLow = (1 << KK) - 1;
   const int lane = threadIdx.x & 63;
   const int xreg = xi[lane];                           // target t lives in lane t
-  // (x - c)^2 = x^2 - 2 x c + c^2, and x^2 is common to all states of a step: a state's step cost in key units is
-  // a - x b with a = c^2 * 2^KK + j and b = 2 c * 2^KK, constants of the (lane, slot) in each arrangement
-  int a0[4], a1[4], b0[4], b1[4], sid[4], key[4];
+  const int (&a0)[4] = C.a0, (&a1)[4] = C.a1, (&b0)[4] = C.b0, (&b1)[4] = C.b1;
+  int sid[4], key[4];
 #pragma unroll
   for (int k = 0; k < 4; ++k) {
     sid[k] = state_at<KK, 0>(lane, k);
-    const int s1 = state_at<KK, 1>(lane, k), c0 = tab(sid[k]), c1 = tab(s1);
-    a0[k] = ((c0 * c0) << KK) | (sid[k] >> (8 - KK)); b0[k] = (2 * c0) << KK;
-    a1[k] = ((c1 * c1) << KK) | (s1 >> (8 - KK));     b1[k] = (2 * c1) << KK;
     key[k] = ((sid[k] == 0 ? 0 : kFar) << KK) | (sid[k] >> (8 - KK));
   }
   // is this lane the keeper of a group, and of which: its record of chosen predecessors goes to LDS every four steps
@@ -416,30 +427,37 @@ __global__ void __launch_bounds__(256) tb_search_kernel(TbEncArgs A) {
   __shared__ int target[256];
   __shared__ __align__(16) uint8_t back[4][64 * 32];
   __shared__ uint8_t chosen[256];
+  __shared__ int16_t table[256];
   const int d = threadIdx.x, wave = d >> 6, lane = d & 63;
   const int row = blockIdx.x / A.nm, mult = blockIdx.x % A.nm;
   const Profile P{A.blob, A.desc, A.ngrp, A.mult_off};
   const RowRef R = locate_row(A, row, rot_buf);
   const GroupRec G = read_group(P, R.group);
   if (!G.present || R.pos < G.guard || G.mode != 0) return;                // uniform over the block: nothing to search
-  const Residual Q = residual_of(part8, P, G, R.x);
+  // everything the search needs from memory is requested before the residual's block reductions
   const TableRec T = read_table(P, G);
-  const float s = trial_scale(P, Q.rms, mult);
+  const auto tab = [&](int state) { return table_int(P, T, state); };
+  StepConsts C{};
+  int ci4[4] = {0, 0, 0, 0};
+  if (G.bits == 5) C = step_consts<5>(tab);
+  else if (G.bits == 4) C = step_consts<4>(tab);
+  else {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) ci4[k] = tab(lane + 64 * k);
+  }
+  const float mult_value = P.multiplier(mult);
+  table[d] = (int16_t)tab(d);                            // published by the barriers of the block reductions
+  const Residual Q = residual_of(part8, P, G, R.x);
+  const float s = trial_scale(Q.rms, mult_value);
   // integer target of element d: the residual in units of s / 256, clamped
   target[d] = (int)fminf(fmaxf(rintf(__fmul_rn(__fdiv_rn(Q.r, s), 256.f)), -2048.f), 2048.f);
   __syncthreads();
-  const auto tab = [&](int state) { return table_int(P, T, state); };
-  if (G.bits == 5) wave_chunk<5>(target + 64 * wave, tab, back[wave], chosen + 64 * wave);
-  else if (G.bits == 4) wave_chunk<4>(target + 64 * wave, tab, back[wave], chosen + 64 * wave);
-  else {
-    int ci4[4];
-#pragma unroll
-    for (int k = 0; k < 4; ++k) ci4[k] = tab(lane + 64 * k);
-    wave_chunk3(target + 64 * wave, ci4, back[wave], chosen + 64 * wave);
-  }
+  if (G.bits == 5) wave_chunk<5>(target + 64 * wave, C, back[wave], chosen + 64 * wave);
+  else if (G.bits == 4) wave_chunk<4>(target + 64 * wave, C, back[wave], chosen + 64 * wave);
+  else wave_chunk3(target + 64 * wave, ci4, back[wave], chosen + 64 * wave);
   // squared error of this multiplier: element d of the row is lane `lane` of wave `wave`; summed per run of 32 elements
   const int state = chosen[d];
-  const float miss = __fsub_rn(Q.r, __fmul_rn(table_value(table_int(P, T, state), T.gain), s));
+  const float miss = __fsub_rn(Q.r, __fmul_rn(table_value((int)table[state], T.gain), s));
   float sq = __fmul_rn(miss, miss);
 #pragma unroll
   for (int o = 16; o; o >>= 1) sq = __fadd_rn(sq, __shfl_xor(sq, o, 64));
@@ -496,8 +514,7 @@ __device__ __forceinline__ Coded code_trellis(const TbEncArgs& A, const Profile&
                                               const float* totals, const float* mults) {
   int keep = 0; float least = totals[0];
   for (int i = 1; i < A.nm; ++i) { const float total = totals[i]; if (total < least) { least = total; keep = i; } }
-  float s = round_f16(__fmul_rn(Q.rms, mults[keep]));
-  if (s == 0.f) s = 1.f;
+  const float s = trial_scale(Q.rms, mults[keep]);
   int state = 0;
 #pragma unroll
   for (int i = 0; i < kMaxMult; ++i) state = i == keep ? S.state[i] : state;
