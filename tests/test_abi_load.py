@@ -38,6 +38,50 @@ def test_bad_config_is_rejected_with_a_message(native):
             native.KvCache(**kw)
 
 
+def test_profile_blobs_are_checked_before_any_device_call(native):
+    """Every corruption below is refused by the host-side parser of the profile blob (magic, version, length, element
+    count, multiplier count, offsets, table geometry, table range, group records), so this runs without a GPU."""
+    import struct
+
+    import numpy as np
+
+    from yasakani_amd import kvqp
+    good = kvqp.synthetic(layers=1, kk=5, seed=3, mu=True, dirs=1)
+    info = kvqp.parse(good)
+    y = np.zeros((1, 256), np.float32)
+
+    def refused(blob, frag):
+        with pytest.raises(native.YkaError, match=frag):
+            native.tb_pack_unpack(bytes(blob), y, [0], [0])
+
+    off_m, off_t, off_g = struct.unpack_from("<III", good, 32)
+    (t0,) = struct.unpack_from("<I", good, off_t)
+    (g0,) = struct.unpack_from("<I", good, off_g)
+    assert info is not None and good[:4] == b"KVQP"
+    b = bytearray(good); b[0] = ord("X"); refused(b, "KVQP")
+    b = bytearray(good); struct.pack_into("<H", b, 4, 2); refused(b, "KVQP")                      # version
+    refused(good[:-1], "KVQP")                                                                     # length field disagrees
+    refused(good[:60], "KVQP")                                                                     # shorter than a header
+    b = bytearray(good); struct.pack_into("<H", b, 16, 128); refused(b, "256 elements")
+    b = bytearray(good); struct.pack_into("<H", b, 24, 0); refused(b, "multiplier count")
+    b = bytearray(good); struct.pack_into("<H", b, 24, 17); refused(b, "multiplier count")
+    b = bytearray(good); struct.pack_into("<I", b, 40, len(good) - 2); refused(b, "offsets outside")
+    b = bytearray(good); struct.pack_into("<I", b, 28, 1 << 30); refused(b, "offsets outside")    # group count
+    b = bytearray(good); b[t0] = 7; refused(b, "8 state bits")
+    b = bytearray(good); b[t0 + 2] = 32; refused(b, "chunks of 64")
+    b = bytearray(good); struct.pack_into("<h", b, t0 + 12 + 2 * 100, 1101); refused(b, "out of range")
+    b = bytearray(good); struct.pack_into("<h", b, t0 + 12 + 2 * 5, -1101); refused(b, "out of range")
+    b = bytearray(good); struct.pack_into("<I", b, off_t, len(good) - 100); refused(b, "tables must have|out of range|state bits")
+    b = bytearray(good); struct.pack_into("<I", b, off_g, len(good) - 4); refused(b, "group record")
+    b = bytearray(good); b[g0] = 2; refused(b, "bad group record")                                 # mode
+    b = bytearray(good); b[g0 + 4] = 3; refused(b, "bad group record")                             # directions
+    b = bytearray(good); b[g0 + 1] = 6; refused(b, "3..5 bits")
+    b = bytearray(good); b[g0 + 1] = 2; refused(b, "3..5 bits")
+    b = bytearray(good); b[g0 + 2] = 9; refused(b, "3..5 bits and a table")                        # table index
+    with pytest.raises(native.YkaError, match="stride"):
+        native.tb_pack_unpack(good, y, [0], [0], stride=128)
+
+
 def test_product_does_not_import_the_oracle():
     pkg = os.path.join(ROOT, "yasakani_amd")
     for dirpath, _, files in os.walk(pkg):
