@@ -66,7 +66,8 @@ def test_profile_blobs_are_checked_before_any_device_call(native):
     b = bytearray(good); struct.pack_into("<H", b, 24, 0); refused(b, "multiplier count")
     b = bytearray(good); struct.pack_into("<H", b, 24, 17); refused(b, "multiplier count")
     b = bytearray(good); struct.pack_into("<I", b, 40, len(good) - 2); refused(b, "offsets outside")
-    b = bytearray(good); struct.pack_into("<I", b, 28, 1 << 30); refused(b, "offsets outside")    # group count
+    for count in (1 << 30, 1 << 31, 0xFFFFFFFF):                                                   # group count (also as a negative int)
+        b = bytearray(good); struct.pack_into("<I", b, 28, count); refused(b, "offsets outside")
     b = bytearray(good); b[t0] = 7; refused(b, "8 state bits")
     b = bytearray(good); b[t0 + 2] = 32; refused(b, "chunks of 64")
     b = bytearray(good); struct.pack_into("<h", b, t0 + 12 + 2 * 100, 1101); refused(b, "out of range")

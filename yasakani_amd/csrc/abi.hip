@@ -533,12 +533,14 @@ TbInfo tb_check_blob(const uint8_t* b, size_t n) {
   if (V.half(4) != 1 || V.word(8) != n) bad("not a KVQP v1 profile blob");
   if (V.half(16) != 256) bad("profile blob: rows must have 256 elements");
   TbInfo I;
-  I.layers = (int)V.half(18); I.kv_heads = (int)V.half(20); I.nm = (int)V.half(24); I.ngrp = (int)V.word(28);
+  I.layers = (int)V.half(18); I.kv_heads = (int)V.half(20); I.nm = (int)V.half(24);
+  const size_t n_grp = V.word(28);                       // checked as an unsigned count before it becomes an int
   const unsigned n_tab = V.half(22);
   I.tables = (int)n_tab;
   if (I.nm < 1 || I.nm > 16) bad("profile blob: bad scale-multiplier count");
-  if (V.multipliers() + 4 * (size_t)I.nm > n || (size_t)V.word(36) + 4 * (size_t)n_tab > n || (size_t)V.word(40) + 4 * (size_t)I.ngrp > n)
+  if (V.multipliers() + 4 * (size_t)I.nm > n || (size_t)V.word(36) + 4 * (size_t)n_tab > n || (size_t)V.word(40) + 4 * n_grp > n)
     bad("profile blob: offsets outside the blob");
+  I.ngrp = (int)n_grp;                                   // < n / 4 <= 2^30
   for (unsigned t = 0; t < n_tab; ++t) {
     const size_t rec = V.table_record(t);
     if (rec + 12 + 512 > n || b[rec] != 8 || b[rec + 2] != 64 || b[rec + 3] != 8) bad("profile blob: tables must have 8 state bits, chunks of 64");
@@ -592,12 +594,12 @@ int yka_tb_pack_unpack(const uint8_t* blob, size_t blob_len, const float* x, con
   if (!x || !grp || !pos || rows < 1 || !y_fq || !pay || !side || !y_dec) throw std::runtime_error("bad argument");
   if (stride < 160 || stride > 1024 || stride % 4) throw std::runtime_error("stride must be a multiple of 4 in [160, 1024]");
   const TbInfo I = tb_check_blob(blob, blob_len);
+  const std::vector<uint32_t> desc = tb_descriptors(blob, blob_len, I);   // host work first: nothing is allocated for a bad blob
   constexpr int kTile = 1024;                        // rows per launch
   const size_t nx = (size_t)rows * 256, w_ofs = (size_t)kTile * I.nm * 256;
   DevBuf db(blob_len), dx(nx * 4), dg((size_t)rows * 4), dp((size_t)rows * 4), dy(nx * 4), dpay((size_t)rows * stride), dside((size_t)rows * 8),
          dd(nx * 4), scr(w_ofs + (size_t)kTile * I.nm * 32);
   HIPCHK(hipMemcpy(db.p, blob, blob_len, hipMemcpyHostToDevice));
-  const std::vector<uint32_t> desc = tb_descriptors(blob, blob_len, I);
   DevBuf dd_desc(desc.size() * 4);
   HIPCHK(hipMemcpy(dd_desc.p, desc.data(), desc.size() * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dx.p, x, nx * 4, hipMemcpyHostToDevice));
