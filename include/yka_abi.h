@@ -45,7 +45,9 @@ typedef struct yka_kv_config {
   int32_t device;      /* HIP device ordinal */
 } yka_kv_config;
 
-/* replaces the KV reservation of yskn_open (yskn_abi.h:22; engine35.cpp:303-329). NULL on error. */
+/* replaces the KV reservation of yskn_open (yskn_abi.h:22; engine35.cpp:303-329). NULL on error.  Refused before any
+ * device call: a configuration outside the ranges above, more than 1024 KV heads, or n_layers x max_ctx x n_kv_heads that
+ * describes more than 1 TiB of cache. */
 YKA_API yka_kv* yka_kv_open(const yka_kv_config* cfg);
 /* replaces yskn_close (yskn_abi.h:23) for the KV containers */
 YKA_API void yka_kv_close(yka_kv* kv);

@@ -33,7 +33,8 @@ def test_build_info_and_error_string_without_gpu(native):
 def test_bad_config_is_rejected_with_a_message(native):
     # validation happens before any device call, so this runs without a GPU
     for kw, frag in [(dict(head_dim=64), "head_dim"), (dict(n_heads=28), "n_heads"), (dict(max_ctx=1000), "max_ctx"),
-                     (dict(n_layers=0), "n_layers"), (dict(max_rows=0), "max_rows")]:
+                     (dict(n_layers=0), "n_layers"), (dict(max_rows=0), "max_rows"),
+                     (dict(n_layers=1 << 20, max_ctx=1 << 30), "1 TiB"), (dict(n_heads=6 * 2048, n_kv_heads=2048), "n_kv_heads")]:
         with pytest.raises(native.YkaError, match=frag):
             native.KvCache(**kw)
 

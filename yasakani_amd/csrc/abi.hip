@@ -288,6 +288,14 @@ yka_kv* yka_kv_open(const yka_kv_config* cfg) {
     if (cfg->n_layers < 1) throw std::runtime_error("n_layers must be >= 1");
     if (cfg->max_ctx < kPageTok || cfg->max_ctx % kPageTok) throw std::runtime_error("max_ctx must be a positive multiple of 256");
     if (cfg->max_rows < 1 || cfg->max_rows > 8192) throw std::runtime_error("max_rows must be in [1, 8192]");
+    {
+      // sizes are 64-bit products of four caller-given ints: refuse what cannot exist before one of them wraps around
+      if (cfg->n_kv_heads > 1024) throw std::runtime_error("n_kv_heads must be at most 1024");
+      const unsigned __int128 per_token = cfg->head_dim == 256 ? (unsigned __int128)kPage256Bytes / kPageTok * cfg->n_kv_heads
+                                                                 : (unsigned __int128)kv_page_bytes(cfg->n_kv_heads) / kPageTok;
+      if (per_token * (unsigned __int128)cfg->max_ctx * (unsigned __int128)cfg->n_layers > ((unsigned __int128)1 << 40))
+        throw std::runtime_error("n_layers x max_ctx x n_kv_heads describes a cache of more than 1 TiB");
+    }
     int ndev = 0;
     HIPCHK(hipGetDeviceCount(&ndev));
     if (cfg->device < 0 || cfg->device >= ndev) throw std::runtime_error("device out of range");
