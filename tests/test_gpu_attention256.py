@@ -82,11 +82,13 @@ def test_depth_table_splits_and_pages(native, oracle):
                 few = kv.layer_call(0, q, None, None, ctx, depth=depth)
                 kv.set_opt(1, 97)
                 many = kv.layer_call(0, q, None, None, ctx, depth=depth)
+                kv.set_opt(1, 200)                                            # more than 128: the combiner's widest form
+                most = kv.layer_call(0, q, None, None, ctx, depth=depth)
     ref.append(k[ctx:], v[ctx:], ctx)
     expect = ref.attend_f32(q, ctx, depth=depth)
     assert_attn_close(outs[0], expect, "depth table")
     assert np.array_equal(outs[0].view(np.uint16), outs[1].view(np.uint16))      # paged == contiguous, bit for bit
-    assert_attn_close(few, expect, "3 splits"); assert_attn_close(many, expect, "97 splits")
+    assert_attn_close(few, expect, "3 splits"); assert_attn_close(many, expect, "97 splits"); assert_attn_close(most, expect, "200 splits")
 
 
 def test_entry_points_of_the_other_format_refuse(native):

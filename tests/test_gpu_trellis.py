@@ -163,13 +163,13 @@ def test_depth_table_and_split_counts(native, oracle):
             m = min(64, ctx + M - p)
             kv.append256_f32_host(0, k[p:p + m], v[p:p + m], p, rotate=False)
         outs = []
-        for S in (0, 3, 97):
+        for S in (0, 3, 97, 200):
             kv.set_opt(1, S)
             outs.append(kv.layer_call(0, q, None, None, ctx, depth=depth))
     enc = _oracle_rows(oracle, blob, 0, k, v)
     kd = np.stack([enc[0, h]["x"] for h in range(KVH)]); vd = np.stack([enc[1, h]["x"] for h in range(KVH)])
     expect = oracle.tb_attend_f64(kd, vd, q, ctx, depth=depth)
-    for o, name in zip(outs, ("default", "3 splits", "97 splits")):
+    for o, name in zip(outs, ("default", "3 splits", "97 splits", "200 splits")):
         assert_attn_close(o, expect, name)
 
 

@@ -397,8 +397,8 @@ __global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
 
 // combiner (src/attention_kv4q.cu:325-332) for 256-channel rows: grid (n_heads, M), block 256 = 8 split lanes x 32 channel
 // lanes of 8 channels; the split lanes run in parallel and are summed through LDS.  S <= 256.  kInFlight = partial rows a
-// split lane requests before it uses any: 16 covers 128 splits in one memory round trip (decode: few, long workgroups),
-// 4 keeps the register count low where thousands of workgroups run (wide windows).  Rows of weight 0 are not read.
+// split lane requests before it uses any: 16 covers 128 splits (decode: few, long workgroups; 32 for up to 256 splits), 4 covers
+// 32 and keeps the register count low where thousands of workgroups run (wide windows).
 template <int kInFlight>
 __global__ void __launch_bounds__(256) combine256_kernel(CombineArgs A) {
   __shared__ float s_w[256];
@@ -406,6 +406,18 @@ __global__ void __launch_bounds__(256) combine256_kernel(CombineArgs A) {
   __shared__ float s_wsum[8];
   const int head = blockIdx.x, tok = blockIdx.y, tid = threadIdx.x;
   const size_t p0 = (size_t)tok * A.S * A.n_heads + head;
+  // 8 split lanes; each takes splits sl, sl + 8, ... (at most kInFlight of them: the launcher picks kInFlight so that
+  // 8 * kInFlight >= S).  Their partial rows are requested first, together with the (m, l) pairs the weights come from:
+  // one memory round trip instead of two.  A row of weight 0 may be one that no workgroup wrote: it is zeroed before use.
+  const int sl = tid >> 5, c8 = (tid & 31) * 8;
+  const uint16_t* src = A.pacc16 + p0 * kD2 + c8;
+  const size_t stride = (size_t)A.n_heads * kD2;
+  uint4 u[kInFlight];
+#pragma unroll
+  for (int k = 0; k < kInFlight; ++k) {
+    const int sp = sl + 8 * k;
+    u[k] = sp < A.S ? *reinterpret_cast<const uint4*>(src + (size_t)sp * stride) : make_uint4(0, 0, 0, 0);
+  }
   float pmv = -1e30f, plv = 0.f;
   if (tid < A.S) { pmv = A.pm[p0 + (size_t)tid * A.n_heads]; plv = A.pl[p0 + (size_t)tid * A.n_heads]; }
   float M2 = pmv;
@@ -417,26 +429,17 @@ __global__ void __launch_bounds__(256) combine256_kernel(CombineArgs A) {
   __syncthreads();
   s_w[tid] = (tid < A.S && pmv > -1e29f) ? exp2f(pmv - M2) * plv : 0.f;
   __syncthreads();
-  const int sl = tid >> 5, c8 = (tid & 31) * 8;
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float wsum = 0.f;
-  const uint16_t* src = A.pacc16 + p0 * kD2 + c8;
-  const size_t stride = (size_t)A.n_heads * kD2;
-  for (int s0 = sl; s0 < A.S; s0 += 8 * kInFlight) {
-    uint4 u[kInFlight]; float w[kInFlight];
 #pragma unroll
-    for (int k = 0; k < kInFlight; ++k) {
-      const int sp = s0 + 8 * k;
-      w[k] = sp < A.S ? s_w[sp] : 0.f;
-      u[k] = (sp < A.S && w[k] != 0.f) ? *reinterpret_cast<const uint4*>(src + (size_t)sp * stride) : make_uint4(0, 0, 0, 0);
-    }
+  for (int k = 0; k < kInFlight; ++k) {
+    const int sp = sl + 8 * k;
+    const float w = sp < A.S ? s_w[sp] : 0.f;
+    const uint4 r = w != 0.f ? u[k] : make_uint4(0, 0, 0, 0);
+    const h8 v = __builtin_bit_cast(h8, r);
 #pragma unroll
-    for (int k = 0; k < kInFlight; ++k) {
-      const h8 v = __builtin_bit_cast(h8, u[k]);
-#pragma unroll
-      for (int c = 0; c < 8; ++c) acc[c] += w[k] * (float)v[c];
-      wsum += w[k];
-    }
+    for (int c = 0; c < 8; ++c) acc[c] += w * (float)v[c];
+    wsum += w;
   }
 #pragma unroll
   for (int c = 0; c < 8; ++c) s_o[sl][c8 + c] = acc[c];
@@ -464,7 +467,9 @@ void launch_attend256(const AttnArgs& A, hipStream_t st) {
   else hipLaunchKernelGGL(attend256_kernel<false>, dim3(A.S, A.kv.n_kv, (A.M + 1) / 2), dim3(256), 0, st, A);
 }
 void launch_combine256(const CombineArgs& A, hipStream_t st) {
-  if (A.S > 32) hipLaunchKernelGGL(combine256_kernel<16>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
+  // 8 split lanes x kInFlight rows each must cover the S <= 256 splits
+  if (A.S > 128) hipLaunchKernelGGL(combine256_kernel<32>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
+  else if (A.S > 32) hipLaunchKernelGGL(combine256_kernel<16>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
   else hipLaunchKernelGGL(combine256_kernel<4>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
 }
 void launch_export_rows256(const KvView& kv, int pos0, int n, uint32_t* kw, float* ks, uint32_t* vw, float* vs, hipStream_t st) {
