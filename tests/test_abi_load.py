@@ -84,6 +84,32 @@ def test_profile_blobs_are_checked_before_any_device_call(native):
         native.tb_pack_unpack(good, y, [0], [0], stride=128)
 
 
+def test_probe_entry_points_refuse_bad_arguments_before_any_device_call(native):
+    import numpy as np
+    L = native.lib()
+    x = np.zeros((2, 256), np.float32); y = np.zeros_like(x); sc = np.zeros(2, np.float32)
+    q8 = np.zeros((2, 256), np.int8); words = np.zeros((2, 32), np.uint32)
+    P = native._ptr
+
+    def refused(rc, frag):
+        assert rc != 0 and frag in L.yka_last_error().decode()
+
+    refused(L.yka_kvx256_probe(None, 2, 0, 0, P(q8), None, P(sc), P(y)), "bad argument")
+    refused(L.yka_kvx256_probe(P(x), 0, 0, 0, P(q8), None, P(sc), P(y)), "bad argument")
+    refused(L.yka_kvx256_probe(P(x), -5, 1, 0, None, P(words), P(sc), P(y)), "bad argument")
+    refused(L.yka_kvx256_probe(P(x), 2, 2, 0, P(q8), P(words), P(sc), P(y)), "bad argument")
+    refused(L.yka_kvx256_probe(P(x), 2, 0, 0, None, P(words), P(sc), P(y)), "selected mode")
+    refused(L.yka_kvx256_probe(P(x), 2, 1, 1, P(q8), None, P(sc), P(y)), "selected mode")
+    from yasakani_amd import kvqp
+    blob = np.frombuffer(kvqp.synthetic(), np.uint8)
+    grp = np.zeros(2, np.int32); pay = np.zeros((2, 160), np.uint8); side = np.zeros((2, 2), np.uint32)
+    refused(L.yka_tb_pack_unpack(P(blob), blob.size, None, P(grp), P(grp), 2, 160, P(y), P(pay), P(side), P(x)), "bad argument")
+    refused(L.yka_tb_pack_unpack(P(blob), blob.size, P(x), P(grp), P(grp), 0, 160, P(y), P(pay), P(side), P(x)), "bad argument")
+    refused(L.yka_tb_pack_unpack(P(blob), blob.size, P(x), P(grp), P(grp), 2, 162, P(y), P(pay), P(side), P(x)), "stride")
+    refused(L.yka_tb_pack_unpack(P(blob), blob.size, P(x), P(grp), P(grp), 2, 2048, P(y), P(pay), P(side), P(x)), "stride")
+    refused(L.yka_tb_pack_unpack(None, 0, P(x), P(grp), P(grp), 2, 160, P(y), P(pay), P(side), P(x)), "KVQP")
+
+
 def test_product_does_not_import_the_oracle():
     pkg = os.path.join(ROOT, "yasakani_amd")
     for dirpath, _, files in os.walk(pkg):
