@@ -222,6 +222,22 @@ def test_window_across_a_page_boundary_in_shuffled_pages(native, oracle):
         _rows_equal(kv, oc, ctx, M)
 
 
+@pytest.mark.parametrize("ctx", [31, 1023, 1024])
+def test_rows_no_query_row_sees_are_still_stored(native, oracle, ctx):
+    """Two sibling rows (depth table [0, 0]): no query row of the pass sees the second row, and when it opens a new 32-key
+    tile (ctx + 1 a multiple of 32) no workgroup's key range holds it - the decode launch must store it all the same."""
+    M = 2
+    kv, oc, q, kn, vn = _fill(native, oracle, 640 + ctx, ctx, M)
+    depth = np.array([0, 0], np.uint8)
+    with kv:
+        out = kv.layer_call(0, q, kn, vn, ctx, depth=depth)
+        oc.append(kn, vn, ctx)
+        got = kv.export_rows(0, ctx, M)
+        assert (got[0] == oc.kc[:, ctx:ctx + M]).all() and (got[1] == oc.ks[:, ctx:ctx + M]).all()
+        assert (got[2] == oc.vc[:, ctx:ctx + M]).all() and (got[3] == oc.vs[:, ctx:ctx + M]).all()
+        assert_attn_close(out, oc.attend_f32(q, ctx, depth, want_f32=True)[1], f"siblings at ctx={ctx}")
+
+
 def test_depth_table_on_a_wide_window(native, oracle):
     ctx, M = 900, 24
     kv, oc, q, kn, vn = _fill(native, oracle, 612, ctx, M)

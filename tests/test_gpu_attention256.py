@@ -91,6 +91,24 @@ def test_depth_table_splits_and_pages(native, oracle):
     assert_attn_close(few, expect, "3 splits"); assert_attn_close(many, expect, "97 splits"); assert_attn_close(most, expect, "200 splits")
 
 
+@pytest.mark.parametrize("ctx", [31, 1023])
+def test_rows_no_query_row_sees_are_still_stored(native, oracle, ctx):
+    """Sibling rows (depth table [0, 0]) whose second row opens a new 32-key tile: stored although no key range holds it."""
+    M = 2
+    q, k, v = _inputs(90 + ctx, ctx, M)
+    depth = np.array([0, 0], np.uint8)
+    ref = oracle.Cache(1280, NH, KVH, D)
+    with native.KvCache(head_dim=D, max_ctx=1280) as kv:
+        _fill(kv, ref, k, v, ctx)
+        out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx, depth=depth)
+        got = kv.export_rows(0, ctx, M)
+    ref.append(k[ctx:], v[ctx:], ctx)
+    assert np.array_equal(got[0], ref.kc[:, ctx:ctx + M]) and np.array_equal(got[2], ref.vc[:, ctx:ctx + M])
+    assert np.array_equal(got[1].view(np.uint32), ref.ks[:, ctx:ctx + M].view(np.uint32))
+    assert np.array_equal(got[3].view(np.uint32), ref.vs[:, ctx:ctx + M].view(np.uint32))
+    assert_attn_close(out, ref.attend_f32(q, ctx, depth=depth), f"siblings at ctx={ctx}")
+
+
 def test_entry_points_of_the_other_format_refuse(native):
     with native.KvCache(head_dim=D, max_ctx=256) as kv:
         with pytest.raises(native.YkaError, match="128"):

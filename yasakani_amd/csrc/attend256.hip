@@ -252,7 +252,10 @@ __global__ void __launch_bounds__(256, 2) attend256_kernel(AttnArgs A) {
     bool mine = false;
     for (int t = 0; t < A.M; ++t) {
       const int r = pos + A.tok0 + t;
-      if (r < 0 || r >= A.kv.max_ctx || (r >> 5) < tile0 || (r >> 5) >= tile1) continue;    // uniform over the workgroup
+      // A row no query row of this launch can see (a depth table may say so) lies past the last tile when it opens a new
+      // one: nobody reads it now, the last workgroup in use stores it.  All conditions are uniform over the workgroup.
+      const bool held = (r >> 5) >= tile0 && (r >> 5) < tile1, unseen = (r >> 5) >= ntiles && split == s_used - 1;
+      if (r < 0 || r >= A.kv.max_ctx || !(held || unseen)) continue;
       mine = true;
       const size_t e = ((size_t)(A.tok0 + t) * A.kv.n_kv + kvh) * kD2 + threadIdx.x;
       quant_store_row256(A.kv, kvh, r, false, __half2float(__ushort_as_half(A.k16[e])), threadIdx.x, a_red, a_fld);

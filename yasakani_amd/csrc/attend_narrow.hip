@@ -159,7 +159,10 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
     bool mine = false;
     for (int t = 0; t < A.M; ++t) {
       const int r = pos + A.tok0 + t;              // k16/v16 point at row 0 of the pass, this slice starts at row tok0
-      if (r < 0 || r >= A.kv.max_ctx || (r >> 5) < tile0 || (r >> 5) >= tile1) continue;
+      // A row no query row of this launch can see (a depth table may say so) lies past the last tile when it opens a new
+      // one: nobody reads it now, the last workgroup in use stores it.  All conditions are uniform over the workgroup.
+      const bool held = (r >> 5) >= tile0 && (r >> 5) < tile1, unseen = (r >> 5) >= ntiles && split == s_used - 1;
+      if (r < 0 || r >= A.kv.max_ctx || !(held || unseen)) continue;
       mine = true;
       const bool isv = threadIdx.x >= 128;
       const uint16_t* src = (isv ? A.v16 : A.k16) + ((size_t)(A.tok0 + t) * A.kv.n_kv + kvh) * kD;
