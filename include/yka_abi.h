@@ -83,7 +83,9 @@ YKA_API int yka_append(yka_kv* kv, int layer, const uint16_t* d_k16, const uint1
                        const int* d_pos, void* hip_stream);
 
 /* Attention over the cache: row t of d_q16 ([M][n_heads][128] fp16) attends to keys [0, *d_pos + depth(t) + 1),
- * depth(t) = d_depth ? d_depth[t] : t (q35_atx.cu:110-118); writes d_out16 [M][n_heads][128] fp16.
+ * depth(t) = d_depth ? d_depth[t] : t (q35_atx.cu:110-118); writes d_out16 [M][n_heads][128] fp16.  A depth table names rows
+ * of the pass, so depth(t) <= t: a larger value reaches past the rows this pass appends, into rows nobody has written
+ * (the table lives on the device and is not checked).
  * Replaces launch_q35_prefill_atx_pk / launch_q35_atx_pk + launch_q35_combine (q35_atxpk.hpp:15-24, q35.hpp:153-156;
  * call site engine35.cpp:921-934) and launch_attention + launch_attn_combine of the v1 engine (args.hpp:36-37). */
 YKA_API int yka_attend(yka_kv* kv, int layer, const uint16_t* d_q16, int M, const int* d_pos,
