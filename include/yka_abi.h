@@ -268,6 +268,21 @@ YKA_API void yka_pass_destroy(yka_pass* p);
 YKA_API int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, int pos,
                            int mode, int use_graph, int reps, float* ms, uint16_t* out16_last);
 
+/* Machine probe: fixed instruction mixes that time themselves, for the figures the kernels are designed around and the
+ * roofline is read against.  Model: the timing part of the reference's bench hooks (kvx_probe.cu:407-413).  Synchronous;
+ * allocates.  `blocks` workgroups of `threads` (256 or 512) lanes; every kind runs once untimed, then once timed.
+ *   kind 0: per wave, iters x 4 x (one v_mfma_f32_32x32x16_f16 followed by p0 independent v_fma_f32), p0 in {0,2,4,6,8}
+ *   kind 1: per wave, iters x 8 v_mfma_f32_16x16x32_f16 (256 lanes)
+ *   kind 2: per wave, iters x 32 instructions of one vector opcode: p0 = 0 v_exp_f32, 1 v_pk_mul_f16, 2 v_cvt_pk_f16_f32,
+ *           3 v_max3_f32, 4 v_and_or_b32, 5 v_pk_add_f16, 6 v_perm_b32, 7 v_mul_f32, 8 v_fma_f32
+ *   kind 3: 512 lanes; waves 0-3 of a workgroup run kind 0 with p0 = 0, waves 4-7 run p0 iterations of 32 v_fma_f32: two
+ *           waves per SIMD, one of each kind
+ *   kind 4: streaming read of iters MiB in 16-byte pieces; p0 != 0: nontemporal loads
+ * out[0] = milliseconds of the timed launch (events); out[1], out[2] = mean shader-clock cycles and mean wall-clock
+ * ticks a wave measured around its loop (kind 3: waves 0-3); out[3], out[4] the same for waves 4-7 of kind 3;
+ * out[5] = wall-clock ticks per millisecond. */
+YKA_API int yka_machine_probe(int kind, int p0, int iters, int blocks, int threads, double* out);
+
 #ifdef __cplusplus
 }
 #endif

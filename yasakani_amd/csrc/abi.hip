@@ -963,6 +963,71 @@ int yka_append_host(yka_kv* kv, int layer, const uint16_t* k16, const uint16_t* 
   YKA_CATCH_INT
 }
 
+int yka_machine_probe(int kind, int p0, int iters, int blocks, int threads, double* out) {
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  int rc = 0;
+  try {
+    if (!out || kind < 0 || kind > 4 || iters < 1 || blocks < 1 || blocks > 65536) throw std::runtime_error("bad argument");
+    if (threads != 256 && threads != 512) throw std::runtime_error("threads must be 256 or 512");
+    if (kind == 0 && (p0 < 0 || p0 > 8 || (p0 & 1))) throw std::runtime_error("kind 0: p0 = vector FMAs per MFMA, one of 0 2 4 6 8");
+    if (kind == 2 && (p0 < 0 || p0 > 8)) throw std::runtime_error("kind 2: p0 = opcode 0..8");
+    if (kind == 3 && (p0 < 1 || threads != 512)) throw std::runtime_error("kind 3: p0 = iterations of the vector waves, 512 threads");
+    if (kind == 4 && iters > 4096) throw std::runtime_error("kind 4: iters = MiB to read, at most 4096");
+    if (kind == 1) threads = 256;
+    const int waves = blocks * (threads / 64);
+    const size_t nbytes = kind == 4 ? (size_t)iters << 20 : 16;
+    DevBuf sink((size_t)blocks * 512 * 4), rec((size_t)waves * 16), src(nbytes);
+    HIPCHK(hipMemset(rec.p, 0, (size_t)waves * 16));
+    if (kind == 4) HIPCHK(hipMemset(src.p, 1, nbytes));
+    HIPCHK(hipEventCreate(&e0));
+    HIPCHK(hipEventCreate(&e1));
+    HIPCHK(hipDeviceSynchronize());
+    auto run = [&]() {
+      unsigned long long* r = rec.as<unsigned long long>();
+      switch (kind) {
+        case 0: launch_probe_mix(p0, true, sink.as<float>(), r, iters, 0, 0, blocks, threads, nullptr); break;
+        case 1: launch_probe_mfma16(sink.as<float>(), r, iters, blocks, nullptr); break;
+        case 2: if (p0 == 8) launch_probe_mix(0, false, sink.as<float>(), r, iters, 0, 0, blocks, threads, nullptr);
+                else launch_probe_valu(p0, sink.as<float>(), r, iters, blocks, threads, nullptr);
+                break;
+        case 3: launch_probe_mix(0, true, sink.as<float>(), r, iters, p0, 1, blocks, 512, nullptr); break;
+        default: launch_probe_read(p0 != 0, src.p, nbytes, sink.as<float>(), blocks, nullptr); break;
+      }
+    };
+    run();                                        // warm
+    HIPCHK(hipGetLastError());
+    HIPCHK(hipDeviceSynchronize());
+    HIPCHK(hipEventRecord(e0, nullptr));
+    run();
+    HIPCHK(hipEventRecord(e1, nullptr));
+    HIPCHK(hipEventSynchronize(e1));
+    float ms = 0.f;
+    HIPCHK(hipEventElapsedTime(&ms, e0, e1));
+    HIPCHK(hipGetLastError());
+    std::vector<unsigned long long> h((size_t)waves * 2);
+    HIPCHK(hipMemcpy(h.data(), rec.p, h.size() * 8, hipMemcpyDeviceToHost));
+    // class A: waves 0..3 of a workgroup (or all waves), class B: waves 4..7 when the workgroup is split into two roles
+    double sum[4] = {0, 0, 0, 0}; size_t cnt[2] = {0, 0};
+    const int wpb = threads / 64;
+    for (int w = 0; w < waves; ++w) {
+      const int cls = (kind == 3 && (w % wpb) >= 4) ? 1 : 0;
+      sum[2 * cls] += (double)h[2 * (size_t)w]; sum[2 * cls + 1] += (double)h[2 * (size_t)w + 1]; ++cnt[cls];
+    }
+    int wall_khz = 0;
+    int dev = 0;
+    HIPCHK(hipGetDevice(&dev));
+    HIPCHK(hipDeviceGetAttribute(&wall_khz, hipDeviceAttributeWallClockRate, dev));
+    out[0] = ms;
+    out[1] = cnt[0] ? sum[0] / cnt[0] : 0; out[2] = cnt[0] ? sum[1] / cnt[0] : 0;
+    out[3] = cnt[1] ? sum[2] / cnt[1] : 0; out[4] = cnt[1] ? sum[3] / cnt[1] : 0;
+    out[5] = wall_khz;
+  } catch (const std::exception& e) { g_err = e.what(); rc = -1; }
+  catch (...) { g_err = "unknown error"; rc = -1; }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  return rc;
+}
+
 struct yka_pass { hipGraph_t graph = nullptr; hipGraphExec_t exec = nullptr; int device = 0; };
 
 yka_pass* yka_pass_capture(yka_kv* kv, const int32_t* layers, int n, const uint16_t* d_q16, const uint16_t* d_k16,
@@ -1013,6 +1078,7 @@ int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const u
   hipEvent_t e0 = nullptr, e1 = nullptr;
   hipGraph_t graph = nullptr; hipGraphExec_t gexec = nullptr;
   int rc = 0;
+  bool capturing = false;
   try {
     on_device(kv); check_rows(kv, M);
     if (!q16 || !ms || reps < 1 || mode < 0 || mode > 2) throw std::runtime_error("bad argument");
@@ -1032,9 +1098,12 @@ int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const u
                   mode == 0 ? dk.as<uint16_t>() : nullptr, mode == 0 ? dv.as<uint16_t>() : nullptr);
       }
     };
+    for (int l = 0; l < kv->cfg.n_layers; ++l) check_tb_layer(kv, l);   // what a sweep would refuse is refused before the capture begins
     if (use_graph) {
       HIPCHK(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+      capturing = true;
       sweep();
+      capturing = false;
       HIPCHK(hipStreamEndCapture(st, &graph));
       HIPCHK(hipGraphInstantiate(&gexec, graph, nullptr, nullptr, 0));
     }
@@ -1055,6 +1124,7 @@ int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const u
     if (out16_last) HIPCHK(hipMemcpy(out16_last, dout.p, nq * 2, hipMemcpyDeviceToHost));
   } catch (const std::exception& e) { g_err = e.what(); rc = -1; }
   catch (...) { g_err = "unknown error"; rc = -1; }
+  if (capturing) { hipGraph_t g = nullptr; (void)hipStreamEndCapture(kv->stream, &g); if (g) (void)hipGraphDestroy(g); }   // leave the stream out of capture mode
   if (gexec) (void)hipGraphExecDestroy(gexec);
   if (graph) (void)hipGraphDestroy(graph);
   if (e0) (void)hipEventDestroy(e0);

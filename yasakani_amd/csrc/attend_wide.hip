@@ -105,7 +105,7 @@ __device__ __forceinline__ void wait_raw(Raw& R) {
 // the optimizer so that the select form survives to instruction selection
 __device__ __forceinline__ uint32_t nib(uint32_t w, uint32_t mask, uint32_t magic) { return (w & mask) | (magic & ~mask); }
 
-__device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw& R, uint32_t magic) {
+__device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw& R, uint32_t magic, float sc_log2) {
   const h2 c1032 = {(_Float16)1032.f, (_Float16)1032.f}, c1152 = {(_Float16)1152.f, (_Float16)1152.f};
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
@@ -118,9 +118,9 @@ __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw&
     o.w = as_u32(as_h2(nib(t, 0x00f000f0u, magic)) - c1152);
     *reinterpret_cast<uint4*>(buf + kLdsK + key * kKPitch + (4 * (p & 3) + (p >> 2)) * 16) = o;
   }
-  {                                                                  // K group scales as fp32, [group][a][h][b] for key 8a+4h+b;
-    const int key = (tid & 127) >> 2, m = tid & 3;                   // waves 2 and 3 repeat waves 0 and 1 (no divergent branch)
-    reinterpret_cast<float*>(buf + kLdsS)[m * 32 + (key >> 3) * 8 + (key & 7)] = (float)as_h2(R.ks)[0];
+  {                                                                  // K group scales as fp32, [group][a][h][b] for key 8a+4h+b,
+    const int key = (tid & 127) >> 2, m = tid & 3;                   // times log2(e)/sqrt(d): scores come out in log2 units
+    reinterpret_cast<float*>(buf + kLdsS)[m * 32 + (key >> 3) * 8 + (key & 7)] = (float)as_h2(R.ks)[0] * sc_log2;   // waves 2 and 3 repeat waves 0 and 1 (no divergent branch)
   }
   {
     const int pair = tid >> 4, dw = tid & 15;
@@ -216,7 +216,6 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
     asm volatile("" ::: "memory");             // the tile loads below are instructions the compiler does not see as loads
   }
 
-  const float sc_log2 = kLog2e / sqrtf((float)kD);
   float m_run = -1e30f, l_run = 0.f;           // m_run in log2 units, shared by the two lanes of a row
   f16v o[4];
 #pragma unroll
@@ -224,6 +223,7 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
 
+  const float sc_log2 = kLog2e / sqrtf((float)kD);
   Raw raw0{}, raw1{};                          // raw codes of the next two tiles: loads run two tiles ahead of their use
   const LaneOffs offs = lane_offs(tid, h);
   uint32_t magic = kMagic;
@@ -232,7 +232,7 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
   if (tile0 < tile1) {
     load_tile_raw(tile0, raw0);
     wait_raw<0>(raw0);
-    dequant_to_lds(lds[0], tid, raw0, magic);
+    dequant_to_lds(lds[0], tid, raw0, magic, sc_log2);
     load_tile_raw(min(tile0 + 1, tile1 - 1), raw1);
     load_tile_raw(min(tile0 + 2, tile1 - 1), raw0);
   }
@@ -267,11 +267,16 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
       pv();
     }
     wait_raw<6>(rs);                           // the six loads of the other register set stay in flight
-    dequant_to_lds(lds[cb ^ 1], tid, rs, magic);
+    dequant_to_lds(lds[cb ^ 1], tid, rs, magic, sc_log2);
     load_tile_raw(min(T + 3, tile1 - 1), rs);  // always issued (past the end: the last tile again), so that the count of loads in flight is static
     if constexpr (kCompute) {
       const int t0 = T << 5;
-      // ---- scores: per scale group two chained MFMAs (32 channels), then the fp32 sum times the group scale ----
+      // ---- scores: per scale group two chained MFMAs (32 channels), then the fp32 sum times the group scale.  The
+      //      scales in LDS carry log2(e)/sqrt(d), and the chain of fused multiply-adds starts from minus the row's
+      //      running maximum: s comes out as (score in log2 units) - m_run, the exponent of its probability.  A row
+      //      that has seen no key yet (m_run is the "no keys" marker) starts from 0. ----
+      const bool first = m_run < -1e29f;
+      const float m_sub = first ? 0.f : m_run;
       float s[16];
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
@@ -287,15 +292,16 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
           const float sh = (&sc4[r >> 2].x)[r & 3];
-          s[r] = m == 0 ? part[r] * sh : __builtin_fmaf(part[r], sh, s[r]);
+          s[r] = __builtin_fmaf(part[r], sh, m == 0 ? -m_sub : s[r]);
         }
       }
       // the V fragments are requested here and used after the barrier: their LDS latency runs under the softmax arithmetic
 #pragma unroll
       for (int c = 0; c < 8; ++c)
         vfr[c] = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsV + (32 * (c >> 1) + j) * kVPitch + (16 * (c & 1) + 8 * h) * 2));
-      // ---- online softmax with a lazily raised maximum.  s stays in raw units; the factor log2(e)/sqrt(d) is
-      //      folded into the exponent's fused multiply-add: p = 2^(s * sc_log2 - m_run) ----
+      // ---- online softmax with a lazily raised maximum: a row's offset m_run only moves when a score exceeds it by
+      //      more than 2^kRaise (or when the row sees its first keys), so the accumulators stay untouched on almost
+      //      every tile.  The row sum is taken from the fp16 probabilities the PV product uses (two per dot2). ----
       if (t0 + 32 > minlen) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -306,24 +312,31 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
       float tmax = -INFINITY;
 #pragma unroll
       for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, s[r]);
-      tmax *= sc_log2;
-      if (__any(tmax > m_run + kRaise)) {
+      if (__any(tmax > (first ? -INFINITY : kRaise))) {
         tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-        const float m_new = fmaxf(m_run, tmax);
-        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-        m_run = m_new; l_run *= alpha;
+        const bool seen = tmax > -INFINITY;                       // false: every key of the tile lies past the row's length
+        const float d = first ? (seen ? tmax : 0.f) : fmaxf(tmax, 0.f);
+        const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-d);   // a first tile finds zeros in l and o
+        if (!first || seen) m_run = m_sub + d;
+        l_run *= alpha;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
           for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
-      }
-      float lsum = 0.f;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(s[r], sc_log2, -m_run));
-        lsum += p; pf[r >> 3][r & 7] = (_Float16)p;
+        for (int r = 0; r < 16; ++r) s[r] -= d;
       }
-      l_run += lsum;
+      float lsum0 = 0.f, lsum1 = 0.f;
+      const h2 ones = {(_Float16)1.f, (_Float16)1.f};
+#pragma unroll
+      for (int r = 0; r < 16; r += 4) {
+        const h2 p01 = {(_Float16)__builtin_amdgcn_exp2f(s[r]), (_Float16)__builtin_amdgcn_exp2f(s[r + 1])};
+        const h2 p23 = {(_Float16)__builtin_amdgcn_exp2f(s[r + 2]), (_Float16)__builtin_amdgcn_exp2f(s[r + 3])};
+        lsum0 = __builtin_amdgcn_fdot2(p01, ones, lsum0, false);
+        lsum1 = __builtin_amdgcn_fdot2(p23, ones, lsum1, false);
+        pf[r >> 3][r & 7] = p01[0]; pf[r >> 3][(r & 7) + 1] = p01[1]; pf[r >> 3][(r & 7) + 2] = p23[0]; pf[r >> 3][(r & 7) + 3] = p23[1];
+      }
+      l_run += lsum0 + lsum1;
     }
     __syncthreads();
   };

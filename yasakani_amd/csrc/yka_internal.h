@@ -144,6 +144,12 @@ void launch_row256_decode(int rows, int mode, int rot, const int8_t* q8, const u
 // the step after attention for 256-channel heads: gate, signs, 512-point Hadamard transform, int8 groups of 512 (n_heads even)
 void launch_attn_out256(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads, int8_t* qx, float* alpha, hipStream_t);
 
+// machine probe (probe.hip): fixed instruction mixes that time themselves; rec gets (shader cycles, wall ticks) per wave
+void launch_probe_mix(int nv, bool mfma, float* sink, unsigned long long* rec, int iters, int iters_b, int split, int blocks, int threads, hipStream_t);
+void launch_probe_mfma16(float* sink, unsigned long long* rec, int iters, int blocks, hipStream_t);
+void launch_probe_valu(int op, float* sink, unsigned long long* rec, int iters, int blocks, int threads, hipStream_t);
+void launch_probe_read(bool nt, const void* src, size_t bytes, float* sink, int blocks, hipStream_t);
+
 // start of the (page, kv head) block that holds token t
 __device__ __forceinline__ uint8_t* kv_page(const KvView& kv, int kvh, int t) {
   const int lp = t / kPageTok;

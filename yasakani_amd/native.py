@@ -78,6 +78,7 @@ def _load():
         "yka_pass_launch": (i32, [vp, vp]),
         "yka_pass_destroy": (None, [vp]),
         "yka_attn_bench": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp, vp]),
+        "yka_machine_probe": (i32, [i32, i32, i32, i32, i32, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(lib, name)
@@ -90,7 +91,7 @@ EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "y
            "yka_attn_post_host", "yka_kv_export_rows", "yka_kv_export_rows256", "yka_kv_import_rows256",
            "yka_attn_out256", "yka_attn_out256_host", "yka_append256_f32", "yka_rotate_q256", "yka_append256_f32_host", "yka_rotate_q256_host",
            "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
-           "yka_append_host", "yka_pass_capture", "yka_pass_launch", "yka_pass_destroy", "yka_attn_bench")
+           "yka_append_host", "yka_pass_capture", "yka_pass_launch", "yka_pass_destroy", "yka_attn_bench", "yka_machine_probe")
 
 _lib = None
 
@@ -122,6 +123,17 @@ def _u16(a, shape):
 
 def build_info() -> str:
     return lib().yka_build_info().decode()
+
+
+def machine_probe(kind, p0=0, iters=1000, blocks=256, threads=256):
+    """One launch of a fixed instruction mix (see yka_machine_probe in include/yka_abi.h).  Returns a dict with the
+    event time and what the waves measured themselves: shader cycles, wall ticks, and the shader clock they imply."""
+    out = np.zeros(6, np.float64)
+    _chk(lib().yka_machine_probe(kind, p0, iters, blocks, threads, _ptr(out)))
+    r = {"ms": out[0], "cycles": out[1], "wall_ticks": out[2], "cycles_b": out[3], "wall_ticks_b": out[4], "wall_khz": out[5]}
+    if out[2] > 0 and out[5] > 0:
+        r["shader_mhz"] = out[1] / (out[2] / out[5]) / 1e3
+    return r
 
 
 def codec_probe(x16):
