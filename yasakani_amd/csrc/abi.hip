@@ -90,15 +90,15 @@ int narrow_splits(const yka_kv* kv, int M) {
   return std::min(S, (int)(kWsPairs / (size_t)M));
 }
 
-// Wide kernel geometry: a workgroup owns 128 query rows (4 waves x 32) and one split; two workgroups share a CU.
-// Splits: about two workgroups per CU; the partial sums (M * S * 24 * 264 bytes) stay below the KV stream they summarise.
+// Wide kernel geometry: a workgroup of 8 waves owns 128 query rows and one split (its two wave groups take alternate
+// tiles of the split and merge on chip), one workgroup per compute unit.  Splits: one workgroup per CU (256 of them), at
+// least four 32-key tiles (two steps of either group) per workgroup, sized like the decode grid by the expected context.
+// At 64 rows (three row blocks) that is 21 splits: 64 x 21 x 24 partial rows of 264 bytes, 8.5 MB.
 int wide_rows_per_block(int) { return 128; }
 int wide_splits(const yka_kv* kv, int M) {
   const int rows = kG * M, rpb = wide_rows_per_block(M), rb = (rows + rpb - 1) / rpb;
-  // about two workgroups per CU, and (sized like the decode grid, by the expected context) at least 2 * rb 32-key
-  // tiles per workgroup: measured best at 4k context for 16 and 64 rows, no change at 32k
   const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
-  int S = kv->opt_splits_wide > 0 ? kv->opt_splits_wide : std::min(512 / (kv->cfg.n_kv_heads * rb), ((ctx + 31) / 32) / (2 * rb));
+  int S = kv->opt_splits_wide > 0 ? kv->opt_splits_wide : std::min(256 / (kv->cfg.n_kv_heads * rb), ((ctx + 31) / 32) / 4);
   S = std::max(1, std::min(kMaxSplits, S));
   return std::min(S, std::max(1, (int)kWsPairs / M));
 }

@@ -2,27 +2,38 @@
 //
 // Same mathematics as the narrow kernel (reference: src/q35_atxpk4.cuh:71-499 for the window shape, row geometry
 // src/q35_atxpk.cu:391-411): every row t of the window runs an online softmax over the keys [0, len(t)) of its
-// split and leaves (m, l, acc) partials for the combiner.  What differs is who dequantizes:
-//   * a workgroup of 4 waves owns up to 128 query rows (token-major, 6 heads per token) and one split of the keys.
-//     Each 32-key tile is dequantized ONCE per workgroup into LDS - K as exact integer codes in fp16 (n-8, odd nibbles
+// split and leaves (m, l, acc) partials for the combiner.  What differs is who dequantizes and how the work of a
+// compute unit is laid out in time:
+//   * one workgroup of 8 waves per compute unit owns up to 128 query rows (token-major, 6 heads per token) and one
+//     split of the keys.  The waves form two groups of four; group g walks the tiles tile0 + g, tile0 + g + 2, ... of
+//     the split, each with its own softmax state, and the two states are merged through LDS at the end: one partial
+//     row per (row, split), half as many splits as workgroups of four waves would need to fill the chip;
+//   * a group dequantizes each of its 32-key tiles ONCE into LDS - K as exact integer codes in fp16 (n-8, odd nibbles
 //     16(n-8)), V scaled and transposed (channel-major, the operand shape of the token-contracting MFMA) - and every
-//     wave reads its MFMA fragments from there;
+//     wave of the group reads its MFMA fragments from there;
 //   * a wave owns one tile of 32 rows (MFMA 32x32x16: one K or V fragment read from LDS serves 32 rows) and stays
-//     under 256 registers, so two waves share a SIMD and all MFMA results live in ordinary VGPRs (no accumulator-file
-//     copies).  Matrix and vector instructions share the SIMD's issue port and overlap little on this chip: the loop
-//     runs at about the sum of its MFMA time and its vector time;
+//     under 256 registers, so the two waves of a SIMD (one of each group) fit and all MFMA results live in ordinary
+//     VGPRs (no accumulator-file copies);
+//   * a step of a group has two phases with a workgroup barrier after each: a MATRIX phase (the PV product of the
+//     previous tile, the score MFMAs of this tile with the scale multiply-adds in their shadow, fragment reads) and a
+//     VECTOR phase (softmax, dequantization of the group's next tile, requests for the tile after that).  The groups run
+//     half a step apart: while one is in its matrix phase the other is in its vector phase, so the two waves of a SIMD
+//     never compete for the matrix pipe and vector work of one wave runs under the MFMAs of the other.  Two waves
+//     left to themselves do not find this arrangement: measured, two independent 4-wave workgroups per compute unit
+//     take as long as the same two one after the other;
 //   * the group scales of K are applied to the fp32 partial sum of each 32-channel group (two chained MFMAs per
-//     group), so K is never rounded; V carries one fp16 rounding;
+//     group), so K is never rounded; V carries one fp16 rounding.  The scales in LDS carry log2(e)/sqrt(d) and the
+//     chain of multiply-adds starts from minus the row's running maximum: a score leaves it as the exponent of its
+//     probability;
 //   * the running maximum of a row is only raised when a score exceeds it by more than 2^8: accumulators stay in
 //     their registers untouched on almost every tile;
-//   * LDS is double buffered: tile n+1 is dequantized while tile n is consumed; one barrier per tile.  The PV product of
-//     a tile is issued one step later, next to that dequantization; the raw tile loads run two tiles ahead as explicit
-//     load instructions with their own counter waits;
+//   * LDS is double buffered per group; the raw tile loads run two tiles ahead as explicit load instructions with
+//     their own counter waits;
 //   * the last split owns the tiles that hold the rows this pass appends and quantizes them itself before reading
 //     them (quantize-on-append without a launch of its own).
-// The values the instruction-form loads produce must reach their wait in the registers they were loaded into: the
-// generated code is checked for copies or spills of those registers whenever this file changes (none; they are loop
-// carried in fixed registers), and every parity test would fail on one.
+// The values the instruction-form loads produce must reach their wait in the registers they were loaded into: they are
+// loop carried in fixed registers, every request is waited for before the loop's registers are given up, and every
+// parity test would fail on a copy made before its wait.
 // LDS image of one tile (19456 bytes):
 //   K  [32 keys][272 B]   chunk 4m+g of a key = channels 32m+8g..+7 in the order n0,n4,n1,n5,n2,n6,n3,n7; the 272-byte
 //                          pitch makes the lanes of a fragment read hit distinct banks
@@ -53,7 +64,8 @@ constexpr uint32_t kMagic = 0x64006400u;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kKPitch = 272, kVPitch = 80;
 constexpr int kLdsK = 0, kLdsV = 32 * kKPitch, kLdsS = kLdsV + 128 * kVPitch, kLdsBuf = kLdsS + 512;   // 19456
-constexpr int NT = 256;                        // threads per workgroup
+constexpr int NT = 512;                        // threads per workgroup: two groups of four waves
+constexpr int NTG = 256;                       // threads per group
 constexpr float kRaise = 8.f;                  // log2 slack before a running maximum is raised
 
 struct Raw {                                   // one thread's share of a raw 32-key tile
@@ -90,7 +102,7 @@ __device__ __forceinline__ uint32_t gload16(const uint8_t* base, uint32_t off) {
 __device__ __forceinline__ void load_raw(const uint8_t* pg, int tp, const LaneOffs& L, Raw& R) {
   const uint8_t* kt = pg + (uint32_t)tp * 64u;            // K and V code rows of the tile start here (+ plane offset)
   R.kw[0] = gload32<0>(kt, L.k);
-  R.kw[1] = gload32<NT * 4>(kt, L.k);
+  R.kw[1] = gload32<NTG * 4>(kt, L.k);
   R.vw[0] = gload32<0>(kt, L.v);
   R.vw[1] = gload32<64>(kt, L.v);
   R.vs = gload32<0>(pg + (uint32_t)tp * 2u, L.vs);
@@ -109,7 +121,7 @@ __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw&
   const h2 c1032 = {(_Float16)1032.f, (_Float16)1032.f}, c1152 = {(_Float16)1152.f, (_Float16)1152.f};
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
-    const int idx = tid + u * NT, key = idx >> 4, p = idx & 15;      // physical dword p = 4g+m of the key row
+    const int idx = tid + u * NTG, key = idx >> 4, p = idx & 15;      // physical dword p = 4g+m of the key row
     const uint32_t w = R.kw[u], t = w >> 8;
     uint4 o;
     o.x = as_u32(as_h2(nib(w, 0x000f000fu, magic)) - c1032);
@@ -144,11 +156,13 @@ __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw&
 
 }  // namespace
 
-// grid (S, n_kv, ceil(6M / rows_per_block)), block 256; wave w owns rows [32 w, 32 (w+1)) of the block
-__global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
-  __shared__ __align__(16) uint8_t lds[2][kLdsBuf];
+// grid (S, n_kv, ceil(6M / rows_per_block)), block 512; wave w of either group owns rows [32 w, 32 (w+1)) of the block
+__global__ void __launch_bounds__(NT) attend_wide_kernel(AttnArgs A) {
+  __shared__ __align__(16) uint8_t lds[2][2][kLdsBuf];               // [group][buffer]
   const int split = blockIdx.x, kvh = blockIdx.y, rb = blockIdx.z;
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, j = lane & 31, h = lane >> 5;
+  const int tid = threadIdx.x, gt = tid & (NTG - 1);                  // gt: thread index inside the group
+  const int grp = __builtin_amdgcn_readfirstlane(tid >> 8);           // wave uniform
+  const int wave = __builtin_amdgcn_readfirstlane(gt >> 6), lane = tid & 63, j = lane & 31, h = lane >> 5;
   const int pos = *A.d_pos;
   const int nrows = kG * A.M;
 
@@ -191,30 +205,39 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
   else if (split == A.S - 1) { tile0 = Tw; tile1 = ntiles; }
   else { const int tps = (Tw + A.S - 2) / (A.S - 1); tile0 = split * tps; tile1 = min(Tw, tile0 + tps); }
   // ---- fused quantize-on-append: every workgroup of the window split stores the slice's rows up to its own last
-  //      token (the row blocks of one kv head write identical bytes) and reads them back after a workgroup barrier:
-  //      writer and readers are waves of one CU and one write-through L1 ----
+  //      token (the row blocks of one kv head write identical bytes: each row is the same sequence of IEEE operations
+  //      on the same inputs whoever computes it) and reads them back after a workgroup barrier: writer and readers
+  //      are waves of one CU and one write-through L1.  Group 0 quantizes; the barrier is the workgroup's. ----
   if (A.k16 && split == A.S - 1) {
     // 16 lanes per 128-channel row, 16 rows (K and V of 8 tokens) per step; all loads of the slice (at most 64 tokens)
     // are requested before the first row is quantized
     static_assert(kMaxSlice <= 64, "8 steps of 16 rows cover K and V of a slice");
-    const int c = tid & 15, slot = tid >> 4;
-    uint4 rawv[8];
+    if (grp == 0) {
+      const int c = gt & 15, slot = gt >> 4;
+      uint4 rawv[8];
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      const int hh = it * 16 + slot, t = hh >> 1;
-      const uint16_t* src = ((hh & 1) ? A.v16 : A.k16) + ((size_t)(A.tok0 + t) * A.kv.n_kv + kvh) * kD + 8 * c;
-      rawv[it] = t < tok_hi ? *reinterpret_cast<const uint4*>(src) : make_uint4(0, 0, 0, 0);
-    }
+      for (int it = 0; it < 8; ++it) {
+        const int hh = it * 16 + slot, t = hh >> 1;
+        const uint16_t* src = ((hh & 1) ? A.v16 : A.k16) + ((size_t)(A.tok0 + t) * A.kv.n_kv + kvh) * kD + 8 * c;
+        rawv[it] = t < tok_hi ? *reinterpret_cast<const uint4*>(src) : make_uint4(0, 0, 0, 0);
+      }
 #pragma unroll
-    for (int it = 0; it < 8; ++it) {
-      const int hh = it * 16 + slot, t = hh >> 1, r = pos + A.tok0 + t;
-      if (t < tok_hi && r >= 0 && r < A.kv.max_ctx) quant_store_chunk8(A.kv, kvh, r, hh & 1, rawv[it], c);
+      for (int it = 0; it < 8; ++it) {
+        const int hh = it * 16 + slot, t = hh >> 1, r = pos + A.tok0 + t;
+        if (t < tok_hi && r >= 0 && r < A.kv.max_ctx) quant_store_chunk8(A.kv, kvh, r, hh & 1, rawv[it], c);
+      }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __syncthreads();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     asm volatile("" ::: "memory");             // the tile loads below are instructions the compiler does not see as loads
   }
+
+  // tiles of this group: tile0 + grp + 2u, u = 0 .. nu-1; both groups walk nsteps steps (a group one tile short idles in
+  // its last step) so that every wave of the workgroup meets the same number of barriers
+  const int ntl = max(0, tile1 - tile0);
+  const int nsteps = (ntl + 1) >> 1, nu = (ntl + 1 - grp) >> 1;
+  auto tile_of = [&](int u) __attribute__((always_inline)) { return tile0 + grp + 2 * min(u, nu - 1); };   // past the end: the last tile again
 
   float m_run = -1e30f, l_run = 0.f;           // m_run in log2 units, shared by the two lanes of a row
   f16v o[4];
@@ -224,24 +247,22 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
     for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
 
   const float sc_log2 = kLog2e / sqrtf((float)kD);
-  Raw raw0{}, raw1{};                          // raw codes of the next two tiles: loads run two tiles ahead of their use
-  const LaneOffs offs = lane_offs(tid, h);
+  Raw raw0{}, raw1{};                          // raw codes of the group's next two tiles: loads run two tiles ahead of their use
+  const LaneOffs offs = lane_offs(gt, h);
   uint32_t magic = kMagic;
   asm volatile("" : "+v"(magic));
   auto load_tile_raw = [&](int T, Raw& r) __attribute__((always_inline)) { load_raw(kv_page_uniform(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, r); };
-  if (tile0 < tile1) {
-    load_tile_raw(tile0, raw0);
+  if (nu > 0) {
+    load_tile_raw(tile_of(0), raw0);
     wait_raw<0>(raw0);
-    dequant_to_lds(lds[0], tid, raw0, magic, sc_log2);
-    load_tile_raw(min(tile0 + 1, tile1 - 1), raw1);
-    load_tile_raw(min(tile0 + 2, tile1 - 1), raw0);
+    dequant_to_lds(lds[grp][0], gt, raw0, magic, sc_log2);
+    load_tile_raw(tile_of(1), raw1);
+    load_tile_raw(tile_of(2), raw0);
   }
   __syncthreads();
 
-  // The loop is software pipelined inside the wave: the probabilities and the V fragments of a tile stay in registers
-  // across the barrier, and their eight MFMAs are issued at the start of the NEXT step, next to the dequantization of
-  // the tile after that - matrix and vector work with no dependence on each other in one basic block.  The first step
-  // multiplies zeros; the product of the last tile is issued after the loop.
+  // The probabilities and the V fragments of a tile stay in registers across the two barriers of a step; their eight
+  // MFMAs open the NEXT matrix phase.  The first one multiplies zeros; the product of the last tile follows the loop.
   h8 pf[2], vfr[8];
 #pragma unroll
   for (int c = 0; c < 8; ++c)
@@ -253,55 +274,56 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
 #pragma unroll
       for (int u = 0; u < 2; ++u) o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vfr[2 * dt + u], pf[u], o[dt], 0, 0, 0);
   };
-  // One tile: `rs` holds the raw codes of tile T+1, which are dequantized into the other LDS buffer (unconditionally:
-  // after the last tile that buffer is read by nobody) and replaced by the request for tile T+3; cb, the LDS buffer of
-  // tile T, is a literal at both call sites.  kCompute is false for a wave whose rows all lie past the window.
-  auto tile_step = [&](auto compute_tag, const int T, const int cb, Raw& rs) __attribute__((always_inline)) {
-    constexpr bool kCompute = decltype(compute_tag)::value;
-    const uint8_t* buf = lds[cb];
+  float s[16];                                 // exponents of the tile in hand: written by the matrix phase, used by the vector phase
+  float m_sub = 0.f;
+  bool first = true;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s[r] = -INFINITY;
+
+  // ---- matrix phase of the group's tile u (buffer cb of the group): PV of the tile before, scores of this one ----
+  auto matrix_phase = [&](const int u, const int cb) __attribute__((always_inline)) {
+    if (!has_rows) return;                     // wave uniform
+    const uint8_t* buf = lds[grp][cb];
     h8 kfr[8];
-    if constexpr (kCompute) {
 #pragma unroll
-      for (int c = 0; c < 8; ++c)
-        kfr[c] = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsK + j * kKPitch + (4 * (c >> 1) + 2 * (c & 1) + h) * 16));
-      pv();
-    }
-    wait_raw<6>(rs);                           // the six loads of the other register set stay in flight
-    dequant_to_lds(lds[cb ^ 1], tid, rs, magic, sc_log2);
-    load_tile_raw(min(T + 3, tile1 - 1), rs);  // always issued (past the end: the last tile again), so that the count of loads in flight is static
-    if constexpr (kCompute) {
-      const int t0 = T << 5;
-      // ---- scores: per scale group two chained MFMAs (32 channels), then the fp32 sum times the group scale.  The
-      //      scales in LDS carry log2(e)/sqrt(d), and the chain of fused multiply-adds starts from minus the row's
-      //      running maximum: s comes out as (score in log2 units) - m_run, the exponent of its probability.  A row
-      //      that has seen no key yet (m_run is the "no keys" marker) starts from 0. ----
-      const bool first = m_run < -1e29f;
-      const float m_sub = first ? 0.f : m_run;
-      float s[16];
+    for (int c = 0; c < 8; ++c)
+      kfr[c] = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsK + j * kKPitch + (4 * (c >> 1) + 2 * (c & 1) + h) * 16));
+    pv();
+    // scores: per scale group two chained MFMAs (32 channels), then the fp32 sum times the group scale.  A row that has
+    // seen no key yet (m_run is the "no keys" marker) starts its chain from 0.
+    first = m_run < -1e29f;
+    m_sub = first ? 0.f : m_run;
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        float4 sc4[4];                         // fp32 scales of group m for the lane's 16 keys, the same for all 32 lanes of a half
+    for (int m = 0; m < 4; ++m) {
+      float4 sc4[4];                           // fp32 scales of group m for the lane's 16 keys, the same for all 32 lanes of a half
 #pragma unroll
-        for (int a = 0; a < 4; ++a) sc4[a] = *reinterpret_cast<const float4*>(buf + kLdsS + ((m * 4 + a) * 2 + h) * 16);
-        f16v part;
+      for (int a = 0; a < 4; ++a) sc4[a] = *reinterpret_cast<const float4*>(buf + kLdsS + ((m * 4 + a) * 2 + h) * 16);
+      f16v part;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) part[r] = 0.f;
-        part = __builtin_amdgcn_mfma_f32_32x32x16_f16(kfr[2 * m], qf[2 * m], part, 0, 0, 0);
-        part = __builtin_amdgcn_mfma_f32_32x32x16_f16(kfr[2 * m + 1], qf[2 * m + 1], part, 0, 0, 0);
-        // part[r]: key 8(r/4) + 4h + r%4 of the tile against row j
+      for (int r = 0; r < 16; ++r) part[r] = 0.f;
+      part = __builtin_amdgcn_mfma_f32_32x32x16_f16(kfr[2 * m], qf[2 * m], part, 0, 0, 0);
+      part = __builtin_amdgcn_mfma_f32_32x32x16_f16(kfr[2 * m + 1], qf[2 * m + 1], part, 0, 0, 0);
+      // part[r]: key 8(r/4) + 4h + r%4 of the tile against row j
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float sh = (&sc4[r >> 2].x)[r & 3];
-          s[r] = __builtin_fmaf(part[r], sh, m == 0 ? -m_sub : s[r]);
-        }
+      for (int r = 0; r < 16; ++r) {
+        const float sh = (&sc4[r >> 2].x)[r & 3];
+        s[r] = __builtin_fmaf(part[r], sh, m == 0 ? -m_sub : s[r]);
       }
-      // the V fragments are requested here and used after the barrier: their LDS latency runs under the softmax arithmetic
+    }
+    // the V fragments are requested here and used in the next matrix phase: their latency runs under the vector phase
 #pragma unroll
-      for (int c = 0; c < 8; ++c)
-        vfr[c] = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsV + (32 * (c >> 1) + j) * kVPitch + (16 * (c & 1) + 8 * h) * 2));
-      // ---- online softmax with a lazily raised maximum: a row's offset m_run only moves when a score exceeds it by
-      //      more than 2^kRaise (or when the row sees its first keys), so the accumulators stay untouched on almost
-      //      every tile.  The row sum is taken from the fp16 probabilities the PV product uses (two per dot2). ----
+    for (int c = 0; c < 8; ++c)
+      vfr[c] = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsV + (32 * (c >> 1) + j) * kVPitch + (16 * (c & 1) + 8 * h) * 2));
+  };
+  // ---- vector phase of tile u: softmax of its scores; `rs` holds the raw codes of tile u+1, which are dequantized into
+  //      the group's other buffer (unconditionally: after the last tile that buffer is read by nobody) and replaced by
+  //      the request for tile u+3 ----
+  auto vector_phase = [&](const int u, const int cb, Raw& rs) __attribute__((always_inline)) {
+    if (has_rows) {
+      const int t0 = tile_of(u) << 5;
+      // online softmax with a lazily raised maximum: a row's offset m_run only moves when a score exceeds it by more
+      // than 2^kRaise (or when the row sees its first keys).  The row sum is taken from the fp16 probabilities the PV
+      // product uses (two per dot2).
       if (t0 + 32 > minlen) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -338,22 +360,67 @@ __global__ void __launch_bounds__(NT, 2) attend_wide_kernel(AttnArgs A) {
       }
       l_run += lsum0 + lsum1;
     }
+    wait_raw<6>(rs);                           // the six loads of the other register set stay in flight
+    dequant_to_lds(lds[grp][cb ^ 1], gt, rs, magic, sc_log2);
+    load_tile_raw(tile_of(u + 3), rs);         // always issued (past the end: the last tile again), so that the count of loads in flight is static
+  };
+  // Group 1 starts one barrier late and group 0 ends with one barrier more: the groups stay a phase apart, and every
+  // wave executes 2 * nsteps + 1 barriers whatever its group (a group one tile short only meets the barriers of its
+  // last step).  cb and the register set are literals at every call site.
+  if (grp == 1) __syncthreads();
+  for (int u = 0; u < nu; u += 2) {
+    matrix_phase(u, 0);
     __syncthreads();
-  };
-  auto run = [&](auto compute_tag) __attribute__((always_inline)) {
-    for (int T = tile0; T < tile1; T += 2) {
-      tile_step(compute_tag, T, 0, raw1);
-      if (T + 1 < tile1) tile_step(compute_tag, T + 1, 1, raw0);
+    vector_phase(u, 0, raw1);
+    __syncthreads();
+    if (u + 1 < nu) {
+      matrix_phase(u + 1, 1);
+      __syncthreads();
+      vector_phase(u + 1, 1, raw0);
+      __syncthreads();
     }
-  };
-  if (has_rows) { run(std::true_type{}); pv(); } else run(std::false_type{});
-  if (!has_rows) return;                       // no barrier follows
+  }
+  for (int u = nu; u < nsteps; ++u) { __syncthreads(); __syncthreads(); }
+  if (grp == 0) __syncthreads();
+  // every request has been answered before the registers it names are given up
+  wait_raw<0>(raw0);
+  wait_raw<0>(raw1);
+  if (has_rows) pv();
+
+  // ---- the two groups' states of a row are merged: group 1 leaves its registers in LDS (the tile buffers are free
+  //      after the last barrier), group 0 folds them into its own.  Wave w of either group holds the same rows in the
+  //      same registers, so the exchange is a plain register image: [wave][register][lane]. ----
+  float* xo = reinterpret_cast<float*>(&lds[0][0][0]);               // 4 waves x 64 registers x 64 lanes = 65536 bytes
+  float* xm = xo + 4 * 64 * 64;                                       // then m and l, [wave][lane]: 2048 bytes
+  float* xl = xm + 4 * 64;
+  static_assert(4 * 64 * 64 * 4 + 2 * 4 * 64 * 4 <= 4 * kLdsBuf, "the register image of group 1 fits the tile buffers");
+  if (grp == 1 && has_rows) {
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) xo[(wave * 64 + dt * 16 + r) * 64 + lane] = o[dt][r];
+    xm[wave * 64 + lane] = m_run; xl[wave * 64 + lane] = l_run;
+  }
+  __syncthreads();
+  if (grp == 1 || !has_rows) return;           // no barrier follows
+  {
+    const float mb = xm[wave * 64 + lane], lb = xl[wave * 64 + lane];
+    const float m2 = fmaxf(m_run, mb);
+    const float wa = __builtin_amdgcn_exp2f(m_run - m2), wb = __builtin_amdgcn_exp2f(mb - m2);   // both markers: 2^0, sums stay 0
+    m_run = m2; l_run = wa * l_run + wb * lb;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[dt][r] = wa * o[dt][r] + wb * xo[(wave * 64 + dt * 16 + r) * 64 + lane];
+  }
   // ---- partials: normalised fp16.  o[dt][4a+b] of lane (row j, half h) is V-image row 32dt + 8a + 4h + b, i.e.
   //      channel 64(a&1) + 32h + 8b + 4(a>>1) + dt: for each (a&1, b) the lane owns 8 consecutive channels.
-  //      Rows go through LDS (the tile buffers are free after the last barrier) so that every store instruction
-  //      writes whole 256-byte rows: 16 lanes per row instead of 64 scattered 16-byte pieces. ----
+  //      Rows go through LDS so that every store instruction writes whole 256-byte rows: 16 lanes per row instead of
+  //      64 scattered 16-byte pieces.  A wave stages its rows inside the part of the register image only it has read. ----
   constexpr int kOPitch = 2 * kD + 16;                       // bytes per staged row
-  uint8_t* stage = &lds[0][0] + wave * 32 * kOPitch;         // 4 waves x 8704 bytes
+  static_assert(32 * kOPitch <= 64 * 64 * 4, "a wave's staging area lies inside its own part of the register image");
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");     // the image has been read before the wave overwrites it
+  uint8_t* stage = &lds[0][0][0] + wave * (64 * 64 * 4);     // 4 waves x 8704 bytes, 16384 bytes apart
   float l = l_run;
   l += __shfl_xor(l, 32, 64);
   if (vrow && h == 0) { A.pm[pidx] = m_run; A.pl[pidx] = l; }
