@@ -27,9 +27,13 @@ TOKEN_BYTES = KVH * 2 * (D // 2 + 2 * (D // 32))      # 576 B per cached token p
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 # HBM bytes per launch of the dominant kernel from two `rocprofv3 --pmc` runs (FETCH_SIZE x 2.00 + WRITE_SIZE x 1.00,
-# factors from a 256 MiB copy in the same runs; see profiles/attend_*_ctx32768.md).  Keyed by (rows, ctx, containers
-# irrelevant); any other workload reports null.
-MEASURED_TRAFFIC_BYTES = {(64, 32768): 39.9e6, (1, 32768): 19.6e6}
+# factors from a 256 MiB copy in the same runs).  A cited constant, not something this run measures: each entry names
+# the summary it was taken from, and the JSON line carries that name so that a stale figure can be told from a fresh one.
+# Keyed by (rows, ctx); any other workload reports null.
+MEASURED_TRAFFIC = {
+    (64, 32768): (31.1e6, "profiles/attend_wide_kernel_verify64_ctx32768.md"),
+    (1, 32768): (19.6e6, "profiles/attend_narrow_kernel_decode_ctx32768.md"),
+}
 
 
 def algorithmic_bytes(ctx, M):
@@ -62,7 +66,10 @@ def fill_cache(kv, k, v, ctx, chunk=4096):
 
 
 def timed_passes(torch, kv, layers, q, kn, vn, ctx, M, steps, warmup):
-    """K layer calls = replays of a captured pass over all containers (+ single calls for a remainder)."""
+    """Exactly `steps` layer calls, issued the same way whatever `steps` is: replays of captured passes that walk the
+    containers in order (full sweeps over all of them, then one pass over the first steps % L).  Before the timed region
+    every container is swept once and `warmup` further calls run.  Timed with events on the stream the passes are
+    launched on; the host clock around the same region is returned beside it."""
     dev = torch.device("cuda:0")
     dq = torch.from_numpy(q.view(np.int16)).to(dev)
     dk = torch.from_numpy(kn.view(np.int16)).to(dev)
@@ -72,27 +79,37 @@ def timed_passes(torch, kv, layers, q, kn, vn, ctx, M, steps, warmup):
     torch.cuda.synchronize()
     stream = torch.cuda.current_stream().cuda_stream
     L = len(layers)
-    sweep = kv.capture_pass(layers, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), M, dpos.data_ptr(), dout.data_ptr())
-    singles = [kv.capture_pass([l], dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), M, dpos.data_ptr(), dout.data_ptr())
-               for l in layers[: steps % L]]
+
+    def capture(ls):
+        return kv.capture_pass(ls, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), M, dpos.data_ptr(), dout.data_ptr())
+
+    sweep = capture(layers)
+    passes = {L: sweep}
 
     def run(n):
         for _ in range(n // L):
             sweep.launch(stream)
-        for s in singles[: n % L]:
-            s.launch(stream)
+        if n % L:
+            if n % L not in passes:
+                passes[n % L] = capture(layers[: n % L])
+            passes[n % L].launch(stream)
 
+    run(L)                                   # every container once
     run(warmup)
+    run(steps % L)                           # captures the remainder pass outside the timed region
     torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    e0.record()
     run(steps)
+    e1.record()
     torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    host_dt = time.perf_counter() - t0
+    dt = e0.elapsed_time(e1) * 1e-3
     out = dout.cpu().numpy().view(np.float16)
-    sweep.close()
-    for s in singles:
-        s.close()
-    return dt, out
+    for p in passes.values():
+        p.close()
+    return dt, host_dt, out
 
 
 def small_decode(native, ctx=4096, L=128):
@@ -277,25 +294,65 @@ def append_vs_post(torch, native, kv, ctx, rows_list=(1, 64), calls=400):
     return out
 
 
-def cpu_baseline(kv, q, ctx, M, budget_s=12.0):
-    """The CPU oracle (threaded port of the reference's token-streaming split-KV loop) on the same quantized cache.
-    Bounded sample: whole layer calls are repeated until about `budget_s` seconds of CPU work are spent."""
+def cpu_baseline(kv, q, ctx, M, budget_s=10.0):
+    """The CPU oracle on the same quantized cache: the reference's token-streaming split-KV loop restated in C, its inner
+    loops written so that the compiler vectorises them (AVX2), parallel over (KV head x split) with OpenMP.  Bounded
+    sample: whole layer calls are repeated until about `budget_s` seconds of CPU work are spent.  Beside the headline
+    figure (all threads) the same call is timed on one thread and on the two decode configurations."""
     from oracle import yko
     threads = min(16, os.cpu_count() or 1)
     oc = yko.Cache(kv.max_ctx)
     n = ctx + M
     oc.kc[:, :n], oc.ks[:, :n], oc.vc[:, :n], oc.vs[:, :n] = kv.export_rows(0, 0, n)
-    calls, t0 = 0, time.perf_counter()
-    while True:
-        ref16 = oc.attend_f32(q, ctx, threads=threads)
-        calls += 1
-        el = time.perf_counter() - t0
-        if el > budget_s and calls >= 3:
-            break
-    per_call = el / calls
-    return {"value": algorithmic_bytes(ctx, M) / per_call / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-            "us_per_layer": per_call * 1e6,
-            "sample": f"{calls} whole layer calls (attention + combine, no append) of the same workload, {el:.1f} s"}, ref16
+
+    def sample(qq, pos, thr, budget, least=3):
+        calls, t0 = 0, time.perf_counter()
+        while True:
+            r = oc.attend_f32(qq, pos, threads=thr)
+            calls += 1
+            el = time.perf_counter() - t0
+            if el > budget and calls >= least:
+                return el / calls, calls, el, r
+
+    per_call, calls, el, ref16 = sample(q, ctx, threads, budget_s)
+    base = {"value": algorithmic_bytes(ctx, M) / per_call / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
+            "us_per_layer": per_call * 1e6, "build": "gcc -O3 -mavx2 -fopenmp (vectorised inner loops)",
+            "sample": f"{calls} whole layer calls (attention + combine, no append) of the same workload, {el:.1f} s"}
+    other = {}
+    one, c1, e1, _ = sample(q, ctx, 1, 3.0, least=1)
+    other["headline_one_thread"] = {"us_per_layer": one * 1e6, "value_GBs": algorithmic_bytes(ctx, M) / one / 1e9, "cores": 1,
+                                    "sample": f"{c1} calls, {e1:.1f} s"}
+    for name, pos in (("decode_4096", min(4096, ctx)), ("decode_32768", min(32768, ctx))):
+        for thr in (threads, 1):
+            t, c, e, _ = sample(q[:1], pos, thr, 1.0)
+            other[f"{name}_{thr}_threads"] = {"us_per_layer": t * 1e6, "value_GBs": algorithmic_bytes(pos, 1) / t / 1e9, "cores": thr,
+                                              "sample": f"{c} calls, {e:.1f} s"}
+    base["other_configs"] = other
+    return base, ref16
+
+
+def machine_figures(native):
+    """What this GPU sustains on fixed instruction mixes (yka_machine_probe): dense fp16 MFMA rate, streaming read rate,
+    and how far vector instructions hide behind MFMAs of the same wave.  The roofline stays priced at the published
+    peaks; these are the ceilings a kernel can actually reach on this box."""
+    it = 4000
+    out = {}
+    for blocks, name in ((256, "one_wave_per_simd"), (512, "two_waves_per_simd")):
+        r = native.machine_probe(0, 0, it, blocks, 256)
+        out[f"mfma_f16_32x32x16_tflops_{name}"] = blocks * 4 * it * 4 * 32768.0 / (r["ms"] * 1e-3) / 1e12
+        out[f"shader_mhz_under_mfma_{name}"] = r.get("shader_mhz")
+    r0 = native.machine_probe(0, 0, it, 256, 256)
+    r6 = native.machine_probe(0, 6, it, 256, 256)
+    out["cycles_per_mfma_alone"] = r0["cycles"] / (it * 4)
+    out["cycles_per_mfma_with_6_fma_behind_it"] = r6["cycles"] / (it * 4)
+    rf = native.machine_probe(2, 8, it, 256, 256)
+    out["cycles_per_v_fma_f32_one_wave"] = rf["cycles"] / (it * 32)
+    for nt in (0, 1):
+        r = native.machine_probe(4, nt, 2048, 16384, 256)
+        out["read_GBs_nontemporal" if nt else "read_GBs_plain"] = 2048 * 1048576 / (r["ms"] * 1e-3) / 1e9
+    out["measured_mfma_peak_tflops"] = max(v for k, v in out.items() if k.startswith("mfma_f16"))
+    out["measured_read_GBs"] = max(out["read_GBs_plain"], out["read_GBs_nontemporal"])
+    return out
 
 
 def main():
@@ -314,6 +371,7 @@ def main():
                     help="run only the passes over the reference's 256-channel rows and print their figures (for profiling those kernels)")
     ap.add_argument("--trellis-only", action="store_true",
                     help="run only the passes over trellis-coded rows (5 and 4 bits per element) and print their figures")
+    ap.add_argument("--machine", action="store_true", help="only run the machine probe (MFMA rate, read rate, overlap) and print it")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three device-to-device copies of 256 MiB (a kernel of known traffic, for scaling FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -325,6 +383,9 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py: no GPU visible")
 
+    if args.machine:
+        print(json.dumps({"machine": machine_figures(native)}))
+        return
     if args.r256_only:
         print(json.dumps({"reference_rows_head_dim_256": r256_figures(native, args.ctx)}))
         return
@@ -340,7 +401,7 @@ def main():
     kn, vn = k[ctx:], v[ctx:]
 
     def measure(rows, steps, warmup):
-        dt, out = timed_passes(torch, kv, layers, q[:rows], kn[:rows], vn[:rows], ctx, rows, steps, warmup)
+        dt, host_dt, out = timed_passes(torch, kv, layers, q[:rows], kn[:rows], vn[:rows], ctx, rows, steps, warmup)
         us = dt / steps * 1e6
         # the dominant kernel alone, hipEvents on the library's stream, replayed from a graph over all containers
         ms, _ = kv.bench(q[:rows], None, None, ctx, mode=2, use_graph=True, reps=20)
@@ -352,8 +413,9 @@ def main():
         else:
             roof = {"bound": "hbm", "achieved": by / (k_us * 1e-6) / 1e9, "peak": HBM_PEAK_GBS, "unit": "GB/s"}
         roof["frac"] = roof["achieved"] / roof["peak"]
-        roof["traffic"] = MEASURED_TRAFFIC_BYTES.get((rows, ctx))
+        roof["traffic"], roof["traffic_source"] = MEASURED_TRAFFIC.get((rows, ctx), (None, None))
         roof["kernel_us"] = k_us
+        roof["host_clock_us_per_layer"] = host_dt / steps * 1e6
         roof["hbm_frac"] = by / (k_us * 1e-6) / 1e9 / HBM_PEAK_GBS
         return us, by / (us * 1e-6) / 1e9, roof, out
 
@@ -388,7 +450,7 @@ def main():
         # is the cache-hot figure, not an HBM figure
         hot = {}
         for rows in (64, 1):
-            dt, _ = timed_passes(torch, kv, [0] * L, q[:rows], kn[:rows], vn[:rows], ctx, rows, L * 8, L)
+            dt, _, _ = timed_passes(torch, kv, [0] * L, q[:rows], kn[:rows], vn[:rows], ctx, rows, L * 8, L)
             hot[f"rows_{rows}"] = {"us_per_layer": dt / (L * 8) * 1e6}
         line["cache_hot_single_container"] = hot
         line["decode_4096"] = small_decode(native)
@@ -409,6 +471,10 @@ def main():
         torch.cuda.synchronize()
         line["calibration_copy_bytes"] = 256 << 20
     if not args.no_extra:
+        line["machine"] = machine_figures(native)
+        mf = line["machine"]
+        line["roofline"]["frac_of_measured_ceiling"] = (line["roofline"]["achieved"] / mf["measured_mfma_peak_tflops"] if line["roofline"]["bound"] == "mfma"
+                                                         else line["roofline"]["achieved"] / mf["measured_read_GBs"])
         line["other_configs"] = big_configs(native)
         line["reference_rows_head_dim_256"] = r256_figures(native)
         line["trellis_rows"] = {"bits_5": trellis_figures(native, torch=torch)}

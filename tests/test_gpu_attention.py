@@ -126,6 +126,21 @@ def test_multi_layer_containers_are_independent(native, oracle):
         assert (o2b.view(np.uint16) == o0.view(np.uint16)).all()
 
 
+@pytest.mark.parametrize("M", [65, 66])
+def test_tail_slice_of_one_or_two_rows(native, oracle, M):
+    # 64 rows on the wide kernel, then a slice of 1 or 2 rows on the decode kernel that starts at row 64 of the pass and
+    # stores its own rows
+    ctx = 700
+    kv, oc, q, kn, vn = _fill(native, oracle, 600 + M, ctx, M, max_rows=128)
+    with kv:
+        out = kv.layer_call(0, q, kn, vn, ctx)
+        oc.append(kn, vn, ctx)
+        assert_attn_close(out, oc.attend_f32(q, ctx, threads=8, want_f32=True)[1], f"{M}-row pass")
+        got = kv.export_rows(0, ctx, M)
+        for a, b in zip(got, (oc.kc, oc.ks, oc.vc, oc.vs)):
+            assert (a == b[:, ctx:ctx + M]).all()
+
+
 def test_wide_pass_is_cut_into_slices(native, oracle):
     # passes wider than 64 rows are cut into 64-row slices (src/engine35.cpp:935-947)
     ctx, M = 300, 150

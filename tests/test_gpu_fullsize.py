@@ -33,7 +33,7 @@ def _oracle_cache(oracle, kv, n, max_ctx):
     return oc
 
 
-@pytest.mark.parametrize("M", [1, 16, 64])
+@pytest.mark.parametrize("M", [1, 16, 32, 64])
 def test_config_1_2_decode_and_verify_at_32k(native, oracle, M):
     ctx = 32768
     q, k, v = _inputs(oracle, 900 + M, ctx, M)
@@ -41,13 +41,16 @@ def test_config_1_2_decode_and_verify_at_32k(native, oracle, M):
         _fill(kv, k, v, ctx)
         out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx)
         oc = _oracle_cache(oracle, kv, ctx + M, 33024)
-        # the cache the GPU built is what the oracle's quantizer gives (spot check of the first and last 2048 rows)
-        chk = oracle.Cache(2304)
-        chk.append(k[:2048], v[:2048], 0)
-        assert (chk.kc[:, :2048] == oc.kc[:, :2048]).all() and (chk.vs[:, :2048] == oc.vs[:, :2048]).all()
+        # the cache the GPU built is what the oracle's quantizer gives: all four planes of the first 2048 rows, of the last
+        # 2048 cached rows and of the rows this call appended
+        for lo, n in ((0, 2048), (ctx - 2048, 2048 + M)):
+            chk = oracle.Cache(2304)
+            chk.append(k[lo:lo + n], v[lo:lo + n], 0)
+            for plane_chk, plane_gpu in ((chk.kc, oc.kc), (chk.ks, oc.ks), (chk.vc, oc.vc), (chk.vs, oc.vs)):
+                assert (plane_chk[:, :n] == plane_gpu[:, lo:lo + n]).all()
         ref16, ref32 = oc.attend_f32(q, ctx, threads=16, want_f32=True)
         assert_attn_close(out, ref32, f"32k M={M}")
-        assert np.abs(out.astype(np.float64) - ref32).max() <= 2e-3   # at the measured size the plain absolute bar holds, unscaled
+        assert np.abs(out.astype(np.float64) - ref32).max() <= 2e-3   # at the measured size the plain absolute bar holds against the unrounded result too
 
 
 def test_config_3_prefill_chunk_2048_on_131072(native, oracle):
@@ -56,12 +59,15 @@ def test_config_3_prefill_chunk_2048_on_131072(native, oracle):
     max_ctx = ctx + M
     with native.KvCache(max_ctx=max_ctx, max_rows=2048) as kv:
         _fill(kv, k, v, ctx)
-        out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx)      # quantizes the chunk into the cache, 32 slices of 64 rows
+        out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx)      # quantizes the chunk into the cache
         oc = _oracle_cache(oracle, kv, ctx + M, max_ctx)
-        rows = [0, 1, 63, 64, 65, 511, 1024, 1500, 2046, 2047]
-        for t in rows:                                         # row t of the chunk = a single-row call at position ctx + t
-            ref32 = oc.attend_f32(q[t:t + 1], ctx + t, threads=16, want_f32=True)[1]
-            assert_attn_close(out[t:t + 1], ref32, f"prefill row {t}")
+        # every 16th row of the chunk plus the first and the last row of every 64-row group: the rows of one group are one
+        # oracle call (a window at position ctx + 64 g whose depth table names the sampled rows)
+        for g in range(M // 64):
+            sel = np.array([0, 16, 32, 48, 63], dtype=np.uint8)
+            rows = 64 * g + sel.astype(np.int64)
+            ref32 = oc.attend_f32(q[rows], ctx + 64 * g, depth=sel, threads=16, want_f32=True)[1]
+            assert_attn_close(out[rows], ref32, f"prefill rows {rows.tolist()}")
         # causality: changing the K/V of chunk row 1000 must leave rows < 1000 untouched
         k2, v2 = k[ctx:].copy(), v[ctx:].copy()
         k2[1000] = -k2[1000]; v2[1000] = -v2[1000]

@@ -1,9 +1,19 @@
 """Comparison bars for attention outputs (north star: max-abs 2e-3 and relative L2 1e-3 against the reference's
-fp32-accumulated math on the same seeded inputs).  Codes, scales and dequantized values are compared bit-exactly."""
+fp32-accumulated math on the same seeded inputs).  Codes, scales and dequantized values are compared bit-exactly.
+
+Outputs are fp16, as the reference's are (it rounds its fp32 result once, src/attention_kv4q.cu:325-332), so the
+absolute bar is taken against the oracle's fp32 result rounded to fp16: what the reference itself would emit.
+  * wherever |ref| <= PLAIN_UP_TO the bar is the plain one: |out - ref16| <= 2e-3;
+  * above that the fp16 grid alone is coarser than the bar (spacing 2^-8 = 3.9e-3 from 4 upward), which only very
+    short contexts reach (a row dominated by one V row): there the bar is 2e-3 * |ref| - the "scaled" bar, counted and
+    reported separately;
+  * relative L2 is always taken against the unrounded fp32 result.
+"""
 import numpy as np
 
 MAX_ABS = 2e-3
 REL_L2 = 1e-3
+PLAIN_UP_TO = 4.0
 
 
 def attn_errors(out, ref):
@@ -12,13 +22,24 @@ def attn_errors(out, ref):
     return float(np.abs(a - b).max()), float(np.linalg.norm(a - b) / np.linalg.norm(b))
 
 
-def assert_attn_close(out, ref, what=""):
-    """max-abs is taken at unit scale: |out - ref| <= 2e-3 * max(1, |ref|).  Outputs are fp16; above |x| = 4 the spacing of
-    fp16 (2^-8) alone exceeds 2e-3, which only happens at very short contexts where a row is dominated by one V row.
-    At the measured configurations (thousands of keys) every |ref| is far below 1 and this is the plain bar."""
+def attn_report(out, ref):
+    """(plain max-abs over |ref| <= 4 against ref16, scaled max-abs over the rest, rel-L2 against ref, elements above 4)."""
     a = np.asarray(out, np.float64)
     b = np.asarray(ref, np.float64)
-    ma = float((np.abs(a - b) / np.maximum(1.0, np.abs(b))).max())
-    rl = float(np.linalg.norm(a - b) / np.linalg.norm(b))
-    assert ma <= MAX_ABS and rl <= REL_L2, f"{what}: max-abs {ma:.3e} (bar {MAX_ABS}), rel-L2 {rl:.3e} (bar {REL_L2})"
-    return ma, rl
+    with np.errstate(over="ignore"):
+        b16 = np.asarray(ref, np.float32).astype(np.float16).astype(np.float64)
+    d = np.abs(a - b16)
+    small = np.abs(b) <= PLAIN_UP_TO
+    plain = float(d[small].max()) if small.any() else 0.0
+    scaled = float((d[~small] / np.abs(b[~small])).max()) if (~small).any() else 0.0
+    nb = float(np.linalg.norm(b))
+    rl = float(np.linalg.norm(a - b) / nb) if nb > 0 else float(np.abs(a).max())
+    return plain, scaled, rl, int((~small).sum())
+
+
+def assert_attn_close(out, ref, what=""):
+    plain, scaled, rl, n_big = attn_report(out, ref)
+    assert plain <= MAX_ABS and scaled <= MAX_ABS and rl <= REL_L2, (
+        f"{what}: max-abs {plain:.3e} (plain bar {MAX_ABS}, |ref| <= {PLAIN_UP_TO}), scaled max-abs {scaled:.3e} over {n_big} "
+        f"elements above that, rel-L2 {rl:.3e} (bar {REL_L2})")
+    return max(plain, scaled), rl

@@ -8,22 +8,23 @@
 //     split of the keys.  The waves form two groups of four; group g walks the tiles tile0 + g, tile0 + g + 2, ... of
 //     the split, each with its own softmax state, and the two states are merged through LDS at the end: one partial
 //     row per (row, split), half as many splits as workgroups of four waves would need to fill the chip;
-//   * a group dequantizes each of its 32-key tiles ONCE into LDS, and every wave of the group reads its MFMA fragments
-//     from there.  K goes there WITH its group scales, exactly: the fp16 scale s is cut into hi (its upper 8 significant
-//     bits) and lo = s - hi (3 bits); code * hi and code * lo (|code| <= 7) are both exact in fp16, and the MFMA adds the
-//     two products in fp32.  The scores come out of 16 chained MFMAs with no vector instruction at all.  (Rounding
-//     code * s to ONE fp16 costs 1e-3 relative L2 on inputs with outlier channels, the whole budget; applying the
-//     scales to per-group partial sums costs 64 multiply-adds and 16 LDS reads per row tile on the vector pipe.)  V is
-//     scaled in fp16 (one rounding) and transposed (channel-major, the operand shape of the token-contracting MFMA);
+//   * a group dequantizes each of its 32-key tiles ONCE into LDS - K as exact integer codes in fp16 (n-8, odd nibbles
+//     16(n-8)), V scaled and transposed (channel-major, the operand shape of the token-contracting MFMA) - and every
+//     wave of the group reads its MFMA fragments from there;
 //   * a wave owns one tile of 32 rows (MFMA 32x32x16: one K or V fragment read from LDS serves 32 rows) and stays
 //     under 256 registers, so the two waves of a SIMD (one of each group) fit and all MFMA results live in ordinary
 //     VGPRs (no accumulator-file copies);
-//   * a step of a group has two phases with a workgroup barrier after each: a MATRIX phase (24 MFMAs - the PV product
-//     of the previous tile and the scores of this one - and their fragment reads, no vector arithmetic) and a VECTOR
-//     phase (softmax, dequantization of the group's next tile, requests for the tile after that, no MFMA).  The groups
-//     run half a step apart: while one is in its matrix phase the other is in its vector phase, so the two waves of a
-//     SIMD use different pipes at any time.  Two waves left to themselves do not find this arrangement: measured, two
-//     independent 4-wave workgroups per compute unit take as long as the same two one after the other;
+//   * a step of a group has two phases with a workgroup barrier after each: a MATRIX phase (the PV product of the
+//     previous tile, the score MFMAs of this tile with the scale multiply-adds in their shadow, fragment reads) and a
+//     VECTOR phase (softmax, dequantization of the group's next tile, requests for the tile after that).  The groups run
+//     half a step apart: while one is in its matrix phase the other is in its vector phase, so the two waves of a SIMD
+//     never compete for the matrix pipe and vector work of one wave runs under the MFMAs of the other.  Two waves
+//     left to themselves do not find this arrangement: measured, two independent 4-wave workgroups per compute unit
+//     take as long as the same two one after the other;
+//   * the group scales of K are applied to the fp32 partial sum of each 32-channel group (two chained MFMAs per
+//     group), so K is never rounded; V carries one fp16 rounding.  The scales in LDS carry log2(e)/sqrt(d) and the
+//     chain of multiply-adds starts from minus the row's running maximum: a score leaves it as the exponent of its
+//     probability;
 //   * the running maximum of a row is only raised when a score exceeds it by more than 2^8: accumulators stay in
 //     their registers untouched on almost every tile;
 //   * LDS is double buffered per group; the raw tile loads run two tiles ahead as explicit load instructions with
@@ -33,14 +34,16 @@
 // The values the instruction-form loads produce must reach their wait in the registers they were loaded into: they are
 // loop carried in fixed registers, every request is waited for before the loop's registers are given up, and every
 // parity test would fail on a copy made before its wait.
-// LDS image of one tile (27648 bytes):
-//   Khi [32 keys][272 B]  chunk 4m+g of a key = channels 32m+8g..+7 in the order n0,n4,n1,n5,n2,n6,n3,n7, each code times
-//   Klo [32 keys][272 B]  hi (lo) of the scale of group m; the 272-byte pitch makes the lanes of a fragment read hit
-//                          distinct banks
-//   V   [128 rows][80 B]  channel 8*dw+c lives in row 16*sigma(c)+dw, sigma(c) = 2*(c&3) + (c>>2): the 16 lanes that
+// LDS image of one tile (19456 bytes):
+//   K  [32 keys][272 B]   chunk 4m+g of a key = channels 32m+8g..+7 in the order n0,n4,n1,n5,n2,n6,n3,n7; the 272-byte
+//                          pitch makes the lanes of a fragment read hit distinct banks
+//   V  [128 rows][80 B]   channel 8*dw+c lives in row 16*sigma(c)+dw, sigma(c) = 2*(c&3) + (c>>2): the 16 lanes that
 //                          dequantize one byte position write 16 consecutive rows, and an output lane ends up with runs
 //                          of 8 consecutive channels.  Inside a row token 16u+8a+4h+b sits at position 16u+8h+4a+b, so
 //                          the 8 tokens an MFMA lane needs are 16 contiguous bytes
+//   S  [4 groups][4 a][2 h][4 b] fp32   K group scale of key 8a+4h+b: every lane needs the scales of 16 keys x 4 groups,
+//                          the same for all 32 lanes of a wave half; converted to fp32 once per workgroup, each lane reads
+//                          four of them per instruction (a broadcast read) and multiplies with a plain fp32 FMA
 // Partial results leave through the same LDS after the last tile so that every store writes whole 256-byte rows.
 #include "codec_device.h"
 #include <hip/hip_fp16.h>
@@ -60,30 +63,30 @@ __device__ __forceinline__ uint32_t as_u32(h2 h) { return __builtin_bit_cast(uin
 constexpr uint32_t kMagic = 0x64006400u;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr int kKPitch = 272, kVPitch = 80;
-constexpr int kLdsKhi = 0, kLdsKlo = 32 * kKPitch, kLdsV = 2 * 32 * kKPitch, kLdsBuf = kLdsV + 128 * kVPitch;   // 27648
+constexpr int kLdsK = 0, kLdsV = 32 * kKPitch, kLdsS = kLdsV + 128 * kVPitch, kLdsBuf = kLdsS + 512;   // 19456
 constexpr int NT = 512;                        // threads per workgroup: two groups of four waves
 constexpr int NTG = 256;                       // threads per group
 constexpr float kRaise = 8.f;                  // log2 slack before a running maximum is raised
 
 struct Raw {                                   // one thread's share of a raw 32-key tile
-  uint32_t kw[2];                              // K code dwords tid and tid + 256 of the tile (key idx / 16, physical dword idx % 16)
-  uint32_t ks[2];                              // fp16 scale of that key and of the dword's group (idx % 4)
+  uint32_t kw[2];
   uint32_t vw[2];
   uint32_t vs;
+  uint32_t ks;                                 // fp16 scale of (key (tid & 127) / 4, group tid % 4)
 };
-constexpr int kRawLoads = 7;
 
 // Byte offsets of one thread inside a page, fixed for the whole kernel; the page pointer and the tile's first token
 // are wave uniform, so every load is "scalar base + 32-bit lane offset".
 struct LaneOffs { uint32_t k, v, vs, ks; };
-__device__ __forceinline__ LaneOffs lane_offs(int tid) {
+__device__ __forceinline__ LaneOffs lane_offs(int tid, int h) {
   const uint32_t pair = tid >> 4, dw = tid & 15;
+  (void)h;
   return LaneOffs{(uint32_t)tid * 4u, kPageVc + pair * 128u + dw * 4u, kPageVs + (dw >> 2) * (kPageTok * 2u) + pair * 4u,
-                  kPageKs + pair * 8u + ((uint32_t)tid & 3u) * 2u};
+                  kPageKs + ((uint32_t)tid & 127u) * 2u};
 }
 // The tile loads are written as instructions: they stay in flight across two loop steps, and the counter wait the
 // compiler would place at the loop header (it merges the header's predecessors conservatively) drains all of them.
-// Every load here is "wave-uniform base in scalar registers + 32-bit lane offset"; wait_raw<N> ties the registers
+// Every load here is "wave-uniform base in scalar registers + 32-bit lane offset"; wait_raw<N> ties the six registers
 // of a tile to a wait that leaves the N younger loads in flight.  Loads return in order and nothing stores in the loop.
 template <int IMM>
 __device__ __forceinline__ uint32_t gload32(const uint8_t* base, uint32_t off) {
@@ -91,55 +94,51 @@ __device__ __forceinline__ uint32_t gload32(const uint8_t* base, uint32_t off) {
   asm volatile("global_load_dword %0, %1, %2 offset:%3" : "=v"(v) : "v"(off), "s"(base), "n"(IMM));
   return v;
 }
-template <int IMM>
 __device__ __forceinline__ uint32_t gload16(const uint8_t* base, uint32_t off) {
   uint32_t v;
-  asm volatile("global_load_ushort %0, %1, %2 offset:%3" : "=v"(v) : "v"(off), "s"(base), "n"(IMM));
+  asm volatile("global_load_ushort %0, %1, %2" : "=v"(v) : "v"(off), "s"(base));
   return v;
 }
 __device__ __forceinline__ void load_raw(const uint8_t* pg, int tp, const LaneOffs& L, Raw& R) {
   const uint8_t* kt = pg + (uint32_t)tp * 64u;            // K and V code rows of the tile start here (+ plane offset)
-  const uint8_t* st = pg + (uint32_t)tp * 8u;             // K scale rows of the tile
   R.kw[0] = gload32<0>(kt, L.k);
   R.kw[1] = gload32<NTG * 4>(kt, L.k);
-  R.ks[0] = gload16<0>(st, L.ks);
-  R.ks[1] = gload16<128>(st, L.ks);                       // 16 keys further
   R.vw[0] = gload32<0>(kt, L.v);
   R.vw[1] = gload32<64>(kt, L.v);
   R.vs = gload32<0>(pg + (uint32_t)tp * 2u, L.vs);
+  R.ks = gload16(pg + (uint32_t)tp * 8u, L.ks);
 }
 template <int N>
 __device__ __forceinline__ void wait_raw(Raw& R) {
-  asm volatile("s_waitcnt vmcnt(%7)" : "+v"(R.kw[0]), "+v"(R.kw[1]), "+v"(R.ks[0]), "+v"(R.ks[1]), "+v"(R.vw[0]), "+v"(R.vw[1]), "+v"(R.vs) : "n"(N));
+  asm volatile("s_waitcnt vmcnt(%6)" : "+v"(R.kw[0]), "+v"(R.kw[1]), "+v"(R.vw[0]), "+v"(R.vw[1]), "+v"(R.vs), "+v"(R.ks) : "n"(N));
 }
 
 // (w & mask) | magic as one bit-field insert: `magic` (0x64006400, no bit inside either nibble mask) is kept opaque to
 // the optimizer so that the select form survives to instruction selection
 __device__ __forceinline__ uint32_t nib(uint32_t w, uint32_t mask, uint32_t magic) { return (w & mask) | (magic & ~mask); }
 
-__device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw& R, uint32_t magic) {
+__device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw& R, uint32_t magic, float sc_log2) {
   const h2 c1032 = {(_Float16)1032.f, (_Float16)1032.f}, c1152 = {(_Float16)1152.f, (_Float16)1152.f};
-  const h2 sixteenth = {(_Float16)0.0625f, (_Float16)0.0625f};
 #pragma unroll
   for (int u = 0; u < 2; ++u) {
     const int idx = tid + u * NTG, key = idx >> 4, p = idx & 15;      // physical dword p = 4g+m of the key row
     const uint32_t w = R.kw[u], t = w >> 8;
-    // the scale in both halves; hi = its upper 8 significant bits, lo = the rest: code * hi and code * lo are exact.
-    // Odd nibbles come out as 16 (n - 8) and take a sixteenth of the scale (exact unless the scale is below 2^-13).
-    const uint32_t s2b = __builtin_amdgcn_perm(0u, R.ks[u], 0x01000100u);
-    const h2 hi = as_h2(s2b & 0xfff8fff8u), lo = as_h2(s2b) - hi;
-    const h2 hiq = hi * sixteenth, loq = lo * sixteenth;
-    const h2 e0 = as_h2(nib(w, 0x000f000fu, magic)) - c1032, e1 = as_h2(nib(w, 0x00f000f0u, magic)) - c1152;
-    const h2 e2 = as_h2(nib(t, 0x000f000fu, magic)) - c1032, e3 = as_h2(nib(t, 0x00f000f0u, magic)) - c1152;
-    const int at = key * kKPitch + (4 * (p & 3) + (p >> 2)) * 16;
-    *reinterpret_cast<uint4*>(buf + kLdsKhi + at) = make_uint4(as_u32(e0 * hi), as_u32(e1 * hiq), as_u32(e2 * hi), as_u32(e3 * hiq));
-    *reinterpret_cast<uint4*>(buf + kLdsKlo + at) = make_uint4(as_u32(e0 * lo), as_u32(e1 * loq), as_u32(e2 * lo), as_u32(e3 * loq));
+    uint4 o;
+    o.x = as_u32(as_h2(nib(w, 0x000f000fu, magic)) - c1032);
+    o.y = as_u32(as_h2(nib(w, 0x00f000f0u, magic)) - c1152);
+    o.z = as_u32(as_h2(nib(t, 0x000f000fu, magic)) - c1032);
+    o.w = as_u32(as_h2(nib(t, 0x00f000f0u, magic)) - c1152);
+    *reinterpret_cast<uint4*>(buf + kLdsK + key * kKPitch + (4 * (p & 3) + (p >> 2)) * 16) = o;
+  }
+  {                                                                  // K group scales as fp32, [group][a][h][b] for key 8a+4h+b,
+    const int key = (tid & 127) >> 2, m = tid & 3;                   // times log2(e)/sqrt(d): scores come out in log2 units
+    reinterpret_cast<float*>(buf + kLdsS)[m * 32 + (key >> 3) * 8 + (key & 7)] = (float)as_h2(R.ks)[0] * sc_log2;   // waves 2 and 3 repeat waves 0 and 1 (no divergent branch)
   }
   {
     const int pair = tid >> 4, dw = tid & 15;
     const int t0 = 2 * pair;                                         // token 16u + 8a + 4h + b -> position 16u + 8h + 4a + b
     const int posn = (t0 & 16) + 8 * ((t0 >> 2) & 1) + 4 * ((t0 >> 3) & 1) + (t0 & 3);
-    const h2 s2 = as_h2(R.vs), s2q = s2 * sixteenth;
+    const h2 s2 = as_h2(R.vs), s2q = s2 * h2{(_Float16)0.0625f, (_Float16)0.0625f};
     const uint32_t w0 = R.vw[0], w1 = R.vw[1];
     uint8_t* vb = buf + kLdsV + dw * kVPitch + posn * 2;
 #pragma unroll
@@ -180,11 +179,12 @@ __global__ void __launch_bounds__(NT) attend_wide_kernel(AttnArgs A) {
   h8 qf[8];
   {
     const uint16_t* qrow = A.q16 + ((size_t)tl * A.n_heads + head) * kD;
+    const _Float16 sx = (_Float16)0.0625f;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       uint4 u = vrow ? *reinterpret_cast<const uint4*>(qrow + 32 * (ks >> 1) + 8 * (2 * (ks & 1) + h)) : make_uint4(0, 0, 0, 0);
       const h8 c = __builtin_bit_cast(h8, u);
-      qf[ks] = h8{c[0], c[4], c[1], c[5], c[2], c[6], c[3], c[7]};
+      qf[ks] = h8{c[0], c[4], c[1] * sx, c[5] * sx, c[2], c[6], c[3] * sx, c[7] * sx};
     }
   }
   const bool has_rows = row0 < min(nrows, (rb + 1) * RPB);             // wave uniform
@@ -248,14 +248,14 @@ __global__ void __launch_bounds__(NT) attend_wide_kernel(AttnArgs A) {
 
   const float sc_log2 = kLog2e / sqrtf((float)kD);
   Raw raw0{}, raw1{};                          // raw codes of the group's next two tiles: loads run two tiles ahead of their use
-  const LaneOffs offs = lane_offs(gt);
+  const LaneOffs offs = lane_offs(gt, h);
   uint32_t magic = kMagic;
   asm volatile("" : "+v"(magic));
   auto load_tile_raw = [&](int T, Raw& r) __attribute__((always_inline)) { load_raw(kv_page_uniform(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, r); };
   if (nu > 0) {
     load_tile_raw(tile_of(0), raw0);
     wait_raw<0>(raw0);
-    dequant_to_lds(lds[grp][0], gt, raw0, magic);
+    dequant_to_lds(lds[grp][0], gt, raw0, magic, sc_log2);
     load_tile_raw(tile_of(1), raw1);
     load_tile_raw(tile_of(2), raw0);
   }
@@ -280,29 +280,36 @@ __global__ void __launch_bounds__(NT) attend_wide_kernel(AttnArgs A) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) s[r] = -INFINITY;
 
-  // ---- matrix phase of the group's tile u (buffer cb of the group): PV of the tile before, scores of this one.  Nothing
-  //      but MFMAs and fragment reads: the vector pipe of the SIMD belongs to the other group's wave.  The 16 score MFMAs
-  //      (8 k-steps of the hi image, 8 of the lo image) form one chain; the 8 independent PV MFMAs are issued between
-  //      them, so that no MFMA waits for the one issued just before it. ----
+  // ---- matrix phase of the group's tile u (buffer cb of the group): PV of the tile before, scores of this one ----
   auto matrix_phase = [&](const int u, const int cb) __attribute__((always_inline)) {
     if (!has_rows) return;                     // wave uniform
     const uint8_t* buf = lds[grp][cb];
-    h8 kfr[16];
+    h8 kfr[8];
 #pragma unroll
-    for (int f = 0; f < 16; ++f) {
-      const int c = f & 7;
-      kfr[f] = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + (f < 8 ? kLdsKhi : kLdsKlo) + j * kKPitch + (4 * (c >> 1) + 2 * (c & 1) + h) * 16));
+    for (int c = 0; c < 8; ++c)
+      kfr[c] = __builtin_bit_cast(h8, *reinterpret_cast<const uint4*>(buf + kLdsK + j * kKPitch + (4 * (c >> 1) + 2 * (c & 1) + h) * 16));
+    pv();
+    // scores: per scale group two chained MFMAs (32 channels), then the fp32 sum times the group scale.  A row that has
+    // seen no key yet (m_run is the "no keys" marker) starts its chain from 0.
+    first = m_run < -1e29f;
+    m_sub = first ? 0.f : m_run;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      float4 sc4[4];                           // fp32 scales of group m for the lane's 16 keys, the same for all 32 lanes of a half
+#pragma unroll
+      for (int a = 0; a < 4; ++a) sc4[a] = *reinterpret_cast<const float4*>(buf + kLdsS + ((m * 4 + a) * 2 + h) * 16);
+      f16v part;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) part[r] = 0.f;
+      part = __builtin_amdgcn_mfma_f32_32x32x16_f16(kfr[2 * m], qf[2 * m], part, 0, 0, 0);
+      part = __builtin_amdgcn_mfma_f32_32x32x16_f16(kfr[2 * m + 1], qf[2 * m + 1], part, 0, 0, 0);
+      // part[r]: key 8(r/4) + 4h + r%4 of the tile against row j
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float sh = (&sc4[r >> 2].x)[r & 3];
+        s[r] = __builtin_fmaf(part[r], sh, m == 0 ? -m_sub : s[r]);
+      }
     }
-    f16v acc;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-#pragma unroll
-    for (int f = 0; f < 16; ++f) {
-      acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(kfr[f], qf[f & 7], acc, 0, 0, 0);
-      if (f & 1) { const int k = f >> 1; o[k >> 1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vfr[2 * (k >> 1) + (k & 1)], pf[k & 1], o[k >> 1], 0, 0, 0); }
-    }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) s[r] = acc[r];
     // the V fragments are requested here and used in the next matrix phase: their latency runs under the vector phase
 #pragma unroll
     for (int c = 0; c < 8; ++c)
@@ -315,13 +322,8 @@ __global__ void __launch_bounds__(NT) attend_wide_kernel(AttnArgs A) {
     if (has_rows) {
       const int t0 = tile_of(u) << 5;
       // online softmax with a lazily raised maximum: a row's offset m_run only moves when a score exceeds it by more
-      // than 2^kRaise (or when the row sees its first keys).  s arrives in raw units; its exponent is
-      // s * log2(e)/sqrt(d) - m_run, and a row that has seen no key yet (m_run is the "no keys" marker) starts from 0.
-      // The row sum is taken from the fp16 probabilities the PV product uses (two per dot2).
-      first = m_run < -1e29f;
-      m_sub = first ? 0.f : m_run;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) s[r] = __builtin_fmaf(s[r], sc_log2, -m_sub);
+      // than 2^kRaise (or when the row sees its first keys).  The row sum is taken from the fp16 probabilities the PV
+      // product uses (two per dot2).
       if (t0 + 32 > minlen) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -358,8 +360,8 @@ __global__ void __launch_bounds__(NT) attend_wide_kernel(AttnArgs A) {
       }
       l_run += lsum0 + lsum1;
     }
-    wait_raw<kRawLoads>(rs);                   // the loads of the other register set stay in flight
-    dequant_to_lds(lds[grp][cb ^ 1], gt, rs, magic);
+    wait_raw<6>(rs);                           // the six loads of the other register set stay in flight
+    dequant_to_lds(lds[grp][cb ^ 1], gt, rs, magic, sc_log2);
     load_tile_raw(tile_of(u + 3), rs);         // always issued (past the end: the last tile again), so that the count of loads in flight is static
   };
   // Group 1 starts one barrier late and group 0 ends with one barrier more: the groups stay a phase apart, and every

@@ -77,18 +77,17 @@ __global__ void __launch_bounds__(512) mix_kernel(float* sink, unsigned long lon
 
 __global__ void __launch_bounds__(256) mfma16_kernel(float* sink, unsigned long long* rec, int iters) {
   const int wave_id = blockIdx.x * 4 + (threadIdx.x >> 6);
-  f4 a[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) a[i] = f4{0.f, 0.f, 0.f, 0.f};
+  f4 b0{}, b1{}, b2{}, b3{}, b4{}, b5{}, b6{}, b7{};
   const h8 fa = {1, 1, 1, 1, 1, 1, 1, 1}, fb = {1, 1, 1, 1, 1, 1, 1, 1};
   const WaveClock t = tick();
+#define YKA_MF16(n) "v_mfma_f32_16x16x32_f16 %" #n ", %8, %9, %" #n "\n\t"
   for (int it = 0; it < iters; ++it)
-#pragma unroll
-    for (int i = 0; i < 8; ++i) a[i] = __builtin_amdgcn_mfma_f32_16x16x32_f16(fa, fb, a[i], 0, 0, 0);
+    asm volatile(YKA_MF16(0) YKA_MF16(1) YKA_MF16(2) YKA_MF16(3) YKA_MF16(4) YKA_MF16(5) YKA_MF16(6) YKA_MF16(7)
+                 : "+v"(b0), "+v"(b1), "+v"(b2), "+v"(b3), "+v"(b4), "+v"(b5), "+v"(b6), "+v"(b7) : "v"(fa), "v"(fb));
+#undef YKA_MF16
+  asm volatile("s_nop 15\n\ts_nop 15" : "+v"(b0), "+v"(b1), "+v"(b2), "+v"(b3), "+v"(b4), "+v"(b5), "+v"(b6), "+v"(b7));
   tock(t, rec, wave_id);
-  float s = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) s += a[i][i & 3];
+  const float s = b0[0] + b1[1] + b2[2] + b3[3] + b4[0] + b5[1] + b6[2] + b7[3];
   if (s == 12345.678f) sink[wave_id] = s;
 }
 
