@@ -100,6 +100,20 @@ YKA_API int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, cons
                               const uint16_t* d_v16, int M, const int* d_pos, const uint8_t* d_depth,
                               uint16_t* d_out16, void* hip_stream);
 
+/* The same layer call for callers that cannot allocate and must not depend on memory the handle allocated for its split
+ * partials (code under graph capture that is handed a foreign handle, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference.  Same inputs, outputs and results as yka_append_attend - the same kernels
+ * and split counts, bit for bit - but the split partials live in a static array inside the library's device code
+ * (9,732,096 bytes, held by every GPU the library is used on until the process ends) whose device address is looked up
+ * once per device when a handle is opened there.  Limits: head_dim 128 handles, 1 <= M <= 64 rows (one slice), at most
+ * 24 query heads; anything else returns -1 with a message.  The call allocates nothing, frees nothing, synchronises
+ * nothing.  Every call on one GPU uses that GPU's one array: calls that overlap on a GPU (two streams, two handles) race
+ * on it; calls on one stream, or otherwise ordered, are safe.  Nothing in the array has to start at zero: every launch
+ * writes every partial it later reads. */
+YKA_API int yka_append_attend_static(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16_t* d_k16,
+                                     const uint16_t* d_v16, int M, const int* d_pos, const uint8_t* d_depth,
+                                     uint16_t* d_out16, void* hip_stream);
+
 /* Multi-stream pass (batched decode): row t of the pass belongs to the stream whose KV container is d_row_slot[t]
  * (a container index in [0, n_layers): the handle's containers are then one per stream of the layer being run) and sits
  * at position d_row_pos[t] of it.  If d_k16 / d_v16 are given, row t of them is quantized into that row first; then row

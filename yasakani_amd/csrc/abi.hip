@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <stdexcept>
 #include <string>
 #include <vector>
@@ -55,7 +56,33 @@ struct yka_kv {
   }
 };
 
+// Workspace of the allocation-free entry point: the split partials of one slice, in device memory the library's code
+// object carries itself (every GPU that loads the library holds its own copy until the process ends).  The name is a
+// host-side stand-in, not a device address: the address of a device's copy is looked up once per device with that
+// device current, and only that address is ever handed to a kernel.
+constexpr size_t kStaticPairs = 1536;                              // (token, split) pairs: 64 rows x 21 splits, or 16 rows x 64, ...
+constexpr size_t kStaticHeads = 24;                                // query heads the array is sized for
+constexpr size_t kStaticPmBytes = kStaticPairs * kStaticHeads * 4;  // a multiple of 256
+constexpr size_t kStaticWsBytes = 2 * kStaticPmBytes + kStaticPairs * kStaticHeads * kD * 2;   // 9,732,096 bytes
+static __device__ __align__(256) unsigned char scratch[kStaticWsBytes];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_static_mu;
+unsigned char* g_static_ptr[kMaxDevices] = {};                      // device address of `scratch` on each device, once looked up
+// must be called with `device` current
+unsigned char* static_workspace(int device) {
+  if (device < 0 || device >= kMaxDevices) throw std::runtime_error("device ordinal beyond the static workspace table");
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  if (!g_static_ptr[device]) {
+    void* p = nullptr;
+    HIPCHK(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) throw std::runtime_error("hipGetSymbolAddress returned no address for the static workspace");
+    g_static_ptr[device] = static_cast<unsigned char*>(p);
+  }
+  return g_static_ptr[device];
+}
 
 struct DevBuf {  // device buffer that frees itself (hooks only; the launch path never allocates)
   void* p = nullptr;
@@ -77,8 +104,8 @@ constexpr size_t kWsPairs = 4096;  // (token, split) pairs the partial workspace
 // splits for the narrow kernel: one workgroup per CU (256 of them) while a workgroup then walks at most 48 tiles - its
 // waves keep the next tile in flight, and half as many partial rows make the combiner cheaper (measured: 12.2 against
 // 13.1 us per layer call at 32k, 16.0 / 16.9 at 65k) - and two per CU beyond that (35.4 against 41.8 us at 262k)
-int narrow_splits(const yka_kv* kv, int M) {
-  if (kv->opt_splits_narrow > 0) return std::min(kv->opt_splits_narrow, (int)(kWsPairs / (size_t)M));
+int narrow_splits(const yka_kv* kv, int M, size_t ws_pairs = kWsPairs) {
+  if (kv->opt_splits_narrow > 0) return std::min(kv->opt_splits_narrow, (int)(ws_pairs / (size_t)M));
   const int tiles = (M + 1) / 2;
   // launching a split costs more than letting it exit: the grid is sized for the context the caller expects (option
   // key 5; by default the capacity of the handle), two 32-key tiles per workgroup at least
@@ -87,7 +114,7 @@ int narrow_splits(const yka_kv* kv, int M) {
   const int wgs = ctx_tiles > 48 * 64 ? 512 : 256;
   int S = std::min(wgs / (kv->cfg.n_kv_heads * tiles), ctx_tiles / 2);
   S = std::max(2, std::min(kMaxSplits, S));
-  return std::min(S, (int)(kWsPairs / (size_t)M));
+  return std::min(S, (int)(ws_pairs / (size_t)M));
 }
 
 // Wide kernel geometry: a workgroup of 8 waves owns 128 query rows and one split (its two wave groups take alternate
@@ -95,12 +122,12 @@ int narrow_splits(const yka_kv* kv, int M) {
 // least four 32-key tiles (two steps of either group) per workgroup, sized like the decode grid by the expected context.
 // At 64 rows (three row blocks) that is 21 splits: 64 x 21 x 24 partial rows of 264 bytes, 8.5 MB.
 int wide_rows_per_block(int) { return 128; }
-int wide_splits(const yka_kv* kv, int M) {
+int wide_splits(const yka_kv* kv, int M, size_t ws_pairs = kWsPairs) {
   const int rows = kG * M, rpb = wide_rows_per_block(M), rb = (rows + rpb - 1) / rpb;
   const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
   int S = kv->opt_splits_wide > 0 ? kv->opt_splits_wide : std::min(256 / (kv->cfg.n_kv_heads * rb), ((ctx + 31) / 32) / 4);
   S = std::max(1, std::min(kMaxSplits, S));
-  return std::min(S, std::max(1, (int)kWsPairs / M));
+  return std::min(S, std::max(1, (int)(ws_pairs / (size_t)M)));
 }
 
 void check_layer(const yka_kv* kv, int layer) {
@@ -159,9 +186,11 @@ void need_128(const yka_kv* kv) {
 
 // mode 0: attention + combine; 2: attention kernel alone.  k16/v16 != nullptr asks for quantize-on-append as well:
 // rows of at most 2 tokens fuse it into the attention launch, wider passes launch the append kernel first.
+struct Workspace { float* pm; float* pl; uint16_t* pacc16; size_t pairs; };
 void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_pos, const uint8_t* depth, uint16_t* out16,
-               hipStream_t st, int mode = 0, const uint16_t* k16 = nullptr, const uint16_t* v16 = nullptr) {
+               hipStream_t st, int mode = 0, const uint16_t* k16 = nullptr, const uint16_t* v16 = nullptr, const Workspace* ws = nullptr) {
   const int NH = kv->cfg.n_heads;
+  const Workspace W = ws ? *ws : Workspace{kv->pm, kv->pl, kv->pacc16, kWsPairs};
   if (kv->tb) {
     // trellis-coded rows: the encoder runs first (two launches); rows of at most 2 tokens (or option key 3) run on row
     // tiles of 2 tokens x 6 heads, wider slices on 128-row workgroups that decode every tile once into LDS
@@ -210,11 +239,11 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
   for (int s0 = 0; s0 < M; s0 += kMaxSlice) {   // 64-row slices, as attn_block cuts wide passes (engine35.cpp:935-947)
     const int Ms = std::min(kMaxSlice, M - s0);
     const bool narrow = Ms <= 2 || kv->opt_force_narrow;
-    const int S = narrow ? narrow_splits(kv, Ms) : wide_splits(kv, Ms);
-    AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * kD, d_pos, depth, Ms, s0, NH, S, wide_rows_per_block(Ms), kv->pm, kv->pl, kv->pacc16,
+    const int S = narrow ? narrow_splits(kv, Ms, W.pairs) : wide_splits(kv, Ms, W.pairs);
+    AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * kD, d_pos, depth, Ms, s0, NH, S, wide_rows_per_block(Ms), W.pm, W.pl, W.pacc16,
                fuse_append ? k16 : nullptr, fuse_append ? v16 : nullptr};
     if (narrow) launch_attend_narrow(A, st); else launch_attend_wide(A, st);
-    if (mode != 2) launch_combine(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD, kv->opt_unrot}, st);
+    if (mode != 2) launch_combine(CombineArgs{W.pm, W.pl, W.pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD, kv->opt_unrot}, st);
   }
 }
 
@@ -300,6 +329,7 @@ yka_kv* yka_kv_open(const yka_kv_config* cfg) {
     HIPCHK(hipGetDeviceCount(&ndev));
     if (cfg->device < 0 || cfg->device >= ndev) throw std::runtime_error("device out of range");
     HIPCHK(hipSetDevice(cfg->device));
+    if (cfg->device < kMaxDevices) (void)static_workspace(cfg->device);   // address of this device's static workspace, looked up once per device
     kv = new yka_kv();
     kv->cfg = *cfg;
     kv->n_pages = cfg->max_ctx / kPageTok;
@@ -400,6 +430,22 @@ int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16
   on_device(kv); check_layer(kv, layer); check_rows(kv, M);
   if (!d_q16 || !d_k16 || !d_v16 || !d_pos || !d_out16) throw std::runtime_error("null pointer");
   do_attend(kv, layer, d_q16, M, d_pos, d_depth, d_out16, (hipStream_t)hip_stream, 0, d_k16, d_v16);
+  HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_append_attend_static(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16_t* d_k16, const uint16_t* d_v16, int M,
+                             const int* d_pos, const uint8_t* d_depth, uint16_t* d_out16, void* hip_stream) {
+  YKA_TRY
+  on_device(kv); check_layer(kv, layer); need_128(kv);
+  if (!d_q16 || !d_k16 || !d_v16 || !d_pos || !d_out16) throw std::runtime_error("null pointer");
+  if (M < 1 || M > kMaxSlice || M > kv->cfg.max_rows) throw std::runtime_error("the static workspace serves passes of 1 to 64 rows");
+  if ((size_t)kv->cfg.n_heads > kStaticHeads) throw std::runtime_error("the static workspace is sized for at most 24 query heads");
+  unsigned char* base = kv->cfg.device < kMaxDevices ? g_static_ptr[kv->cfg.device] : nullptr;   // looked up when the handle was opened on this device
+  if (!base) throw std::runtime_error("the static workspace of this device has no address");
+  const Workspace W{reinterpret_cast<float*>(base), reinterpret_cast<float*>(base + kStaticPmBytes),
+                    reinterpret_cast<uint16_t*>(base + 2 * kStaticPmBytes), kStaticPairs * kStaticHeads / (size_t)kv->cfg.n_heads};
+  do_attend(kv, layer, d_q16, M, d_pos, d_depth, d_out16, (hipStream_t)hip_stream, 0, d_k16, d_v16, &W);
   HIPCHK(hipGetLastError());
   YKA_CATCH_INT
 }
