@@ -423,7 +423,7 @@ def main():
         dt, host_dt, out = timed_passes(torch, kv, layers, q[:rows], kn[:rows], vn[:rows], ctx, rows, steps, warmup, issue, args.condition_ms)
         us = dt / steps * 1e6
         # the dominant kernel alone, hipEvents on the library's stream, replayed from a graph over all containers
-        ms, _ = kv.bench(q[:rows], None, None, ctx, mode=2, use_graph=True, reps=20)
+        ms, _, inv = kv.bench(q[:rows], None, None, ctx, mode=2, use_graph=True, reps=20, want_inv=True)
         k_us = float(np.median(ms)) * 1e3 / L
         by, fl = algorithmic_bytes(ctx, rows), algorithmic_flops(ctx, rows)
         hbm_s, mfma_s = by / (HBM_PEAK_GBS * 1e9), fl / (MFMA_F16_PEAK_TFLOPS * 1e12)
@@ -436,6 +436,9 @@ def main():
         roof["kernel_us"] = k_us
         roof["host_clock_us_per_layer"] = host_dt / steps * 1e6
         roof["issue"] = issue
+        # the reference's built-in check (kvx_probe.cu:419-441): the window against one-row passes over the same container
+        roof["window_vs_single_rows"] = {"rows_differing": int(inv[0]), "rows": int(inv[1]), "values_differing": int(inv[2]),
+                                         "max_distance_fp16_spacings": int(inv[3])}
         roof["hbm_frac"] = by / (k_us * 1e-6) / 1e9 / HBM_PEAK_GBS
         return us, by / (us * 1e-6) / 1e9, roof, out
 

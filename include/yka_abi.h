@@ -141,10 +141,15 @@ YKA_API int yka_rotate_q256(const float* d_x32, int rows, uint16_t* d_q16, void*
  * per token and per pair of heads (512 values) y * f16(sigmoid(gate)) -> f16 -> x sign -> 512-point Hadamard transform
  * x 1/sqrt(512) -> f16 -> one scale alpha = max|v| / 127 and int8 codes.  d_y16 = attention outputs [M][n_heads][256]
  * (what yka_attend wrote, un-rotated if option key 4 is set), d_gate16 the same shape, d_signs [n_heads * 256] (+1/-1),
- * d_qx [M][n_heads * 256] int8, d_alpha [M][n_heads * 256 / 512] fp32.  The interleaved small-batch layout of the
- * reference's int8 operand (a8_lo_off, a8_prologue.cuh:121) is not produced.  Allocates nothing, synchronises nothing. */
+ * d_qx [M][n_heads * 256] int8, d_alpha [M][n_heads * 256 / 512] fp32.  Allocates nothing, synchronises nothing. */
 YKA_API int yka_attn_out256(const uint16_t* d_y16, const uint16_t* d_gate16, const int8_t* d_signs, int M, int n_heads,
                             int8_t* d_qx, float* d_alpha, void* hip_stream);
+/* The same step writing the reference's interleaved small-batch layout of the int8 operand (Q35CombineArgs::lo;
+ * a8_lo_off, a8_prologue.cuh:121,132; q35_kernels.cu:1428): at most 8 tokens; d_qx [n_heads / 2][4096], element i of
+ * token t of group g at g * 4096 + (i/256)*2048 + ((i/16)%4)*512 + t*64 + ((i/64)%4)*16 + i%16 (bytes of tokens that are
+ * not part of the pass are left as they are); d_alpha as above. */
+YKA_API int yka_attn_out256_lo(const uint16_t* d_y16, const uint16_t* d_gate16, const int8_t* d_signs, int M, int n_heads,
+                               int8_t* d_qx, float* d_alpha, void* hip_stream);
 
 /* The step between the QKV projection and the cache, fused with quantize-on-append; replaces launch_q35_attn_post
  * (q35.hpp:97-105, q35_kernels.cu:1013-1065) + launch_tb_requant (q35_kernels.cu:1084-1092) for 128-channel heads:
@@ -177,9 +182,11 @@ YKA_API int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float*
 YKA_API int yka_ms_call_host(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M,
                              const int32_t* row_pos, const int32_t* row_slot, uint16_t* out16);
 
-/* Host-pointer form of yka_attn_out256. */
+/* Host-pointer forms of yka_attn_out256 and yka_attn_out256_lo (qx [n_heads / 2][4096], zero where no token wrote). */
 YKA_API int yka_attn_out256_host(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads,
                                  int8_t* qx, float* alpha);
+YKA_API int yka_attn_out256_lo_host(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads,
+                                    int8_t* qx, float* alpha);
 /* Host-pointer forms of yka_append256_f32 and yka_rotate_q256. */
 YKA_API int yka_append256_f32_host(yka_kv* kv, int layer, const float* k32, const float* v32, int M, int pos, int rotate);
 YKA_API int yka_rotate_q256_host(const float* x32, int rows, uint16_t* q16);
@@ -208,10 +215,11 @@ YKA_API int yka_kvx256_probe(const float* x, int rows, int mode, int rot, int8_t
  * y_fq [rows][256] = what each row decodes to according to the encoder; pay [rows][stride]: 8 * kb MSB-first words per
  * coded row (kb = the group's bits per element, 4 for flat groups), zero otherwise; side [rows][2]: the row's fp32 scale
  * and two fp16 projection coefficients; y_dec [rows][256] = the decoder's result from pay and side (x for rows that stay
- * uncoded: position below the group's guard, or no such group).  Bit-identical to the reference's arithmetic for the
- * same blob.  Synchronous; allocates. */
+ * uncoded: position below the group's guard, or no such group).  ms_out (may be NULL): milliseconds of the encode and
+ * of the unpack launches, as the reference's hook reports them (kvx_probe.cu:160).  The argument list is that of
+ * yskn_tbp_pack_unpack.  Bit-identical to the reference's arithmetic for the same blob.  Synchronous; allocates. */
 YKA_API int yka_tb_pack_unpack(const uint8_t* blob, size_t blob_len, const float* x, const int* grp, const int* pos, int rows,
-                               int stride, float* y_fq, uint8_t* pay, uint32_t* side, float* y_dec);
+                               int stride, float* y_fq, uint8_t* pay, uint32_t* side, float* y_dec, float* ms_out);
 
 /* Switches a handle opened with head_dim 256 (not paged) to trellis-coded rows under the given "KVQP" v1 profile (host
  * memory; copied).  Replaces the profile loading of the engine (YSKN_TB_PROFILE, engine35.cpp:38-66) and its packed KV
@@ -278,9 +286,14 @@ YKA_API void yka_pass_destroy(yka_pass* p);
  * stream), each sweep = one layer call per layer on distinct containers.  mode 0 = append + attend, 1 = attend only,
  * 2 = the dominant attention kernel alone (no append, no combine).  ms[r] = time of sweep r in milliseconds.
  * use_graph != 0 replays the sweep from a captured hipGraph (the reference replays captured passes,
- * engine35.cpp:1977-1988). */
+ * engine35.cpp:1977-1988).  inv (may be NULL) receives the reference's built-in invariant (kvx_probe.cu:419-441), taken
+ * on container 0 after the timed sweeps: the M-row pass against M one-row passes at positions pos .. pos + M - 1 -
+ * inv[0] = rows whose outputs differ in any bit, inv[1] = rows compared, inv[2] = output values that differ, inv[3] =
+ * the largest distance between two such values in units of the fp16 spacing.  (The reference demands bit equality of
+ * its one kernel family; here windows of 3+ rows and single rows run on different kernels, whose roundings differ in
+ * the last place, so inv reports how far.) */
 YKA_API int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, int pos,
-                           int mode, int use_graph, int reps, float* ms, uint16_t* out16_last);
+                           int mode, int use_graph, int reps, float* ms, uint16_t* out16_last, int* inv);
 
 /* Machine probe: fixed instruction mixes that time themselves, for the figures the kernels are designed around and the
  * roofline is read against.  Model: the timing part of the reference's bench hooks (kvx_probe.cu:407-413).  Synchronous;

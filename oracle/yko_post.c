@@ -11,6 +11,12 @@
  *                  d <  rd/2: f16( f16(xn[d] * cos) + f16(-xn[d + rd/2] * sin) )
  *                  d >= rd/2: f16( f16(xn[d] * cos) + f16( xn[d - rd/2] * sin) )   with (cos, sin) of channel d - rd/2
  *                then [rotation] -> fp16
+ * Two deliberate differences from the reference's kernel (so this restates its algorithm, not its bit pattern; parity
+ * with the reference's own outputs for this step is UNPINNED - its rsqrtf puts bit equality out of reach anyway - and
+ * the functions here are pinned by the independent fp64 / closed-form checks of tests/test_oracle_post.py): the
+ * reference rounds the projected value to its 16-bit type first (y = rbf(buf[tid]), :1030) and uses that everywhere,
+ * here y stays fp32; and the reference folds 8 warp sums of 32-lane butterflies in sequence (:1050-1056), here the
+ * order is the one below.
  * Sum order of ss (fixed so that every implementation can match it bit for bit): inside each half of 64 channels the
  * butterfly a[i] += a[i ^ o], o = 32, 16, 8, 4, 2, 1; then half 0 + half 1.
  * Rotation for 128 channels: signs from the same integer hash as the 256-channel form (src/kvx_codec.cuh:28-32),

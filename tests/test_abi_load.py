@@ -103,11 +103,11 @@ def test_probe_entry_points_refuse_bad_arguments_before_any_device_call(native):
     from yasakani_amd import kvqp
     blob = np.frombuffer(kvqp.synthetic(), np.uint8)
     grp = np.zeros(2, np.int32); pay = np.zeros((2, 160), np.uint8); side = np.zeros((2, 2), np.uint32)
-    refused(L.yka_tb_pack_unpack(P(blob), blob.size, None, P(grp), P(grp), 2, 160, P(y), P(pay), P(side), P(x)), "bad argument")
-    refused(L.yka_tb_pack_unpack(P(blob), blob.size, P(x), P(grp), P(grp), 0, 160, P(y), P(pay), P(side), P(x)), "bad argument")
-    refused(L.yka_tb_pack_unpack(P(blob), blob.size, P(x), P(grp), P(grp), 2, 162, P(y), P(pay), P(side), P(x)), "stride")
-    refused(L.yka_tb_pack_unpack(P(blob), blob.size, P(x), P(grp), P(grp), 2, 2048, P(y), P(pay), P(side), P(x)), "stride")
-    refused(L.yka_tb_pack_unpack(None, 0, P(x), P(grp), P(grp), 2, 160, P(y), P(pay), P(side), P(x)), "KVQP")
+    refused(L.yka_tb_pack_unpack(P(blob), blob.size, None, P(grp), P(grp), 2, 160, P(y), P(pay), P(side), P(x), None), "bad argument")
+    refused(L.yka_tb_pack_unpack(P(blob), blob.size, P(x), P(grp), P(grp), 0, 160, P(y), P(pay), P(side), P(x), None), "bad argument")
+    refused(L.yka_tb_pack_unpack(P(blob), blob.size, P(x), P(grp), P(grp), 2, 162, P(y), P(pay), P(side), P(x), None), "stride")
+    refused(L.yka_tb_pack_unpack(P(blob), blob.size, P(x), P(grp), P(grp), 2, 2048, P(y), P(pay), P(side), P(x), None), "stride")
+    refused(L.yka_tb_pack_unpack(None, 0, P(x), P(grp), P(grp), 2, 160, P(y), P(pay), P(side), P(x), None), "KVQP")
 
 
 def test_product_does_not_import_the_oracle():

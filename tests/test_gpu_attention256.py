@@ -181,6 +181,33 @@ def test_output_step_gate_hadamard_int8(native, oracle):
     assert diff.max() <= 1 and (diff != 0).mean() < 0.01, (diff.max(), (diff != 0).mean())
 
 
+@pytest.mark.parametrize("M", [1, 5, 8])
+def test_output_step_interleaved_small_batch_layout(native, M):
+    """The reference's interleaved layout for passes of at most 8 tokens (a8_lo_off, src/a8_prologue.cuh:121): the same
+    codes as the plain layout, element i of token t of group g at g*4096 + (i/256)*2048 + ((i/16)%4)*512 + t*64 +
+    ((i/64)%4)*16 + i%16; positions of tokens that are not part of the pass stay untouched (zero in the host form)."""
+    rng = np.random.default_rng(41 + M)
+    H = 24
+    y = rng.standard_normal((M, H, D)).astype(np.float16)
+    gate = (rng.standard_normal((M, H, D)) * 3).astype(np.float16)
+    signs = rng.choice(np.array([-1, 1], np.int8), size=H * D)
+    qx, alpha = native.attn_out256(y, gate, signs)
+    lo, alpha_lo = native.attn_out256_lo(y, gate, signs)
+    assert np.array_equal(alpha.view(np.uint32), alpha_lo.view(np.uint32))
+    # the index map, spelled from its bit fields: i = (b8, b76, b54, b3210) -> (b8, b54, t, b76, b3210)
+    i = np.arange(512)
+    place = ((i >> 8) << 11) | (((i >> 4) & 3) << 9) | (((i >> 6) & 3) << 4) | (i & 15)
+    assert len(set(place.tolist())) == 512 and (place & (7 << 6)).max() == 0        # one-to-one, and it leaves the token field free
+    seen = np.zeros((H // 2, 4096), bool)
+    for t in range(M):
+        for g in range(H // 2):
+            assert np.array_equal(lo[g, place | (t << 6)], qx[t, g * 512:(g + 1) * 512]), (t, g)
+            seen[g, place | (t << 6)] = True
+    assert not lo[~seen].any()
+    with pytest.raises(native.YkaError, match="1 to 8 tokens"):
+        native.attn_out256_lo(np.zeros((9, H, D), np.float16), np.zeros((9, H, D), np.float16), signs)
+
+
 @pytest.mark.parametrize("M", [1, 16, 64])
 def test_full_length_32768(native, oracle, M):
     """32,768 cached tokens (4,096 distinct rows tiled over the context): decode, and windows on the 128-row workgroups,

@@ -643,7 +643,9 @@ std::vector<uint32_t> tb_descriptors(const uint8_t* b, size_t n, const TbInfo& I
 extern "C" {
 
 int yka_tb_pack_unpack(const uint8_t* blob, size_t blob_len, const float* x, const int* grp, const int* pos, int rows, int stride,
-                       float* y_fq, uint8_t* pay, uint32_t* side, float* y_dec) {
+                       float* y_fq, uint8_t* pay, uint32_t* side, float* y_dec, float* ms_out) {
+  hipEvent_t ev[3] = {nullptr, nullptr, nullptr};
+  struct EvGuard { hipEvent_t* e; ~EvGuard() { for (int i = 0; i < 3; ++i) if (e[i]) (void)hipEventDestroy(e[i]); } } ev_guard{ev};
   YKA_TRY
   if (!x || !grp || !pos || rows < 1 || !y_fq || !pay || !side || !y_dec) throw std::runtime_error("bad argument");
   if (stride < 160 || stride > 1024 || stride % 4) throw std::runtime_error("stride must be a multiple of 4 in [160, 1024]");
@@ -659,6 +661,8 @@ int yka_tb_pack_unpack(const uint8_t* blob, size_t blob_len, const float* x, con
   HIPCHK(hipMemcpy(dx.p, x, nx * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dg.p, grp, (size_t)rows * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dp.p, pos, (size_t)rows * 4, hipMemcpyHostToDevice));
+  for (int i = 0; i < 3; ++i) HIPCHK(hipEventCreate(&ev[i]));
+  HIPCHK(hipEventRecord(ev[0], nullptr));
   for (int r0 = 0; r0 < rows; r0 += kTile) {
     TbEncArgs A{};
     A.blob = db.as<uint8_t>(); A.nm = I.nm; A.has_trellis = I.has_trellis;
@@ -670,9 +674,15 @@ int yka_tb_pack_unpack(const uint8_t* blob, size_t blob_len, const float* x, con
     HIPCHK(hipGetLastError());
     HIPCHK(hipDeviceSynchronize());                  // the scratch block is reused by the next tile
   }
+  HIPCHK(hipEventRecord(ev[1], nullptr));
   launch_tb_unpack(db.as<uint8_t>(), dg.as<int>(), dp.as<int>(), dpay.as<uint8_t>(), dside.as<uint32_t>(), stride, dx.as<float>(), dd.as<float>(), rows, nullptr);
+  HIPCHK(hipEventRecord(ev[2], nullptr));
   HIPCHK(hipGetLastError());
   HIPCHK(hipDeviceSynchronize());
+  if (ms_out) {                                        // encode and unpack times, as the reference's hook reports them (kvx_probe.cu:160)
+    HIPCHK(hipEventElapsedTime(&ms_out[0], ev[0], ev[1]));
+    HIPCHK(hipEventElapsedTime(&ms_out[1], ev[1], ev[2]));
+  }
   HIPCHK(hipMemcpy(y_fq, dy.p, nx * 4, hipMemcpyDeviceToHost));
   HIPCHK(hipMemcpy(pay, dpay.p, (size_t)rows * stride, hipMemcpyDeviceToHost));
   HIPCHK(hipMemcpy(side, dside.p, (size_t)rows * 8, hipMemcpyDeviceToHost));
@@ -884,8 +894,36 @@ int yka_attn_out256(const uint16_t* d_y16, const uint16_t* d_gate16, const int8_
   YKA_TRY
   if (!d_y16 || !d_gate16 || !d_signs || !d_qx || !d_alpha) throw std::runtime_error("null pointer");
   if (M < 1 || n_heads < 2 || (n_heads & 1)) throw std::runtime_error("M must be positive and n_heads even");
-  launch_attn_out256(d_y16, d_gate16, d_signs, M, n_heads, d_qx, d_alpha, (hipStream_t)hip_stream);
+  launch_attn_out256(d_y16, d_gate16, d_signs, M, n_heads, 0, d_qx, d_alpha, (hipStream_t)hip_stream);
   HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_attn_out256_lo(const uint16_t* d_y16, const uint16_t* d_gate16, const int8_t* d_signs, int M, int n_heads, int8_t* d_qx,
+                       float* d_alpha, void* hip_stream) {
+  YKA_TRY
+  if (!d_y16 || !d_gate16 || !d_signs || !d_qx || !d_alpha) throw std::runtime_error("null pointer");
+  if (M < 1 || M > 8 || n_heads < 2 || (n_heads & 1)) throw std::runtime_error("the interleaved layout holds 1 to 8 tokens; n_heads must be even");
+  launch_attn_out256(d_y16, d_gate16, d_signs, M, n_heads, 1, d_qx, d_alpha, (hipStream_t)hip_stream);
+  HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_attn_out256_lo_host(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads, int8_t* qx, float* alpha) {
+  YKA_TRY
+  if (!y16 || !gate16 || !signs || !qx || !alpha) throw std::runtime_error("null pointer");
+  if (M < 1 || M > 8 || n_heads < 2 || (n_heads & 1)) throw std::runtime_error("the interleaved layout holds 1 to 8 tokens; n_heads must be even");
+  const size_t n = (size_t)M * n_heads * 256, ng = n / 512, nqx = (size_t)(n_heads / 2) * 4096;
+  DevBuf dy(n * 2), dg(n * 2), ds((size_t)n_heads * 256), dq(nqx), da(ng * 4);
+  HIPCHK(hipMemcpy(dy.p, y16, n * 2, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(dg.p, gate16, n * 2, hipMemcpyHostToDevice));
+  HIPCHK(hipMemcpy(ds.p, signs, (size_t)n_heads * 256, hipMemcpyHostToDevice));
+  HIPCHK(hipMemset(dq.p, 0, nqx));
+  launch_attn_out256(dy.as<uint16_t>(), dg.as<uint16_t>(), ds.as<int8_t>(), M, n_heads, 1, dq.as<int8_t>(), da.as<float>(), nullptr);
+  HIPCHK(hipGetLastError());
+  HIPCHK(hipDeviceSynchronize());
+  HIPCHK(hipMemcpy(qx, dq.p, nqx, hipMemcpyDeviceToHost));
+  HIPCHK(hipMemcpy(alpha, da.p, ng * 4, hipMemcpyDeviceToHost));
   YKA_CATCH_INT
 }
 
@@ -898,7 +936,7 @@ int yka_attn_out256_host(const uint16_t* y16, const uint16_t* gate16, const int8
   HIPCHK(hipMemcpy(dy.p, y16, n * 2, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dg.p, gate16, n * 2, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(ds.p, signs, (size_t)n_heads * 256, hipMemcpyHostToDevice));
-  launch_attn_out256(dy.as<uint16_t>(), dg.as<uint16_t>(), ds.as<int8_t>(), M, n_heads, dq.as<int8_t>(), da.as<float>(), nullptr);
+  launch_attn_out256(dy.as<uint16_t>(), dg.as<uint16_t>(), ds.as<int8_t>(), M, n_heads, 0, dq.as<int8_t>(), da.as<float>(), nullptr);
   HIPCHK(hipGetLastError());
   HIPCHK(hipDeviceSynchronize());
   HIPCHK(hipMemcpy(qx, dq.p, n, hipMemcpyDeviceToHost));
@@ -1119,8 +1157,10 @@ void yka_pass_destroy(yka_pass* p) {
   delete p;
 }
 
+static int f16_order(uint16_t b) { return (b & 0x8000u) ? -(int)(b & 0x7fffu) : (int)(b & 0x7fffu); }   // bit pattern -> position on the fp16 number line
+
 int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const uint16_t* v16, int M, int pos, int mode,
-                   int use_graph, int reps, float* ms, uint16_t* out16_last) {
+                   int use_graph, int reps, float* ms, uint16_t* out16_last, int* inv) {
   hipEvent_t e0 = nullptr, e1 = nullptr;
   hipGraph_t graph = nullptr; hipGraphExec_t gexec = nullptr;
   int rc = 0;
@@ -1168,6 +1208,37 @@ int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const u
     }
     HIPCHK(hipGetLastError());
     if (out16_last) HIPCHK(hipMemcpy(out16_last, dout.p, nq * 2, hipMemcpyDeviceToHost));
+    if (inv) {
+      // the reference's built-in check (kvx_probe.cu:419-441): the M-row pass against M one-row passes over the same
+      // container.  inv[0] = rows whose outputs differ in any bit, inv[1] = rows compared, inv[2] = output values that
+      // differ, inv[3] = the largest distance between two such values in units of fp16 spacing.
+      const size_t row = (size_t)kv->cfg.n_heads * kv->D();
+      std::vector<uint16_t> full(nq), one(row);
+      launch_set_int(kv->d_pos, pos, st);
+      do_attend(kv, 0, dq.as<uint16_t>(), M, kv->d_pos, nullptr, dout.as<uint16_t>(), st);
+      HIPCHK(hipGetLastError());
+      HIPCHK(hipStreamSynchronize(st));
+      HIPCHK(hipMemcpy(full.data(), dout.p, nq * 2, hipMemcpyDeviceToHost));
+      int bad_rows = 0, bad_vals = 0, max_ulp = 0;
+      for (int t = 0; t < M; ++t) {
+        launch_set_int(kv->d_pos, pos + t, st);
+        do_attend(kv, 0, dq.as<uint16_t>() + (size_t)t * row, 1, kv->d_pos, nullptr, dout.as<uint16_t>(), st);
+        HIPCHK(hipGetLastError());
+        HIPCHK(hipStreamSynchronize(st));
+        HIPCHK(hipMemcpy(one.data(), dout.p, row * 2, hipMemcpyDeviceToHost));
+        bool differs = false;
+        for (size_t i = 0; i < row; ++i) {
+          const uint16_t a = full[(size_t)t * row + i], b = one[i];
+          if (a == b) continue;
+          differs = true; ++bad_vals;
+          max_ulp = std::max(max_ulp, std::abs(f16_order(a) - f16_order(b)));
+        }
+        bad_rows += differs;
+      }
+      inv[0] = bad_rows; inv[1] = M; inv[2] = bad_vals; inv[3] = max_ulp;
+      launch_set_int(kv->d_pos, pos, st);
+      HIPCHK(hipStreamSynchronize(st));
+    }
   } catch (const std::exception& e) { g_err = e.what(); rc = -1; }
   catch (...) { g_err = "unknown error"; rc = -1; }
   if (capturing) { hipGraph_t g = nullptr; (void)hipStreamEndCapture(kv->stream, &g); if (g) (void)hipGraphDestroy(g); }   // leave the stream out of capture mode

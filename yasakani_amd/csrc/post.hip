@@ -2,6 +2,13 @@
 // per-head RMS normalisation, partial rotary embedding, optional signed Walsh-Hadamard rotation; Q rows leave as fp16,
 // K and V rows go straight into the int4 cache without a round trip through HBM as fp16.
 // Follows q35_attn_post_kernel (src/q35_kernels.cu:1013-1065) with fp16 in the place of the reference's bf16 roundings.
+// Two deliberate differences from that kernel, so this step is the reference's ALGORITHM, not its bit pattern (which
+// its rsqrtf puts out of reach anyway: parity with the reference's own outputs for this step is unpinned, the kernel is
+// pinned against the oracle's restatement of the sequence below):
+//   * the reference first rounds the projected value to its 16-bit type (y = rbf(buf[tid]), :1030) and forms V, the sum
+//     of squares and xn from that; here the projection's fp32 value is used unrounded (one rounding fewer);
+//   * the reference sums squares by a 32-lane butterfly and then folds its 8 warp sums in sequence (:1050-1056); here the
+//     butterfly runs over 64 lanes and the two wave sums are added.
 // Compiled with -ffp-contract=off; every value is a fixed sequence of single IEEE operations:
 //   ss = sum y^2: butterfly a += a[lane ^ o], o = 32..1, inside each wave (= 64-channel half), then half 0 + half 1
 //   r = 1 / sqrt(ss / 128 + eps);  xn = f16(y * r * (1 + w))

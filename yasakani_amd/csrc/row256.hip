@@ -70,8 +70,10 @@ __global__ void __launch_bounds__(256) row256_decode_kernel(int mode, int rot, c
 // The step after attention for 256-channel heads (src/q35_kernels.cu:1420-1428, src/a8_prologue.cuh:87-98,122-133), fp16 in
 // the place of the reference's bf16 roundings: sigmoid gate, signs, 512-point Hadamard transform x 1/sqrt(512), fp16
 // rounding, int8 with one scale per group of 512.  grid (n_heads / 2, M), block 512: thread = element of the group.
+// lo != 0: the reference's interleaved layout for passes of at most 8 tokens (a8_lo_off, src/a8_prologue.cuh:121,132; qx base
+// + group * 4096): element i of token t of a group sits at (i/256)*2048 + ((i/16)%4)*512 + t*64 + ((i/64)%4)*16 + i%16.
 __global__ void __launch_bounds__(512) attn_out256_kernel(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int n_heads,
-                                                          int8_t* qx, float* alpha) {
+                                                          int lo, int8_t* qx, float* alpha) {
   __shared__ float buf[512];
   __shared__ float red[8];
   const int blk = blockIdx.x, tok = blockIdx.y, tid = threadIdx.x;
@@ -111,13 +113,14 @@ __global__ void __launch_bounds__(512) attn_out256_kernel(const uint16_t* y16, c
   if (tid == 0) alpha[(size_t)tok * (N / 512) + blk] = al;
   int q = al > 0.f ? __float2int_rn(__fdiv_rn(v, al)) : 0;
   q = max(-127, min(127, q));
-  qx[e] = (int8_t)q;
+  if (lo) qx[(size_t)blk * 4096 + (((tid >> 8) << 11) | (((tid >> 4) & 3) << 9) | (tok << 6) | (((tid >> 6) & 3) << 4) | (tid & 15))] = (int8_t)q;
+  else qx[e] = (int8_t)q;
 }
 
 }  // namespace
 
-void launch_attn_out256(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads, int8_t* qx, float* alpha, hipStream_t st) {
-  hipLaunchKernelGGL(attn_out256_kernel, dim3(n_heads / 2, M), dim3(512), 0, st, y16, gate16, signs, n_heads, qx, alpha);
+void launch_attn_out256(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads, int lo, int8_t* qx, float* alpha, hipStream_t st) {
+  hipLaunchKernelGGL(attn_out256_kernel, dim3(n_heads / 2, M), dim3(512), 0, st, y16, gate16, signs, n_heads, lo, qx, alpha);
 }
 
 void launch_row256_encode(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, hipStream_t st) {

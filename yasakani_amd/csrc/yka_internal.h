@@ -142,7 +142,7 @@ void launch_set_int(int* p, int v, hipStream_t);
 void launch_row256_encode(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, hipStream_t);
 void launch_row256_decode(int rows, int mode, int rot, const int8_t* q8, const uint32_t* words, const float* scales, float* y, hipStream_t);
 // the step after attention for 256-channel heads: gate, signs, 512-point Hadamard transform, int8 groups of 512 (n_heads even)
-void launch_attn_out256(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads, int8_t* qx, float* alpha, hipStream_t);
+void launch_attn_out256(const uint16_t* y16, const uint16_t* gate16, const int8_t* signs, int M, int n_heads, int lo, int8_t* qx, float* alpha, hipStream_t);
 
 // machine probe (probe.hip): fixed instruction mixes that time themselves; rec gets (shader cycles, wall ticks) per wave
 void launch_probe_mix(int nv, bool mfma, float* sink, unsigned long long* rec, int iters, int iters_b, int split, int blocks, int threads, hipStream_t);

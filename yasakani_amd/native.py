@@ -54,7 +54,7 @@ def _load():
         "yka_codec_probe": (i32, [vp, i32, vp, vp, vp]),
         "yka_kvx256_probe": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_attn_post": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
-        "yka_tb_pack_unpack": (i32, [vp, C.c_size_t, vp, vp, vp, i32, i32, vp, vp, vp, vp]),
+        "yka_tb_pack_unpack": (i32, [vp, C.c_size_t, vp, vp, vp, i32, i32, vp, vp, vp, vp, vp]),
         "yka_kv_set_profile": (i32, [vp, vp, C.c_size_t]),
         "yka_kv_profile_bits": (i32, [vp]),
         "yka_kv_export_rows_tb": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
@@ -62,6 +62,8 @@ def _load():
         "yka_append256_f32": (i32, [vp, i32, vp, vp, i32, vp, i32, vp]),
         "yka_attn_out256": (i32, [vp, vp, vp, i32, i32, vp, vp, vp]),
         "yka_attn_out256_host": (i32, [vp, vp, vp, i32, i32, vp, vp]),
+        "yka_attn_out256_lo": (i32, [vp, vp, vp, i32, i32, vp, vp, vp]),
+        "yka_attn_out256_lo_host": (i32, [vp, vp, vp, i32, i32, vp, vp]),
         "yka_rotate_q256": (i32, [vp, i32, vp, vp]),
         "yka_append256_f32_host": (i32, [vp, i32, vp, vp, i32, i32, i32]),
         "yka_rotate_q256_host": (i32, [vp, i32, vp]),
@@ -78,7 +80,7 @@ def _load():
         "yka_pass_capture": (vp, [vp, vp, i32, vp, vp, vp, i32, vp, vp, vp, i32]),
         "yka_pass_launch": (i32, [vp, vp]),
         "yka_pass_destroy": (None, [vp]),
-        "yka_attn_bench": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp, vp]),
+        "yka_attn_bench": (i32, [vp, vp, vp, vp, i32, i32, i32, i32, i32, vp, vp, vp]),
         "yka_machine_probe": (i32, [i32, i32, i32, i32, i32, vp]),
     }
     for name, (res, args) in sig.items():
@@ -90,7 +92,7 @@ def _load():
 EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "yka_set_opt", "yka_kv_set_page_table",
            "yka_append", "yka_attend", "yka_append_attend", "yka_append_attend_static", "yka_codec_probe", "yka_kvx256_probe", "yka_tb_pack_unpack", "yka_kv_set_profile", "yka_kv_profile_bits", "yka_kv_export_rows_tb", "yka_attn_post", "yka_append_attend_ms", "yka_ms_call_host",
            "yka_attn_post_host", "yka_kv_export_rows", "yka_kv_export_rows256", "yka_kv_import_rows256",
-           "yka_attn_out256", "yka_attn_out256_host", "yka_append256_f32", "yka_rotate_q256", "yka_append256_f32_host", "yka_rotate_q256_host",
+           "yka_attn_out256", "yka_attn_out256_host", "yka_attn_out256_lo", "yka_attn_out256_lo_host", "yka_append256_f32", "yka_rotate_q256", "yka_append256_f32_host", "yka_rotate_q256_host",
            "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
            "yka_append_host", "yka_pass_capture", "yka_pass_launch", "yka_pass_destroy", "yka_attn_bench", "yka_machine_probe")
 
@@ -163,6 +165,20 @@ def attn_out256(y16, gate16, signs):
     return qx, alpha
 
 
+def attn_out256_lo(y16, gate16, signs):
+    """The same step in the reference's interleaved layout for at most 8 tokens: qx [n_heads/2, 4096] int8 (zero where no
+    token wrote), alpha [M, n_heads*256/512] f32."""
+    y = np.ascontiguousarray(y16); g = np.ascontiguousarray(gate16)
+    M, H, _ = y.shape
+    y = _u16(y, (M, H, 256)); g = _u16(g, (M, H, 256))
+    sg = np.ascontiguousarray(signs, np.int8)
+    if sg.shape != (H * 256,):
+        raise ValueError("signs needs n_heads * 256 entries")
+    qx = np.empty((H // 2, 4096), np.int8); alpha = np.empty((M, H * 256 // 512), np.float32)
+    _chk(lib().yka_attn_out256_lo_host(_ptr(y), _ptr(g), _ptr(sg), M, H, _ptr(qx), _ptr(alpha)))
+    return qx, alpha
+
+
 def rotate_q256(x32):
     """Rotated query rows: x32 [..., 256] fp32 -> fp16 of the signed Walsh-Hadamard rotation of every row."""
     x = np.ascontiguousarray(x32, np.float32)
@@ -197,8 +213,9 @@ def tb_pack_unpack(blob, x, grp, pos, stride=160):
     assert grp.shape == (rows,) and pos.shape == (rows,)
     y = np.empty((rows, 256), np.float32); dec = np.empty((rows, 256), np.float32)
     pay = np.empty((rows, stride), np.uint8); side = np.empty((rows, 2), np.uint32)
-    _chk(lib().yka_tb_pack_unpack(_ptr(b), b.size, _ptr(x), _ptr(grp), _ptr(pos), rows, int(stride), _ptr(y), _ptr(pay), _ptr(side), _ptr(dec)))
-    return dict(x=y, words=pay.view(np.uint32), scale=side[:, 0].copy().view(np.float32), pc=side[:, 1].copy(), dec=dec)
+    ms = np.zeros(2, np.float32)
+    _chk(lib().yka_tb_pack_unpack(_ptr(b), b.size, _ptr(x), _ptr(grp), _ptr(pos), rows, int(stride), _ptr(y), _ptr(pay), _ptr(side), _ptr(dec), _ptr(ms)))
+    return dict(x=y, words=pay.view(np.uint32), scale=side[:, 0].copy().view(np.float32), pc=side[:, 1].copy(), dec=dec, ms=ms)
 
 
 class KvCache:
@@ -384,16 +401,18 @@ class KvCache:
             raise YkaError(lib().yka_last_error().decode("utf-8", "replace"))
         return Pass(h)
 
-    def bench(self, q16, k16, v16, pos, mode=0, use_graph=True, reps=20):
-        """Timed sweeps over all layers; returns (ms per sweep [reps], out of the last layer call)."""
+    def bench(self, q16, k16, v16, pos, mode=0, use_graph=True, reps=20, want_inv=False):
+        """Timed sweeps over all layers; returns (ms per sweep [reps], out of the last layer call) and, if asked, the
+        window-against-single-rows invariant (rows differing, rows compared, values differing, largest fp16-spacing distance)."""
         M = q16.shape[0]
         q = _u16(q16, (M, self.cfg.n_heads, self.cfg.head_dim))
         k = None if k16 is None else _u16(k16, (M, self.cfg.n_kv_heads, self.cfg.head_dim))
         v = None if v16 is None else _u16(v16, (M, self.cfg.n_kv_heads, self.cfg.head_dim))
         ms = np.zeros(reps, np.float32)
         out = np.empty((M, self.cfg.n_heads, self.cfg.head_dim), np.uint16)
-        _chk(lib().yka_attn_bench(self._h, _ptr(q), _ptr(k), _ptr(v), M, pos, mode, int(bool(use_graph)), reps, _ptr(ms), _ptr(out)))
-        return ms, out.view(np.float16)
+        inv = np.zeros(4, np.int32) if want_inv else None
+        _chk(lib().yka_attn_bench(self._h, _ptr(q), _ptr(k), _ptr(v), M, pos, mode, int(bool(use_graph)), reps, _ptr(ms), _ptr(out), _ptr(inv)))
+        return (ms, out.view(np.float16), inv) if want_inv else (ms, out.view(np.float16))
 
 
 class Pass:
