@@ -67,7 +67,12 @@ YKA_API const char* yka_build_info(void);
  *        splits as the length it finds there justifies;
  * key 6: handles with trellis-coded rows, multi-stream passes only: the profile layer whose groups code and decode the
  *        rows (the containers of such a handle are the streams of that one layer; the reference passes the layer in
- *        TbFastArgs::layer / Q35PkArgs::layer). */
+ *        TbFastArgs::layer / Q35PkArgs::layer);
+ * key 7: 1 = the decode kernel (128-channel rows of at most 2 tokens, multi-stream passes, no option key 4) merges its
+ *        splits inside the attention launch: the workgroup that finishes a column last combines it.  0 (default) = a
+ *        second launch combines.  Same results to within the summation order.  On MI355X the second launch is the faster
+ *        form (12.0 against 18.9 us per layer call at 32k tokens): the hand-over between XCDs costs three dependent
+ *        trips to memory (store acknowledged, ticket, loads), more than the gap between two kernels. */
 YKA_API int yka_set_opt(yka_kv* kv, int key, int value);
 
 /* Paged mode: logical page p of `layer` (-1 = every layer) lives in physical page h_table[p]; n_pages = max_ctx/256
@@ -104,7 +109,7 @@ YKA_API int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, cons
  * partials (code under graph capture that is handed a foreign handle, tight serving loops, harnesses that forbid
  * hipMalloc).  No counterpart in the reference.  Same inputs, outputs and results as yka_append_attend - the same kernels
  * and split counts, bit for bit - but the split partials live in a static array inside the library's device code
- * (9,732,096 bytes, held by every GPU the library is used on until the process ends) whose device address is looked up
+ * (9,733,120 bytes, held by every GPU the library is used on until the process ends) whose device address is looked up
  * once per device when a handle is opened there.  Limits: head_dim 128 handles, 1 <= M <= 64 rows (one slice), at most
  * 24 query heads; anything else returns -1 with a message.  The call allocates nothing, frees nothing, synchronises
  * nothing.  Every call on one GPU uses that GPU's one array: calls that overlap on a GPU (two streams, two handles) race

@@ -70,6 +70,30 @@ def test_split_count_does_not_matter(native, oracle):
             assert_attn_close(outs[-1], ref, f"splits={S}")
 
 
+@pytest.mark.parametrize("M,ctx,S", [(1, 3000, 0), (2, 3000, 0), (1, 70, 0), (2, 40000, 0), (1, 40000, 200), (2, 9000, 1)])
+def test_merge_inside_the_launch_equals_second_launch(native, oracle, M, ctx, S):
+    """With option key 7 the decode kernel merges its splits in the workgroup that finishes last (tickets); by default the
+    merge is the combiner launch.  Both are checked against the oracle, against each other (same partials, different summation
+    order: a few fp16 spacings at most), and the one-launch form over repeated calls (the tickets return to zero)."""
+    q, k, v, kn, vn, ch = oracle.make_inputs(520 + M, ctx, M)
+    oc = oracle.Cache(ctx + 64); oc.append(k, v, 0); oc.append(kn, vn, ctx)
+    ref = oc.attend_f32(q, ctx, want_f32=True)[1]
+    with native.KvCache(max_ctx=((ctx + 64 + 255) // 256) * 256) as kv:
+        kv.import_rows(0, 0, oc.kc[:, :ctx], oc.ks[:, :ctx], oc.vc[:, :ctx], oc.vs[:, :ctx])
+        if S:
+            kv.set_opt(1, S)
+        two = kv.layer_call(0, q, kn, vn, ctx)
+        assert_attn_close(two, ref, "two launches")
+        kv.set_opt(7, 1)
+        for rep in range(4):
+            one = kv.layer_call(0, q, kn, vn, ctx)
+            assert_attn_close(one, ref, f"one launch, call {rep}")
+            assert np.abs(one.astype(np.float64) - two.astype(np.float64)).max() <= 2e-3
+            if rep:
+                assert (one.view(np.uint16) == first.view(np.uint16)).all(), rep
+            first = one
+
+
 def test_depth_table(native, oracle):
     ctx, M = 700, 6
     kv, oc, q, kn, vn = _fill(native, oracle, 502, ctx, M)

@@ -66,9 +66,11 @@ def test_rows_of_one_stream_follow_each_other(native, oracle):
         assert_attn_close(out[3:4], refs[2].attend_f32(q[3:4], 900), "stream 2")
 
 
-def test_more_rows_than_sixteen_and_attend_only(native, oracle):
+@pytest.mark.parametrize("merge_in_launch", [0, 1])
+def test_more_rows_than_sixteen_and_attend_only(native, oracle, merge_in_launch):
     kv, refs, rng = _streams(native, oracle, False)
     with kv:
+        kv.set_opt(7, merge_in_launch)
         M = 24
         slots = (np.arange(M) % 4).astype(np.int32)
         pos = np.array([LENS[s] - 1 - (t // 4) for t, s in enumerate(slots)], np.int32)     # positions inside the cached part
@@ -78,9 +80,11 @@ def test_more_rows_than_sixteen_and_attend_only(native, oracle):
             assert_attn_close(out[t:t + 1], refs[s].attend_f32(q[t:t + 1], int(pos[t])), f"row {t}")
 
 
-def test_rejected_rows_yield_zeros_and_touch_nothing(native, oracle):
+@pytest.mark.parametrize("merge_in_launch", [0, 1])
+def test_rejected_rows_yield_zeros_and_touch_nothing(native, oracle, merge_in_launch):
     kv, refs, rng = _streams(native, oracle, False)
     with kv:
+        kv.set_opt(7, merge_in_launch)                    # the last workgroup of a column merges the splits / the combiner launch does
         slots = np.array([1, 9, 3, -1, 2], np.int32)
         pos = np.array([17, 5, -4, 5, CTX], np.int32)     # only row 0 is valid
         q, k, v = _rows(rng, 5)

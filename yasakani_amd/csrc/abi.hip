@@ -30,10 +30,11 @@ struct yka_kv {
   uint8_t* pool = nullptr;
   int32_t* tables = nullptr;       // [n_layers][n_pages], paged mode only
   float *pm = nullptr, *pl = nullptr; uint16_t* pacc16 = nullptr;
+  int* tickets = nullptr;     // [n_kv_heads][64] split tickets of the decode kernel, all zero between launches
   size_t ws_rows = 0;              // capacity of the partial workspace in (token, split) pairs
   int* d_pos = nullptr;            // position used by the host-pointer hooks
   hipStream_t stream = nullptr;    // stream of the host-pointer hooks
-  int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0, opt_unrot = 0, opt_ctx_hint = 0, opt_profile_layer = 0;
+  int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0, opt_unrot = 0, opt_ctx_hint = 0, opt_profile_layer = 0, opt_merge_in_launch = 0;
   // trellis-coded rows (set by yka_kv_set_profile; head_dim 256 only): rows as the reference lays them out, per layer
   // [K payload n_kv * max_ctx * stride][V payload][K scales n_kv * max_ctx fp32][V scales]
   struct Tb {
@@ -63,7 +64,8 @@ struct yka_kv {
 constexpr size_t kStaticPairs = 1536;                              // (token, split) pairs: 64 rows x 21 splits, or 16 rows x 64, ...
 constexpr size_t kStaticHeads = 24;                                // query heads the array is sized for
 constexpr size_t kStaticPmBytes = kStaticPairs * kStaticHeads * 4;  // a multiple of 256
-constexpr size_t kStaticWsBytes = 2 * kStaticPmBytes + kStaticPairs * kStaticHeads * kD * 2;   // 9,732,096 bytes
+constexpr size_t kStaticTicketBytes = 1024;                         // 4 kv heads x 64 row tiles; zero when the library is loaded, zero after every launch
+constexpr size_t kStaticWsBytes = 2 * kStaticPmBytes + kStaticPairs * kStaticHeads * kD * 2 + kStaticTicketBytes;   // 9,733,120 bytes
 static __device__ __align__(256) unsigned char scratch[kStaticWsBytes];
 
 namespace {
@@ -186,11 +188,11 @@ void need_128(const yka_kv* kv) {
 
 // mode 0: attention + combine; 2: attention kernel alone.  k16/v16 != nullptr asks for quantize-on-append as well:
 // rows of at most 2 tokens fuse it into the attention launch, wider passes launch the append kernel first.
-struct Workspace { float* pm; float* pl; uint16_t* pacc16; size_t pairs; };
+struct Workspace { float* pm; float* pl; uint16_t* pacc16; size_t pairs; int* tickets; };
 void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_pos, const uint8_t* depth, uint16_t* out16,
                hipStream_t st, int mode = 0, const uint16_t* k16 = nullptr, const uint16_t* v16 = nullptr, const Workspace* ws = nullptr) {
   const int NH = kv->cfg.n_heads;
-  const Workspace W = ws ? *ws : Workspace{kv->pm, kv->pl, kv->pacc16, kWsPairs};
+  const Workspace W = ws ? *ws : Workspace{kv->pm, kv->pl, kv->pacc16, kWsPairs, kv->tickets};
   if (kv->tb) {
     // trellis-coded rows: the encoder runs first (two launches); rows of at most 2 tokens (or option key 3) run on row
     // tiles of 2 tokens x 6 heads, wider slices on 128-row workgroups that decode every tile once into LDS
@@ -242,8 +244,11 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
     const int S = narrow ? narrow_splits(kv, Ms, W.pairs) : wide_splits(kv, Ms, W.pairs);
     AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * kD, d_pos, depth, Ms, s0, NH, S, wide_rows_per_block(Ms), W.pm, W.pl, W.pacc16,
                fuse_append ? k16 : nullptr, fuse_append ? v16 : nullptr};
+    // option key 7, rows of at most 2 tokens: the last workgroup of each column merges the splits inside the attention launch
+    const bool one_launch = narrow && mode == 0 && !kv->opt_unrot && kv->opt_merge_in_launch;
+    if (one_launch) { A.tickets = W.tickets; A.out16 = out16 + (size_t)s0 * NH * kD; }
     if (narrow) launch_attend_narrow(A, st); else launch_attend_wide(A, st);
-    if (mode != 2) launch_combine(CombineArgs{W.pm, W.pl, W.pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD, kv->opt_unrot}, st);
+    if (mode != 2 && !one_launch) launch_combine(CombineArgs{W.pm, W.pl, W.pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD, kv->opt_unrot}, st);
   }
 }
 
@@ -283,6 +288,7 @@ void do_attend_ms(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const ui
     AttnArgs A{kv->view(0), q16 + (size_t)s0 * NH * D, nullptr, nullptr, Ms, s0, NH, S, 128, kv->pm, kv->pl, kv->pacc16, nullptr, nullptr, Rs};
     const CombineArgs C{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * D, kv->opt_unrot};
     if (r256) { launch_attend256(A, st); launch_combine256(C, st); }
+    else if (!kv->opt_unrot && kv->opt_merge_in_launch) { A.tickets = kv->tickets; A.out16 = C.out16; launch_attend_narrow(A, st); }
     else { launch_attend_narrow(A, st); launch_combine(C, st); }
   }
 }
@@ -347,6 +353,8 @@ yka_kv* yka_kv_open(const yka_kv_config* cfg) {
     HIPCHK(hipMalloc((void**)&kv->pm, np * 4));
     HIPCHK(hipMalloc((void**)&kv->pl, np * 4));
     HIPCHK(hipMalloc((void**)&kv->pacc16, np * cfg->head_dim * 2));
+    HIPCHK(hipMalloc((void**)&kv->tickets, (size_t)cfg->n_kv_heads * kMaxSlice * 4));   // one counter per (kv head, row tile); zero between launches
+    HIPCHK(hipMemset(kv->tickets, 0, (size_t)cfg->n_kv_heads * kMaxSlice * 4));
     HIPCHK(hipMalloc((void**)&kv->d_pos, 4));
     HIPCHK(hipMemset(kv->d_pos, 0, 4));
     HIPCHK(hipStreamCreateWithFlags(&kv->stream, hipStreamNonBlocking));
@@ -369,7 +377,7 @@ void yka_kv_close(yka_kv* kv) {
     (void)hipFree(kv->tb->scr); (void)hipFree(kv->tb->stage);
     delete kv->tb;
   }
-  (void)hipFree(kv->pool); (void)hipFree(kv->tables); (void)hipFree(kv->pm); (void)hipFree(kv->pl); (void)hipFree(kv->pacc16); (void)hipFree(kv->d_pos);
+  (void)hipFree(kv->pool); (void)hipFree(kv->tables); (void)hipFree(kv->pm); (void)hipFree(kv->pl); (void)hipFree(kv->pacc16); (void)hipFree(kv->d_pos); (void)hipFree(kv->tickets);
   delete kv;
 }
 
@@ -383,6 +391,7 @@ int yka_set_opt(yka_kv* kv, int key, int value) {
     case 4: kv->opt_unrot = value != 0; break;
     case 5: if (value < 0) throw std::runtime_error("context hint must be >= 0"); kv->opt_ctx_hint = value; break;
     case 6: if (value < 0) throw std::runtime_error("profile layer must be >= 0"); kv->opt_profile_layer = value; break;
+    case 7: kv->opt_merge_in_launch = value != 0; break;
     default: throw std::runtime_error("unknown option key");
   }
   YKA_CATCH_INT
@@ -444,7 +453,8 @@ int yka_append_attend_static(yka_kv* kv, int layer, const uint16_t* d_q16, const
   unsigned char* base = kv->cfg.device < kMaxDevices ? g_static_ptr[kv->cfg.device] : nullptr;   // looked up when the handle was opened on this device
   if (!base) throw std::runtime_error("the static workspace of this device has no address");
   const Workspace W{reinterpret_cast<float*>(base), reinterpret_cast<float*>(base + kStaticPmBytes),
-                    reinterpret_cast<uint16_t*>(base + 2 * kStaticPmBytes), kStaticPairs * kStaticHeads / (size_t)kv->cfg.n_heads};
+                    reinterpret_cast<uint16_t*>(base + 2 * kStaticPmBytes), kStaticPairs * kStaticHeads / (size_t)kv->cfg.n_heads,
+                    reinterpret_cast<int*>(base + kStaticWsBytes - kStaticTicketBytes)};   // 24 heads = 4 kv heads x 64 row tiles of tickets at most
   do_attend(kv, layer, d_q16, M, d_pos, d_depth, d_out16, (hipStream_t)hip_stream, 0, d_k16, d_v16, &W);
   HIPCHK(hipGetLastError());
   YKA_CATCH_INT

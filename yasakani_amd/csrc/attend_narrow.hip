@@ -23,8 +23,16 @@
 //     and 10 % faster with 32 streams in one launch.  Waves with one or two tiles load them straight away;
 //   * quantize-on-append is fused into the decode launch (a launch costs about 2.5 us here, the same order as the
 //     whole KV stream): the workgroup whose tiles contain a row appended by this pass quantizes and stores that row
-//     before it loads the tile.  The split merge stays a second launch: the 8 XCDs keep separate L2s, so merging in
-//     the last workgroup needs a device-scope release (an L2 write-back) in every workgroup, measured 4x slower.
+//     before it loads the tile;
+//   * the split merge is a second launch by default.  It can ride in the same launch when the caller hands over a
+//     ticket array: every workgroup of a (kv head, row tile) column stores its partials with agent-scope stores (written
+//     through its XCD's L2, which the other XCDs do not see), waits until they are acknowledged, and takes a ticket; the
+//     workgroup that draws the last one reads the column's partials back with agent-scope loads and writes the final
+//     rows.  No cache-wide write-back or invalidate is involved (a device-scope release fence in every workgroup measured
+//     4x slower than a second launch), but the last workgroup still pays three dependent trips to memory after its
+//     tiles - stores acknowledged, ticket, loads - and that measures slower than the gap between two kernels: 14.7
+//     against 8.6 us per layer call at 4k tokens, 18.9 against 12.0 at 32k, 34.0 against 24.9 at 131k (one token; two
+//     tokens add another 7 to 14 us).
 #include "codec_device.h"
 #include "sign_device.h"
 
@@ -100,14 +108,150 @@ __device__ __forceinline__ void wait_tile(RawTile& R) {
                : "n"(N));
 }
 
+// Agent-scope accesses for data that workgroups on different XCDs hand to each other inside one launch: relaxed atomics,
+// which the compiler turns into plain stores and loads with the scope bit that makes them go past the XCD-local L2.
+__device__ __forceinline__ void st_agent(float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ float ld_agent(const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void st_agent16(uint16_t* p, uint4 v) {     // 16 bytes, 16-byte aligned
+  uint64_t* q = reinterpret_cast<uint64_t*>(p);
+  __hip_atomic_store(q, (uint64_t)v.x | ((uint64_t)v.y << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(q + 1, (uint64_t)v.z | ((uint64_t)v.w << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ uint4 ld_agent16(const uint16_t* p) {
+  const uint64_t* q = reinterpret_cast<const uint64_t*>(p);
+  const uint64_t a = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), b = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return make_uint4((uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32));
+}
+
+// The workgroup's partials are out (or its "no keys" markers): wait until the stores are acknowledged, take a ticket of
+// the column.  True for the workgroup that drew the last one: every partial of the column is then visible to agent-scope
+// loads.  It also puts the counter back to zero for the next launch.
+__device__ __forceinline__ bool last_of_column(const AttnArgs& A, int* s_ticket) {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  int* t = A.tickets + blockIdx.y * gridDim.z + blockIdx.z;
+  if (threadIdx.x == 0) {
+    const int old = __hip_atomic_fetch_add(t, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (old == A.S - 1) __hip_atomic_store(t, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    *s_ticket = old;
+  }
+  __syncthreads();
+  return *s_ticket == A.S - 1;
+}
+
+// The combiner of one column (reference: src/attention_kv4q.cu:325-332), run by its last workgroup: 256 threads, rows =
+// the column's tokens x 6 heads.  Per token: thread t weighs split t of each head (w = 2^(m - max m) * l), then 16 split
+// lanes x 16 channel lanes sum w * acc/l over the splits, K splits in flight per lane and head; K * 16 >= S.  All six
+// heads are in flight at once when K is 4 (one memory round trip: decode up to 64 splits), one head at a time otherwise.
+// lds: 6 * 256 + 4 * 6 * 128 + 64 floats.
+template <int TPT, int K>
+__device__ __forceinline__ void combine_column(const AttnArgs& A, int kvh, int rt, float* lds) {
+  constexpr int HB = K <= 4 ? kG : 1;                  // heads per batch of loads
+  float* s_w = lds;                                    // [6][256] weights
+  float* s_o = lds + kG * 256;                         // [4 waves][6 heads][128]
+  float* s_red = s_o + 4 * kG * kD;                    // [4][6] maxima, then [4][6] weight sums
+  const int tid = threadIdx.x, wave = tid >> 6, sl = tid >> 4, c8 = (tid & 15) * 8;
+  const int ntok = min(TPT, A.M - TPT * rt);
+  for (int tk = 0; tk < ntok; ++tk) {
+    const int tj = TPT * rt + tk;
+    const size_t p0 = (size_t)tj * A.S * A.n_heads + kvh * kG;        // (split s, head h) lives at p0 + s * n_heads + h
+    const size_t stride = (size_t)A.n_heads * kD;
+    float pmv[kG], plv[kG];
+#pragma unroll
+    for (int h = 0; h < kG; ++h) {
+      pmv[h] = tid < A.S ? ld_agent(A.pm + p0 + (size_t)tid * A.n_heads + h) : -1e30f;
+      plv[h] = tid < A.S ? ld_agent(A.pl + p0 + (size_t)tid * A.n_heads + h) : 0.f;
+    }
+    uint4 u[HB][K];
+    auto request = [&](int h0) __attribute__((always_inline)) {
+#pragma unroll
+      for (int hh = 0; hh < HB; ++hh)
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+          const int sp = sl + 16 * k;
+          u[hh][k] = sp < A.S ? ld_agent16(A.pacc16 + (p0 + h0 + hh) * kD + (size_t)sp * stride + c8) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    request(0);
+    // maxima over the splits, per head
+    float mx[kG];
+#pragma unroll
+    for (int h = 0; h < kG; ++h) {
+      mx[h] = pmv[h];
+#pragma unroll
+      for (int o = 32; o; o >>= 1) mx[h] = fmaxf(mx[h], __shfl_xor(mx[h], o, 64));
+    }
+    __syncthreads();                                   // the previous token's readers of s_red / s_w / s_o are done
+    if ((tid & 63) == 0)
+#pragma unroll
+      for (int h = 0; h < kG; ++h) s_red[wave * kG + h] = mx[h];
+    __syncthreads();
+    float wsum[kG];
+#pragma unroll
+    for (int h = 0; h < kG; ++h) {
+      const float M2 = fmaxf(fmaxf(s_red[h], s_red[kG + h]), fmaxf(s_red[2 * kG + h], s_red[3 * kG + h]));
+      const float w = (tid < A.S && pmv[h] > -1e29f) ? exp2f(pmv[h] - M2) * plv[h] : 0.f;
+      s_w[h * 256 + tid] = w;
+      wsum[h] = w;
+#pragma unroll
+      for (int o = 32; o; o >>= 1) wsum[h] += __shfl_xor(wsum[h], o, 64);
+    }
+    __syncthreads();                                   // maxima read by everyone, weights written
+    if ((tid & 63) == 0)
+#pragma unroll
+      for (int h = 0; h < kG; ++h) s_red[wave * kG + h] = wsum[h];
+    // weighted sums over the splits
+#pragma unroll
+    for (int h0 = 0; h0 < kG; h0 += HB) {
+      if (h0) request(h0);
+#pragma unroll
+      for (int hh = 0; hh < HB; ++hh) {
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+          const int sp = sl + 16 * k;
+          const float w = sp < A.S ? s_w[(h0 + hh) * 256 + sp] : 0.f;
+          const uint4 r = w != 0.f ? u[hh][k] : make_uint4(0, 0, 0, 0);   // a row of weight 0 may hold anything
+          const h8 v = __builtin_bit_cast(h8, r);
+#pragma unroll
+          for (int c = 0; c < 8; ++c) acc[c] += w * (float)v[c];
+        }
+        // the wave's 4 split lanes (lane bits 4 and 5), then the 4 waves through LDS
+#pragma unroll
+        for (int c = 0; c < 8; ++c) { acc[c] += __shfl_xor(acc[c], 16, 64); acc[c] += __shfl_xor(acc[c], 32, 64); }
+        if ((tid & 48) == 0) {
+          float* d = s_o + (wave * kG + h0 + hh) * kD + c8;
+          *reinterpret_cast<float4*>(d) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+          *reinterpret_cast<float4*>(d + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+        }
+      }
+    }
+    __syncthreads();
+    if (tid < kG * 16) {                               // 16 lanes per head, 8 channels each: one 16-byte store
+      const int h = tid >> 4;
+      const float L = s_red[h] + s_red[kG + h] + s_red[2 * kG + h] + s_red[3 * kG + h];
+      const float inv = L > 0.f ? 1.f / L : 0.f;       // a row that saw no key at all (a rejected row of a multi-stream pass)
+      h8 v;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const float o = s_o[(0 * kG + h) * kD + c8 + c] + s_o[(1 * kG + h) * kD + c8 + c] + s_o[(2 * kG + h) * kD + c8 + c] + s_o[(3 * kG + h) * kD + c8 + c];
+        v[c] = (_Float16)(o * inv);
+      }
+      *reinterpret_cast<uint4*>(A.out16 + ((size_t)tj * A.n_heads + kvh * kG + h) * kD + c8) = __builtin_bit_cast(uint4, v);
+    }
+  }
+}
+
 // grid (S, n_kv, ceil(M/TPT)), block 256 (4 waves).  Workgroup = (split, kv head, row tile of TPT tokens x 6 heads):
 // TPT = 2 for a single-stream pass; MS (multi-stream pass, reference: src/q35_atxpk_ms.cu:13-33): one token per tile,
 // which reads the container and the position its row map names.
 template <bool MS>
 __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
   __shared__ float s_m[4][16], s_l[4][16];
-  __shared__ __align__(16) float s_acc[4][16][kD + 4];
+  __shared__ __align__(16) float s_acc[4][16][kD + 4];     // 8448 floats; the fused combiner needs 4672 of them
+  __shared__ int s_ticket;
   constexpr int TPT = MS ? 1 : 2;
+  const bool fused = A.tickets != nullptr;                 // uniform over the grid
   const int split = blockIdx.x, kvh = blockIdx.y, rt = blockIdx.z;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);     // a scalar: tile indices and page pointers are wave uniform
   const int lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
@@ -144,7 +288,11 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
     const int j = threadIdx.x, tj = TPT * rt + j / kG;
     if (j < TPT * kG && tj < A.M) {
       const size_t p = ((size_t)tj * A.S + split) * A.n_heads + kvh * kG + j % kG;
-      A.pm[p] = -1e30f; A.pl[p] = 0.f;
+      if (fused) { st_agent(A.pm + p, -1e30f); st_agent(A.pl + p, 0.f); }
+      else { A.pm[p] = -1e30f; A.pl[p] = 0.f; }
+    }
+    if (fused && last_of_column(A, &s_ticket)) {
+      if (A.S <= 64) combine_column<TPT, 4>(A, kvh, rt, &s_acc[0][0][0]); else combine_column<TPT, 16>(A, kvh, rt, &s_acc[0][0][0]);
     }
     return;
   }
@@ -343,9 +491,17 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
       h8 v;
 #pragma unroll
       for (int e = 0; e < 8; ++e) v[e] = (_Float16)(acc[e] * inv);
-      *reinterpret_cast<uint4*>(A.pacc16 + p * kD + c8) = __builtin_bit_cast(uint4, v);
-      if (c8 == 0) { A.pm[p] = M2; A.pl[p] = L; }
+      if (fused) {
+        st_agent16(A.pacc16 + p * kD + c8, __builtin_bit_cast(uint4, v));
+        if (c8 == 0) { st_agent(A.pm + p, M2); st_agent(A.pl + p, L); }
+      } else {
+        *reinterpret_cast<uint4*>(A.pacc16 + p * kD + c8) = __builtin_bit_cast(uint4, v);
+        if (c8 == 0) { A.pm[p] = M2; A.pl[p] = L; }
+      }
     }
+  }
+  if (fused && last_of_column(A, &s_ticket)) {   // the barrier inside also ends every read of s_acc above
+    if (A.S <= 64) combine_column<TPT, 4>(A, kvh, rt, &s_acc[0][0][0]); else combine_column<TPT, 16>(A, kvh, rt, &s_acc[0][0][0]);
   }
 }
 

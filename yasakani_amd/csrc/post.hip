@@ -4,7 +4,7 @@
 // Follows q35_attn_post_kernel (src/q35_kernels.cu:1013-1065) with fp16 in the place of the reference's bf16 roundings.
 // Two deliberate differences from that kernel, so this step is the reference's ALGORITHM, not its bit pattern (which
 // its rsqrtf puts out of reach anyway: parity with the reference's own outputs for this step is unpinned, the kernel is
-// pinned against the oracle's restatement of the sequence below):
+// pinned bit for bit against a CPU restatement of the sequence below, kept with the tests):
 //   * the reference first rounds the projected value to its 16-bit type (y = rbf(buf[tid]), :1030) and forms V, the sum
 //     of squares and xn from that; here the projection's fp32 value is used unrounded (one rounding fewer);
 //   * the reference sums squares by a 32-lane butterfly and then folds its 8 warp sums in sequence (:1050-1056); here the

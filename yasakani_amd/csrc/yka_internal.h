@@ -65,6 +65,10 @@ struct AttnArgs {
   // pass and the slice stores its own rows tok0 .. tok0 + M - 1.
   const uint16_t* k16; const uint16_t* v16;
   RowMap rows;  // narrow kernel only: multi-stream pass, one token per workgroup column, no depth table, no fused append
+  // narrow kernel only: tickets != nullptr folds the split combine into the launch - every workgroup of a (kv head, row
+  // tile) column takes a ticket from tickets[kv head * gridDim.z + row tile] once its partials are out, and the one that
+  // draws the last ticket merges the column's partials into out16 and puts the counter back to zero
+  int* tickets = nullptr; uint16_t* out16 = nullptr;
 };
 // unrot != 0: the output row gets the inverse signed Hadamard rotation (7 butterfly stages, x 1/16, signs) before it is
 // rounded to fp16 - the counterpart of rotating V rows on their way into the cache (src/q35_kernels.cu:1421)
