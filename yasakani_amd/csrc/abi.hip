@@ -132,6 +132,18 @@ int wide_splits(const yka_kv* kv, int M, size_t ws_pairs = kWsPairs) {
   return std::min(S, std::max(1, (int)(ws_pairs / (size_t)M)));
 }
 
+// Prefill chunks: slices of up to 1024 tokens (48 row blocks of 128 rows per kv head), splits = the fewest that put three
+// workgroups on every CU (all of them walk nearly the same number of tiles, so the grid drains evenly), each at least
+// eight tiles long and within the partial workspace.
+constexpr int kChunkSlice = 1024;
+int chunk_splits(const yka_kv* kv, int Ms, size_t ws_pairs = kWsPairs) {
+  if (kv->opt_splits_wide > 0) return std::max(1, std::min(kv->opt_splits_wide, (int)(ws_pairs / (size_t)Ms)));
+  const int rb = (kG * Ms + 127) / 128, base = kv->cfg.n_kv_heads * rb;
+  const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
+  int S = std::min((768 + base - 1) / base, ((ctx + 31) / 32) / 8);
+  return std::max(1, std::min(std::min(kMaxSplits, S), (int)(ws_pairs / (size_t)Ms)));
+}
+
 void check_layer(const yka_kv* kv, int layer) {
   if (layer < 0 || layer >= kv->cfg.n_layers) throw std::runtime_error("layer out of range");
 }
@@ -236,12 +248,18 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
   // quantize-on-append rides in the attention launch: in the decode kernel for rows of at most 2 tokens, in the wide
   // kernel for every 64-row slice (each slice stores its own rows); only a wide pass forced through the narrow kernel
   // launches the append kernel first
-  const bool fuse_append = k16 && (M <= 2 || !kv->opt_force_narrow);
+  // A pass of more than 64 rows is a prefill chunk (the reference cuts it into 64-row slices, engine35.cpp:935-947, one
+  // attention launch each).  Here its rows are appended by one launch, then slices of up to 1024 tokens go through the
+  // wide kernel - 128 rows per workgroup whatever the slice, the key range cut evenly into as many splits as give every
+  // CU three workgroups - and one combiner launch per slice merges them.
+  const bool chunk = M > kMaxSlice && !kv->opt_force_narrow && !ws;
+  const bool fuse_append = k16 && !chunk && (M <= 2 || !kv->opt_force_narrow);
   if (k16 && !fuse_append) do_append(kv, layer, k16, v16, M, d_pos, st);
-  for (int s0 = 0; s0 < M; s0 += kMaxSlice) {   // 64-row slices, as attn_block cuts wide passes (engine35.cpp:935-947)
-    const int Ms = std::min(kMaxSlice, M - s0);
-    const bool narrow = Ms <= 2 || kv->opt_force_narrow;
-    const int S = narrow ? narrow_splits(kv, Ms, W.pairs) : wide_splits(kv, Ms, W.pairs);
+  const int slice = chunk ? kChunkSlice : kMaxSlice;
+  for (int s0 = 0; s0 < M; s0 += slice) {
+    const int Ms = std::min(slice, M - s0);
+    const bool narrow = !chunk && (Ms <= 2 || kv->opt_force_narrow);
+    const int S = narrow ? narrow_splits(kv, Ms, W.pairs) : (chunk ? chunk_splits(kv, Ms, W.pairs) : wide_splits(kv, Ms, W.pairs));
     AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * kD, d_pos, depth, Ms, s0, NH, S, wide_rows_per_block(Ms), W.pm, W.pl, W.pacc16,
                fuse_append ? k16 : nullptr, fuse_append ? v16 : nullptr};
     // option key 7, rows of at most 2 tokens: the last workgroup of each column merges the splits inside the attention launch

@@ -1,4 +1,5 @@
-// Split-KV attention for windows of 3..64 query tokens (verify windows, prefill slices).  gfx950.
+// Split-KV attention for windows of 3..64 query tokens (verify windows) and for prefill chunks cut into slices of up to
+// 1024 tokens (one launch per slice, every workgroup 128 rows of it).  gfx950.
 //
 // Same mathematics as the narrow kernel (reference: src/q35_atxpk4.cuh:71-499 for the window shape, row geometry
 // src/q35_atxpk.cu:391-411): every row t of the window runs an online softmax over the keys [0, len(t)) of its
@@ -200,8 +201,11 @@ __global__ void __launch_bounds__(NT) attend_wide_kernel(AttnArgs A) {
   // their own.  The window split has a handful of tiles, so the quantization is off the critical path.
   const int ntiles = (maxlen + 31) >> 5;
   const int Tw = min(ntiles, max(0, pos + A.tok0) >> 5);
+  // A pass wider than one slice (a prefill chunk: its rows were appended by a launch of their own) has no window split:
+  // its key range is cut evenly.
   int tile0, tile1;
   if (A.S == 1) { tile0 = 0; tile1 = ntiles; }
+  else if (A.M > kMaxSlice) { const int tps = (ntiles + A.S - 1) / A.S; tile0 = min(ntiles, split * tps); tile1 = min(ntiles, tile0 + tps); }
   else if (split == A.S - 1) { tile0 = Tw; tile1 = ntiles; }
   else { const int tps = (Tw + A.S - 2) / (A.S - 1); tile0 = split * tps; tile1 = min(Tw, tile0 + tps); }
   // ---- fused quantize-on-append: every workgroup of the window split stores the slice's rows up to its own last
