@@ -33,6 +33,7 @@
 //     tiles - stores acknowledged, ticket, loads - and that measures slower than the gap between two kernels: 14.7
 //     against 8.6 us per layer call at 4k tokens, 18.9 against 12.0 at 32k, 34.0 against 24.9 at 131k (one token; two
 //     tokens add another 7 to 14 us).
+#include <type_traits>
 #include "codec_device.h"
 #include "sign_device.h"
 
@@ -325,17 +326,30 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
 
   // Q fragments: B operand of S^T = K Q^T.  MFMA step m (= scale group m), lane (row i, lane group g), element e
   // <-> channel 32m + 8g + pi(e), pi = [0,4,1,5,2,6,3,7] (the order dq_dword_int produces); odd channels carry 1/16.
+  // The four loads are written as instructions and only requested here: the first tiles are requested right behind them
+  // and q_ready<N> then waits for the query alone, leaving the N tile loads in flight - one trip to memory before the
+  // first MFMA instead of two.  Padding lanes read row 0 of the slice (memory that exists) and drop it.
+  // q_ready is called once in every branch below.  It does not name the query registers as operands of its wait (a
+  // wait site per branch that redefines them makes the compiler place copies of the registers in front of one of the
+  // waits, i.e. copies of registers whose loads are still in flight); instead the wait hands out a zero that is OR-ed
+  // into the raw words, so that nothing computed from them can be scheduled ahead of it.
   h8 qf[4];
+  u32x4 qraw[4];
   {
-    const uint16_t* qrow = A.q16 + ((size_t)tl * A.n_heads + head) * kD + 8 * g;
+    const uint16_t* qrow = A.q16 + (vrow ? ((size_t)tl * A.n_heads + head) * kD : (size_t)0) + 8 * g;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(qraw[m]) : "v"(qrow + 32 * m));
+  }
+  auto q_ready = [&](auto n_younger) __attribute__((always_inline)) {
+    uint32_t z;
+    asm volatile("s_waitcnt vmcnt(%1)\n\tv_mov_b32 %0, 0" : "=v"(z) : "n"(decltype(n_younger)::value));
     const _Float16 sx = (_Float16)0.0625f;
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
-      uint4 u = vrow ? *reinterpret_cast<const uint4*>(qrow + 32 * m) : make_uint4(0, 0, 0, 0);
-      const h8 c = __builtin_bit_cast(h8, u);
+      const h8 c = __builtin_bit_cast(h8, vrow ? (qraw[m] | u32x4{z, z, z, z}) : u32x4{0u, 0u, 0u, 0u});
       qf[m] = h8{c[0], c[4], c[1] * sx, c[5] * sx, c[2], c[6], c[3] * sx, c[7] * sx};
     }
-  }
+  };
   const float sc_log2 = kLog2e / sqrtf((float)kD);
 
   float m_run = -1e30f, l_run = 0.f;
@@ -432,6 +446,7 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
     if (T0 + 8 < tile1) {                              // three tiles or more: the next tile is always in flight
       request(T0, ta);
       request(T0 + 4, tb);
+      q_ready(std::integral_constant<int, 2 * kTileLoads>{});
       for (int T = T0; T < tile1; T += 8) {
         if (T + 4 >= tile1) asm volatile("s_waitcnt vmcnt(0)");
         wait_tile<kTileLoads>(ta);
@@ -448,6 +463,7 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
       // measured 2 % faster than both at once.  Separate registers and no loop: nothing for the compiler to merge.
       RawTile t1;
       request(T0, t1);
+      q_ready(std::integral_constant<int, kTileLoads>{});
       wait_tile<0>(t1);
       tile(T0, t1);
       if (T0 + 4 < tile1) {
@@ -456,6 +472,8 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
         wait_tile<0>(t2);
         tile(T0 + 4, t2);
       }
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // a wave without tiles: the query requests are answered before their registers are given up
     }
   }
   // ---- merge the 4 waves of the workgroup, write one partial per (row, split) ----
