@@ -31,8 +31,8 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # the summary it was taken from, and the JSON line carries that name so that a stale figure can be told from a fresh one.
 # Keyed by (rows, ctx); any other workload reports null.
 MEASURED_TRAFFIC = {
-    (64, 32768): (31.1e6, "profiles/attend_wide_kernel_verify64_ctx32768.md"),
-    (1, 32768): (19.6e6, "profiles/attend_narrow_kernel_decode_ctx32768.md"),
+    (64, 32768): (31.9e6, "profiles/attend_wide_kernel_verify64_ctx32768.md"),      # 23.1 MB read + 8.8 MB written
+    (1, 32768): (19.7e6, "profiles/attend_narrow_kernel_decode_ctx32768.md"),       # 19.3 MB read + 0.4 MB written
 }
 
 
@@ -205,22 +205,25 @@ def trellis_figures(native, ctx=32768, L=16, bits=5, torch=None):
     return out
 
 
-def big_configs(native):
-    """Secondary figures for the two large configurations: a 2048-row prefill chunk on 131072 cached tokens (cut into
-    64-row slices inside the library) and decode / verify-64 on 262144 tokens in shuffled 256-token pages."""
-    out = {}
-    # chunked prefill: 4 containers x 76.7 MB
+def prefill_chunk(native, reps=5):
+    """A 2048-row prefill chunk on 131072 cached tokens: one append launch, then two 1024-token slices through the wide
+    kernel (128 rows per workgroup) and their combiner launches.  4 containers x 76.7 MB."""
     ctx, M, L = 131072, 2048, 4
     q, k, v = synth(31, ctx, M)
     kv = native.KvCache(n_layers=L, max_ctx=ctx + M, max_rows=M)
     fill_cache(kv, k, v, ctx, chunk=16384)
-    ms, _ = kv.bench(q, k[ctx:], v[ctx:], ctx, mode=0, use_graph=True, reps=5)
+    ms, _ = kv.bench(q, k[ctx:], v[ctx:], ctx, mode=0, use_graph=True, reps=reps)
     us = float(np.median(ms)) * 1e3 / L
     keys = sum(ctx + t + 1 for t in range(M))
     fl = 4.0 * NH * D * keys
-    out["prefill_2048_at_131072"] = {"us_per_layer": us, "tflops": fl / (us * 1e-6) / 1e12,
-                                     "mfma_peak_frac": fl / (us * 1e-6) / 1e12 / MFMA_F16_PEAK_TFLOPS}
     kv.close()
+    return {"us_per_layer": us, "tflops": fl / (us * 1e-6) / 1e12, "mfma_peak_frac": fl / (us * 1e-6) / 1e12 / MFMA_F16_PEAK_TFLOPS}
+
+
+def big_configs(native):
+    """Secondary figures for the two large configurations: the prefill chunk above and decode / verify-64 on 262144 tokens
+    in shuffled 256-token pages."""
+    out = {"prefill_2048_at_131072": prefill_chunk(native)}
     # 262144 tokens, shuffled pages: 3 containers x 151 MB
     ctx, L = 262144, 3
     q, k, v = synth(32, ctx, 64)
@@ -389,6 +392,7 @@ def main():
                     help="run only the passes over the reference's 256-channel rows and print their figures (for profiling those kernels)")
     ap.add_argument("--trellis-only", action="store_true",
                     help="run only the passes over trellis-coded rows (5 and 4 bits per element) and print their figures")
+    ap.add_argument("--prefill-only", action="store_true", help="only run the 2048-row prefill chunk on 131072 cached tokens and print it")
     ap.add_argument("--machine", action="store_true", help="only run the machine probe (MFMA rate, read rate, overlap) and print it")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three device-to-device copies of 256 MiB (a kernel of known traffic, for scaling FETCH_SIZE / WRITE_SIZE)")
@@ -403,6 +407,9 @@ def main():
 
     if args.machine:
         print(json.dumps({"machine": machine_figures(native)}))
+        return
+    if args.prefill_only:
+        print(json.dumps({"prefill_2048_at_131072": prefill_chunk(native, reps=8)}))
         return
     if args.r256_only:
         print(json.dumps({"reference_rows_head_dim_256": r256_figures(native, args.ctx)}))

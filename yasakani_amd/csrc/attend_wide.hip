@@ -157,10 +157,28 @@ __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw&
 
 }  // namespace
 
-// grid (S, n_kv, ceil(6M / rows_per_block)), block 512; wave w of either group owns rows [32 w, 32 (w+1)) of the block
+// Workgroup = (split, kv head, row block), block 512; wave w of either group owns rows [32 w, 32 (w+1)) of the block.
+// The row blocks of one (split, kv head) pair read the same KV tiles, and each of the 8 XCDs has an L2 of its own, so the
+// grid is one-dimensional and laid out for the dispatcher's round robin (workgroup i runs on XCD i mod 8, strictly: a
+// workgroup waits for a CU of ITS XCD, so the grid holds exactly pairs x n_rb workgroups and no padding).  XCD x gets
+// n_x = total / 8 (+1 if x < total mod 8) workgroups.  The first F * n_rb of them, F = (total / 8) / n_rb, are the row
+// blocks of F whole pairs (the k-th is row block k mod n_rb of pair x + 8 (k / n_rb)): all row blocks of such a pair run
+// on one XCD at about the same time and each tile leaves HBM once.  The workgroups left over on every XCD take the
+// remaining pairs in order.
 __global__ void __launch_bounds__(NT) attend_wide_kernel(AttnArgs A) {
   __shared__ __align__(16) uint8_t lds[2][2][kLdsBuf];               // [group][buffer]
-  const int split = blockIdx.x, kvh = blockIdx.y, rb = blockIdx.z;
+  const int n_rb = (kG * A.M + A.rows_per_block - 1) / A.rows_per_block;
+  int pair, rb;
+  {
+    const int total = gridDim.x, x = blockIdx.x & 7, k = blockIdx.x >> 3, F = (total >> 3) / n_rb;
+    if (k < F * n_rb) { pair = x + 8 * (k / n_rb); rb = k % n_rb; }
+    else {
+      const int base_e = (total >> 3) - F * n_rb;                     // leftover workgroups of an XCD, +1 on the first total mod 8
+      const int jj = x * base_e + min(x, total & 7) + (k - F * n_rb);
+      pair = 8 * F + jj / n_rb; rb = jj % n_rb;
+    }
+  }
+  const int split = pair % A.S, kvh = pair / A.S;
   const int tid = threadIdx.x, gt = tid & (NTG - 1);                  // gt: thread index inside the group
   const int grp = __builtin_amdgcn_readfirstlane(tid >> 8);           // wave uniform
   const int wave = __builtin_amdgcn_readfirstlane(gt >> 6), lane = tid & 63, j = lane & 31, h = lane >> 5;
@@ -454,7 +472,7 @@ __global__ void __launch_bounds__(NT) attend_wide_kernel(AttnArgs A) {
 
 void launch_attend_wide(const AttnArgs& A, hipStream_t st) {
   const int rows = kG * A.M, rb = (rows + A.rows_per_block - 1) / A.rows_per_block;
-  hipLaunchKernelGGL(attend_wide_kernel, dim3(A.S, A.kv.n_kv, rb), dim3(NT), 0, st, A);
+  hipLaunchKernelGGL(attend_wide_kernel, dim3(A.S * A.kv.n_kv * rb), dim3(NT), 0, st, A);
 }
 
 }  // namespace yka
