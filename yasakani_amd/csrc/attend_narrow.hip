@@ -605,7 +605,54 @@ __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
   }
   if (tid < kD) A.out16[((size_t)tok * A.n_heads + head) * kD + tid] = __half_as_ushort(__float2half_rn(y));
 }
+// The combiner for wide passes (many rows, at most 32 splits, no un-rotation): one wave per (token, head) row, four
+// waves per workgroup, no LDS and no barrier.  Lane = (split lane 0..3, 8 channels); a split lane takes splits sl, sl + 4,
+// ... (at most 8), requests their rows together with the (m, l) pairs, and the four split lanes are summed by two
+// cross-lane exchanges.  Same arithmetic as combine_kernel up to the order of the sums.
+__global__ void __launch_bounds__(256) combine_rows_kernel(CombineArgs A) {
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);               // row = tok * n_heads + head
+  if (row >= A.M * A.n_heads) return;
+  const int tok = row / A.n_heads, head = row % A.n_heads, lane = threadIdx.x & 63, sl = lane >> 4, c8 = (lane & 15) * 8;
+  const size_t p0 = (size_t)tok * A.S * A.n_heads + head;
+  const size_t stride = (size_t)A.n_heads * kD;
+  uint4 u[8];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int sp = sl + 4 * k;
+    u[k] = sp < A.S ? *reinterpret_cast<const uint4*>(A.pacc16 + p0 * kD + (size_t)sp * stride + c8) : make_uint4(0, 0, 0, 0);
+  }
+  // lane t < S looks at split t; the maximum and every weight then come from cross-lane reads
+  float pmv = -1e30f, plv = 0.f;
+  if (lane < A.S) { pmv = A.pm[p0 + (size_t)lane * A.n_heads]; plv = A.pl[p0 + (size_t)lane * A.n_heads]; }
+  float M2 = pmv;
+#pragma unroll
+  for (int o = 32; o; o >>= 1) M2 = fmaxf(M2, __shfl_xor(M2, o, 64));
+  const float wl = (lane < A.S && pmv > -1e29f) ? exp2f(pmv - M2) * plv : 0.f;     // weight of split `lane`
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float wsum = 0.f;
+#pragma unroll
+  for (int k = 0; k < 8; ++k) {
+    const int sp = sl + 4 * k;                                       // < 32: a lane of this wave
+    const float w = __shfl(wl, sp, 64);
+    const uint4 r = w != 0.f ? u[k] : make_uint4(0, 0, 0, 0);         // a row of weight 0 may be one that no workgroup wrote
+    const h8 v = __builtin_bit_cast(h8, r);
+#pragma unroll
+    for (int c = 0; c < 8; ++c) acc[c] += w * (float)v[c];
+    wsum += w;
+  }
+#pragma unroll
+  for (int c = 0; c < 8; ++c) { acc[c] += __shfl_xor(acc[c], 16, 64); acc[c] += __shfl_xor(acc[c], 32, 64); }
+  wsum += __shfl_xor(wsum, 16, 64); wsum += __shfl_xor(wsum, 32, 64);
+  if (sl == 0) {
+    const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
+    h8 v;
+#pragma unroll
+    for (int c = 0; c < 8; ++c) v[c] = (_Float16)(acc[c] * inv);
+    *reinterpret_cast<uint4*>(A.out16 + (size_t)row * kD + c8) = __builtin_bit_cast(uint4, v);
+  }
+}
 void launch_combine(const CombineArgs& A, hipStream_t st) {
+  if (A.S <= 32 && !A.unrot && A.M >= 8) { hipLaunchKernelGGL(combine_rows_kernel, dim3((A.M * A.n_heads + 3) / 4), dim3(256), 0, st, A); return; }
   if (A.S > 64) hipLaunchKernelGGL(combine_kernel<16>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);    // S <= 256
   else hipLaunchKernelGGL(combine_kernel<4>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
 }
