@@ -11,7 +11,11 @@
  *     sets no function attribute: everything is reserved in yka_kv_open (engine35.cpp:323-326);
  *   - hooks that take host pointers allocate, copy, launch, synchronise and free inside (src/kvx_probe.cu).
  * One caller at a time per handle; any host thread may call (the device of the handle is made current first,
- * as on_gpu does in c_api.cpp:22-31).
+ * as on_gpu does in c_api.cpp:22-31).  One stream in flight per handle as well: a handle owns ONE set of split
+ * partials, one device position word and (trellis rows) one encoder scratch, which every launch and every replay of a
+ * pass captured from it uses.  Work of one handle issued on two streams, or a replay issued while an earlier call on
+ * the handle may still run on another stream, races on them; order such work with events or keep it on one stream
+ * (the reference replays its passes on the one stream of its engine, engine35.cpp:1977-1988).
  *
  * Formats, selected by head_dim at open:
  *   128: symmetric signed int4 codes stored as q+8, two per byte, even channel in the low nibble; one fp16 scale per
