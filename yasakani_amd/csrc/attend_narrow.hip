@@ -9,8 +9,11 @@
 //     every scale group into that chunk, so MFMA step m contracts exactly the 32 channels of group m.  V is read as
 //     one dword per (lane, token) so that a lane ends up with 8 tokens of the same 8 channels - the operand shape
 //     the token-contracting MFMA needs;
-//   * codes become fp16 without integer conversion: a nibble OR-ed into the mantissa of 1024.0 is 1024+n (or
-//     1024+16n for the odd nibble of a byte); subtracting 1032 (1152) gives n-8 (16(n-8)) exactly;
+//   * codes become fp16 without integer conversion.  V: a nibble OR-ed into the mantissa of 1024.0 is 1024+n (or
+//     1024+16n for the odd nibble of a byte); subtracting 1032 (1152) gives n-8 (16(n-8)) exactly.  K: a nibble left in
+//     place in a zero word IS an fp16, the subnormal n * 2^-24, and the matrix pipe takes subnormal inputs unflushed: an
+//     AND per pair of codes is the whole conversion, the offset -8 rides in the MFMA's initial accumulator as
+//     -8 * 2^-24 * sum(q) per (row, scale group), and the 2^24 is folded into the exponent's scale;
 //   * K stays exact: the MFMA multiplies Q by the integer codes, and the fp16 group scale is applied to the fp32
 //     partial sum of each group (rounding q*scale to fp16 first costs 7e-4 relative L2 on inputs with outlier
 //     channels, most of the 1e-3 budget).  V is scaled in fp16 (one rounding, 2e-4);
@@ -62,6 +65,19 @@ __device__ __forceinline__ void dq_dword_int(uint32_t w, h2* out, uint32_t magic
   out[2] = as_h2(nib(t, 0x000f000fu, magic)) - c1032;
   out[3] = as_h2(nib(t, 0x00f000f0u, magic)) - c1152;
 }
+
+// K codes for the score MFMA need no arithmetic at all: a nibble left in place in an otherwise zero fp16 is the
+// subnormal n * 2^-24 (16 n * 2^-24 for the odd nibble of a byte), which the matrix pipe multiplies exactly like any
+// other fp16.  The offset of the code (-8 per channel) becomes -8 * sum(q) per (row, scale group), which the MFMA gets as
+// its initial accumulator, and the factor 2^24 is folded into the exponent's scale.  Same element order as dq_dword_int.
+__device__ __forceinline__ void dq_dword_sub(uint32_t w, h2* out) {
+  const uint32_t t = w >> 8;
+  out[0] = as_h2(w & 0x000f000fu);
+  out[1] = as_h2(w & 0x00f000f0u);
+  out[2] = as_h2(t & 0x000f000fu);
+  out[3] = as_h2(t & 0x00f000f0u);
+}
+constexpr float kTwo24 = 16777216.f, kTwoM24 = 1.f / 16777216.f;
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
@@ -334,6 +350,7 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
   // waits, i.e. copies of registers whose loads are still in flight); instead the wait hands out a zero that is OR-ed
   // into the raw words, so that nothing computed from them can be scheduled ahead of it.
   h8 qf[4];
+  f4 kinit[4];                 // initial accumulators of the score MFMAs: the code offset -8, see dq_dword_sub
   u32x4 qraw[4];
   {
     const uint16_t* qrow = A.q16 + (vrow ? ((size_t)tl * A.n_heads + head) * kD : (size_t)0) + 8 * g;
@@ -348,9 +365,17 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
     for (int m = 0; m < 4; ++m) {
       const h8 c = __builtin_bit_cast(h8, vrow ? (qraw[m] | u32x4{z, z, z, z}) : u32x4{0u, 0u, 0u, 0u});
       qf[m] = h8{c[0], c[4], c[1] * sx, c[5] * sx, c[2], c[6], c[3] * sx, c[7] * sx};
+      // -8 * 2^-24 * (sum of the row's 32 query channels of group m): the lane's 8 channels, then its 3 sister lanes
+      float qs = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) qs += (float)c[e];
+      qs += __shfl_xor(qs, 16, 64);
+      qs += __shfl_xor(qs, 32, 64);
+      const float c0 = -8.f * kTwoM24 * qs;
+      kinit[m] = f4{c0, c0, c0, c0};
     }
   };
-  const float sc_log2 = kLog2e / sqrtf((float)kD);
+  const float sc_log2 = kTwo24 * kLog2e / sqrtf((float)kD);       // scores carry the 2^-24 of the subnormal codes
 
   float m_run = -1e30f, l_run = 0.f;
   f4 o[8];
@@ -373,9 +398,9 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         h2 k4[4];
-        dq_dword_int(w[m], k4, magic);
+        dq_dword_sub(w[m], k4);
         const h8 kf = h8{k4[0][0], k4[0][1], k4[1][0], k4[1][1], k4[2][0], k4[2][1], k4[3][0], k4[3][1]};
-        part[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[m], f4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+        part[m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf, qf[m], kinit[m], 0, 0, 0);
       }
       // part[m][r] = sum over group m of q * code for key t0 + 16kt + 4g + r and row i
       const uint32_t sw[8] = {cur.ks[kt][0][0], cur.ks[kt][0][1], cur.ks[kt][0][2], cur.ks[kt][0][3],
