@@ -505,10 +505,13 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
   l_run += __shfl_xor(l_run, 16, 64);
   l_run += __shfl_xor(l_run, 32, 64);
   if (g == 0) { s_m[wave][i] = m_run; s_l[wave][i] = l_run; }
+  // o[b][r] of lane (row i, group g) is channel 8 (4g + r) + b: eight consecutive channels per r, two 16-byte writes
 #pragma unroll
-  for (int b = 0; b < 8; ++b)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) s_acc[wave][i][8 * (4 * g + r) + b] = o[b][r];
+  for (int r = 0; r < 4; ++r) {
+    float* d = &s_acc[wave][i][8 * (4 * g + r)];
+    *reinterpret_cast<float4*>(d) = make_float4(o[0][r], o[1][r], o[2][r], o[3][r]);
+    *reinterpret_cast<float4*>(d + 4) = make_float4(o[4][r], o[5][r], o[6][r], o[7][r]);
+  }
   __syncthreads();
   // 16 lanes per row, 8 channels each: one 16-byte store per lane
   if (threadIdx.x < TPT * kG * 16) {
