@@ -31,7 +31,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # the summary it was taken from, and the JSON line carries that name so that a stale figure can be told from a fresh one.
 # Keyed by (rows, ctx); any other workload reports null.
 MEASURED_TRAFFIC = {
-    (64, 32768): (31.9e6, "profiles/attend_wide_kernel_verify64_ctx32768.md"),      # 23.1 MB read + 8.8 MB written
+    (64, 32768): (32.4e6, "profiles/attend_wide_kernel_verify64_ctx32768.md"),      # 23.6 MB read + 8.8 MB written
     (1, 32768): (19.7e6, "profiles/attend_narrow_kernel_decode_ctx32768.md"),       # 19.3 MB read + 0.4 MB written
 }
 
