@@ -364,6 +364,12 @@ def machine_figures(native):
     out["cycles_per_mfma_with_6_fma_behind_it"] = r6["cycles"] / (it * 4)
     rf = native.machine_probe(2, 8, it, 256, 256)
     out["cycles_per_v_fma_f32_one_wave"] = rf["cycles"] / (it * 32)
+    # one wave of MFMAs and one wave of packed-fp16 multiplies on every SIMD: how far the two pipes run side by side
+    rp = native.machine_probe(2, 1, it, 256, 256)
+    rx = native.machine_probe(5, 1, it, 256, 512)
+    out["cycles_per_v_pk_mul_f16_one_wave"] = rp["cycles"] / (it * 32)
+    out["cycles_per_v_pk_mul_f16_beside_an_mfma_wave"] = rx["cycles_b"] / (max(1, it * 2 // 3) * 32)
+    out["cycles_per_mfma_beside_a_vector_wave"] = rx["cycles"] / (it * 4)
     for nt in (0, 1):
         r = native.machine_probe(4, nt, 2048, 16384, 256)
         out["read_GBs_nontemporal" if nt else "read_GBs_plain"] = 2048 * 1048576 / (r["ms"] * 1e-3) / 1e9

@@ -314,8 +314,10 @@ YKA_API int yka_attn_bench(yka_kv* kv, const uint16_t* q16, const uint16_t* k16,
  *   kind 3: 512 lanes; waves 0-3 of a workgroup run kind 0 with p0 = 0, waves 4-7 run p0 iterations of 32 v_fma_f32: two
  *           waves per SIMD, one of each kind
  *   kind 4: streaming read of iters MiB in 16-byte pieces; p0 != 0: nontemporal loads
+ *   kind 5: 512 lanes; waves 0-3 run kind 0 with p0 = 0 (iters x 4 MFMAs), waves 4-7 run (2/3 iters) x 32 instructions
+ *           of the vector opcode p0 of kind 2 (0..7): how far the matrix pipe and that opcode run side by side
  * out[0] = milliseconds of the timed launch (events); out[1], out[2] = mean shader-clock cycles and mean wall-clock
- * ticks a wave measured around its loop (kind 3: waves 0-3); out[3], out[4] the same for waves 4-7 of kind 3;
+ * ticks a wave measured around its loop (kinds 3 and 5: waves 0-3); out[3], out[4] the same for waves 4-7 of kinds 3, 5;
  * out[5] = wall-clock ticks per millisecond. */
 YKA_API int yka_machine_probe(int kind, int p0, int iters, int blocks, int threads, double* out);
 

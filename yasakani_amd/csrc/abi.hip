@@ -1079,11 +1079,13 @@ int yka_machine_probe(int kind, int p0, int iters, int blocks, int threads, doub
   hipEvent_t e0 = nullptr, e1 = nullptr;
   int rc = 0;
   try {
-    if (!out || kind < 0 || kind > 4 || iters < 1 || blocks < 1 || blocks > 65536) throw std::runtime_error("bad argument");
+    if (!out || kind < 0 || kind > 5 || iters < 1 || blocks < 1 || blocks > 65536) throw std::runtime_error("bad argument");
     if (threads != 256 && threads != 512) throw std::runtime_error("threads must be 256 or 512");
     if (kind == 0 && (p0 < 0 || p0 > 8 || (p0 & 1))) throw std::runtime_error("kind 0: p0 = vector FMAs per MFMA, one of 0 2 4 6 8");
     if (kind == 2 && (p0 < 0 || p0 > 8)) throw std::runtime_error("kind 2: p0 = opcode 0..8");
     if (kind == 3 && (p0 < 1 || threads != 512)) throw std::runtime_error("kind 3: p0 = iterations of the vector waves, 512 threads");
+    if (kind == 5 && (p0 < 0 || p0 > 7)) throw std::runtime_error("kind 5: p0 = opcode 0..7");
+    if (kind == 5) threads = 512;
     if (kind == 4 && iters > 4096) throw std::runtime_error("kind 4: iters = MiB to read, at most 4096");
     if (kind == 1) threads = 256;
     const int waves = blocks * (threads / 64);
@@ -1103,6 +1105,7 @@ int yka_machine_probe(int kind, int p0, int iters, int blocks, int threads, doub
                 else launch_probe_valu(p0, sink.as<float>(), r, iters, blocks, threads, nullptr);
                 break;
         case 3: launch_probe_mix(0, true, sink.as<float>(), r, iters, p0, 1, blocks, 512, nullptr); break;
+        case 5: launch_probe_cross(p0, sink.as<float>(), r, iters, std::max(1, iters * 2 / 3), blocks, nullptr); break;
         default: launch_probe_read(p0 != 0, src.p, nbytes, sink.as<float>(), blocks, nullptr); break;
       }
     };
@@ -1122,7 +1125,7 @@ int yka_machine_probe(int kind, int p0, int iters, int blocks, int threads, doub
     double sum[4] = {0, 0, 0, 0}; size_t cnt[2] = {0, 0};
     const int wpb = threads / 64;
     for (int w = 0; w < waves; ++w) {
-      const int cls = (kind == 3 && (w % wpb) >= 4) ? 1 : 0;
+      const int cls = ((kind == 3 || kind == 5) && (w % wpb) >= 4) ? 1 : 0;
       sum[2 * cls] += (double)h[2 * (size_t)w]; sum[2 * cls + 1] += (double)h[2 * (size_t)w + 1]; ++cnt[cls];
     }
     int wall_khz = 0;

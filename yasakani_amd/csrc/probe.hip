@@ -122,6 +122,43 @@ __global__ void __launch_bounds__(512) valu_kernel(float* sink, unsigned long lo
 
 // streaming read: every thread reads 16-byte pieces, a workgroup a contiguous 64 KiB block at a time
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+// One wave of MFMAs and one wave of a given vector opcode on every SIMD (waves 0-3 / 4-7 of a 512-thread workgroup): how
+// far the matrix pipe and that opcode's pipe run side by side when the instructions come from different waves.
+template <int OP>
+__global__ void __launch_bounds__(512) cross_kernel(float* sink, unsigned long long* rec, int iters, int iters_b) {
+  const int wave = threadIdx.x >> 6, wave_id = blockIdx.x * (blockDim.x >> 6) + wave;
+  f16v a0{}, a1{}, a2{}, a3{};
+  float x0 = 0.001f * threadIdx.x, x1 = x0 + 1, x2 = x0 + 2, x3 = x0 + 3, x4 = x0 + 4, x5 = x0 + 5, x6 = x0 + 6, x7 = x0 + 7;
+  const h8 fa = {1, 1, 1, 1, 1, 1, 1, 1}, fb = {1, 1, 1, 1, 1, 1, 1, 1};
+  const float c1 = 0.999f, c2 = 0.001f;
+  float x[8] = {x0, x1, x2, x3, x4, x5, x6, x7};
+  __syncthreads();
+  const WaveClock t = tick();
+  if (wave >= 4) {
+    for (int it = 0; it < iters_b; ++it) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          if (OP == 0) asm volatile("v_exp_f32 %0, %0" : "+v"(x[i]));
+          if (OP == 1) asm volatile("v_pk_mul_f16 %0, %0, %0" : "+v"(x[i]));
+          if (OP == 2) asm volatile("v_cvt_pk_f16_f32 %0, %0, %0" : "+v"(x[i]));
+          if (OP == 3) asm volatile("v_max3_f32 %0, %0, %0, %0" : "+v"(x[i]));
+          if (OP == 4) asm volatile("v_and_or_b32 %0, %0, %0, %0" : "+v"(x[i]));
+          if (OP == 5) asm volatile("v_pk_add_f16 %0, %0, %0" : "+v"(x[i]));
+          if (OP == 6) asm volatile("v_perm_b32 %0, %0, %0, %0" : "+v"(x[i]));
+          if (OP == 7) asm volatile("v_mul_f32 %0, %0, %0" : "+v"(x[i]));
+        }
+    }
+  } else {
+    for (int it = 0; it < iters; ++it) body<0, true>(a0, a1, a2, a3, x0, x1, x2, x3, x4, x5, x6, x7, fa, fb, c1, c2);
+  }
+  YKA_SETTLE;
+  tock(t, rec, wave_id);
+  const float s = a0[0] + a1[1] + a2[2] + a3[3] + x[0] + x[1] + x[2] + x[3] + x[4] + x[5] + x[6] + x[7];
+  if (s == 12345.678f) sink[wave_id] = s;
+}
+
 template <bool NT>
 __global__ void __launch_bounds__(256) read_kernel(const u32x4* src, size_t n16, float* sink) {
   uint32_t acc = 0;
@@ -162,6 +199,14 @@ void launch_probe_valu(int op, float* sink, unsigned long long* rec, int iters, 
     case 4: YKA_V(4); break; case 5: YKA_V(5); break; case 6: YKA_V(6); break; default: YKA_V(7); break;
   }
 #undef YKA_V
+}
+void launch_probe_cross(int op, float* sink, unsigned long long* rec, int iters, int iters_b, int blocks, hipStream_t st) {
+#define YKA_X(OP) hipLaunchKernelGGL(cross_kernel<OP>, dim3(blocks), dim3(512), 0, st, sink, rec, iters, iters_b)
+  switch (op) {
+    case 0: YKA_X(0); break; case 1: YKA_X(1); break; case 2: YKA_X(2); break; case 3: YKA_X(3); break;
+    case 4: YKA_X(4); break; case 5: YKA_X(5); break; case 6: YKA_X(6); break; default: YKA_X(7); break;
+  }
+#undef YKA_X
 }
 void launch_probe_read(bool nt, const void* src, size_t bytes, float* sink, int blocks, hipStream_t st) {
   if (nt) hipLaunchKernelGGL(read_kernel<true>, dim3(blocks), dim3(256), 0, st, (const u32x4*)src, bytes / 16, sink);

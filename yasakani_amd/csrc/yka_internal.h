@@ -152,6 +152,7 @@ void launch_attn_out256(const uint16_t* y16, const uint16_t* gate16, const int8_
 void launch_probe_mix(int nv, bool mfma, float* sink, unsigned long long* rec, int iters, int iters_b, int split, int blocks, int threads, hipStream_t);
 void launch_probe_mfma16(float* sink, unsigned long long* rec, int iters, int blocks, hipStream_t);
 void launch_probe_valu(int op, float* sink, unsigned long long* rec, int iters, int blocks, int threads, hipStream_t);
+void launch_probe_cross(int op, float* sink, unsigned long long* rec, int iters, int iters_b, int blocks, hipStream_t);
 void launch_probe_read(bool nt, const void* src, size_t bytes, float* sink, int blocks, hipStream_t);
 
 // start of the (page, kv head) block that holds token t
