@@ -80,6 +80,19 @@ def test_static_workspace_call_equals_the_allocating_one(native, oracle):
             oc.kc[:, :n], oc.ks[:, :n], oc.vc[:, :n], oc.vs[:, :n] = kv.export_rows(1, 0, n)
             M, off = calls[-1]
             assert_attn_close(b.view(np.float16), oc.attend_f32(q_all[off:off + M], pos - M, threads=4, want_f32=True)[1], "last static call")
+            # with the merge of the decode splits inside the launch (option key 7) the static call takes its split tickets
+            # from the static array too (all zero after every launch): two calls in a row, against the allocating call
+            kv.set_opt(7, 1)
+            for M, off in ((2, 80), (1, 82), (1, 80)):
+                hip.upload(dq, q_all[off:off + M].view(np.uint16)); hip.upload(dk, k_new[off:off + M].view(np.uint16)); hip.upload(dv, v_new[off:off + M].view(np.uint16))
+                hip.upload(dpos, np.array([ctx + off], np.int32))
+                kv.append_attend(0, dq, dk, dv, M, dpos, dout_a)
+                kv.append_attend_static(1, dq, dk, dv, M, dpos, dout_b)
+                hip.sync()
+                a = np.empty((M, 24, 128), np.uint16); b = np.empty((M, 24, 128), np.uint16)
+                hip.download(dout_a, a); hip.download(dout_b, b)
+                assert (a == b).all(), f"outputs differ at M={M} with the merge inside the launch"
+            kv.set_opt(7, 0)
             # limits are refused with a message, before anything is launched
             with pytest.raises(native.YkaError, match="64 rows"):
                 kv.append_attend_static(1, dq, dk, dv, 65, dpos, dout_b)
