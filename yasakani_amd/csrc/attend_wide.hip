@@ -218,10 +218,11 @@ __global__ void __launch_bounds__(NT) attend_wide_kernel(AttnArgs A) {
   // is what lets them be quantized and stored by those workgroups themselves (below) instead of by a launch of
   // their own.
   const int ntiles = (maxlen + 31) >> 5;
-  // The window split takes an even share of the cached context as well, less kWindowCost tiles for the quantization it
-  // does first: every workgroup of the launch then finishes at about the same time (with the window tiles alone, 12 of
-  // the 252 workgroups of a 64-row pass were idle after two tiles and the others walked 51 tiles instead of 49).
-  constexpr int kWindowCost = 3;
+  // The window split takes an even share of the cached context as well, less window_cost tiles for the quantization it
+  // does first (measured: about the time of 7 tiles for 64 rows): every workgroup of the launch then finishes at about
+  // the same time (with the window tiles alone, 12 of the 252 workgroups of a 64-row pass were idle after two tiles and
+  // the others walked 51 tiles instead of 49).
+  const int kWindowCost = A.k16 ? 1 + A.M / 10 : 0;
   const int Tnew = min(ntiles, max(0, pos + A.tok0) >> 5);            // first tile that holds a row of this slice
   const int Tw = A.S > 1 ? min(Tnew, (A.S - 1) * ((ntiles + kWindowCost + A.S - 1) / A.S)) : Tnew;
   // A pass wider than one slice (a prefill chunk: its rows were appended by a launch of their own) has no window split:
