@@ -94,6 +94,21 @@ def test_merge_inside_the_launch_equals_second_launch(native, oracle, M, ctx, S)
             first = one
 
 
+@pytest.mark.parametrize("M,S", [(3, 1), (22, 5), (43, 7), (64, 21), (64, 32), (33, 13), (150, 3)])
+def test_wide_grid_layout_reaches_every_row_block_and_split(native, oracle, M, S):
+    """The wide kernel's one-dimensional grid is laid out for the round robin over the XCDs: whole (split, kv head) pairs
+    per XCD first, the leftover workgroups in order.  Split counts that leave leftovers (pairs x row blocks not a multiple
+    of 8) and counts that do not must both cover every (pair, row block) exactly once: any hole or double shows in the
+    output of the rows it belongs to."""
+    ctx = 2600
+    kv, oc, q, kn, vn = _fill(native, oracle, 530 + M + S, ctx, M, max_rows=max(M, 64))
+    with kv:
+        kv.set_opt(2, S)
+        out = kv.layer_call(0, q, kn, vn, ctx)
+        oc.append(kn, vn, ctx)
+        assert_attn_close(out, oc.attend_f32(q, ctx, threads=8, want_f32=True)[1], f"M={M} splits={S}")
+
+
 def test_depth_table(native, oracle):
     ctx, M = 700, 6
     kv, oc, q, kn, vn = _fill(native, oracle, 502, ctx, M)
@@ -299,3 +314,24 @@ def test_context_hint_only_sizes_the_grid(native, oracle, hint):
             oc.append(kn, vn, ctx)
             assert_attn_close(out, oc.attend_f32(q, ctx, threads=8, want_f32=True)[1], f"hint={hint} ctx={ctx} M={M}")
             _rows_equal(kv, oc, ctx, M)
+
+
+def test_machine_probe_figures_are_plausible(native):
+    """The in-library machine probe (fixed instruction mixes that time themselves): every kind runs, and what the waves
+    measured is in the range this architecture can produce (an MFMA 32x32x16 takes 8 passes of 4 cycles)."""
+    it = 500
+    r = native.machine_probe(0, 0, it, 256, 256)
+    assert 31.0 < r["cycles"] / (it * 4) < 40.0 and 1000 < r["shader_mhz"] < 3000, r
+    r6 = native.machine_probe(0, 6, it, 256, 256)
+    assert r6["cycles"] >= r["cycles"]
+    for op in range(9):
+        v = native.machine_probe(2, op, it, 64, 256)
+        assert 1.0 < v["cycles"] / (it * 32) < 40.0, (op, v)
+    x = native.machine_probe(5, 1, it, 64, 512)
+    assert x["cycles"] > 0 and x["cycles_b"] > 0
+    assert native.machine_probe(1, 0, it, 64, 256)["cycles"] > 0
+    assert native.machine_probe(3, it, it, 64, 512)["cycles_b"] > 0
+    rd = native.machine_probe(4, 0, 64, 1024, 256)
+    assert 64 * 1048576 / (rd["ms"] * 1e-3) / 1e9 > 100.0          # GB/s: a 64 MiB read, mostly from cache
+    with pytest.raises(native.YkaError):
+        native.machine_probe(9, 0, it, 64, 256)
