@@ -117,8 +117,10 @@ YKA_API int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, cons
  * once per device when a handle is opened there.  Limits: head_dim 128 handles, 1 <= M <= 64 rows (one slice), at most
  * 24 query heads; anything else returns -1 with a message.  The call allocates nothing, frees nothing, synchronises
  * nothing.  Every call on one GPU uses that GPU's one array: calls that overlap on a GPU (two streams, two handles) race
- * on it; calls on one stream, or otherwise ordered, are safe.  Nothing in the array has to start at zero: every launch
- * writes every partial it later reads. */
+ * on it; calls on one stream, or otherwise ordered, are safe.  No partial has to start at zero: every launch writes
+ * every partial it later reads.  The last kilobyte holds the split tickets option key 7 uses: zero when the library is
+ * loaded, and put back to zero by the workgroup that draws a column's last ticket, so every launch finds them zero (a
+ * launch that was aborted half way would not: reload the library, or keep option key 7 off, after a GPU fault). */
 YKA_API int yka_append_attend_static(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16_t* d_k16,
                                      const uint16_t* d_v16, int M, const int* d_pos, const uint8_t* d_depth,
                                      uint16_t* d_out16, void* hip_stream);
