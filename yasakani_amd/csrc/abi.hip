@@ -35,6 +35,7 @@ struct yka_kv {
   int* d_pos = nullptr;            // position used by the host-pointer hooks
   hipStream_t stream = nullptr;    // stream of the host-pointer hooks
   int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0, opt_unrot = 0, opt_ctx_hint = 0, opt_profile_layer = 0, opt_merge_in_launch = 0;
+  int opt_mid_rows = 10, opt_splits_mid = 0;   // widest window the mid kernel takes (0: none; measured faster than the wide kernel up to 10 rows), its split count (0: automatic)
   // trellis-coded rows (set by yka_kv_set_profile; head_dim 256 only): rows as the reference lays them out, per layer
   // [K payload n_kv * max_ctx * stride][V payload][K scales n_kv * max_ctx fp32][V scales]
   struct Tb {
@@ -128,6 +129,16 @@ int wide_splits(const yka_kv* kv, int M, size_t ws_pairs = kWsPairs) {
   const int rows = kG * M, rpb = wide_rows_per_block(M), rb = (rows + rpb - 1) / rpb;
   const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
   int S = kv->opt_splits_wide > 0 ? kv->opt_splits_wide : std::min(256 / (kv->cfg.n_kv_heads * rb), ((ctx + 31) / 32) / 4);
+  S = std::max(1, std::min(kMaxSplits, S));
+  return std::min(S, std::max(1, (int)(ws_pairs / (size_t)M)));
+}
+
+// Mid kernel (windows of 3..16 tokens; wider ones as blocks of 16 tokens): one workgroup of 4 waves per CU, every wave
+// at least one tile.
+int mid_splits(const yka_kv* kv, int M, size_t ws_pairs = kWsPairs) {
+  const int nb = (M + 15) / 16;
+  const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
+  int S = kv->opt_splits_mid > 0 ? kv->opt_splits_mid : std::min(256 / (kv->cfg.n_kv_heads * nb), ((ctx + 31) / 32) / 4);
   S = std::max(1, std::min(kMaxSplits, S));
   return std::min(S, std::max(1, (int)(ws_pairs / (size_t)M)));
 }
@@ -259,13 +270,14 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
   for (int s0 = 0; s0 < M; s0 += slice) {
     const int Ms = std::min(slice, M - s0);
     const bool narrow = !chunk && (Ms <= 2 || kv->opt_force_narrow);
-    const int S = narrow ? narrow_splits(kv, Ms, W.pairs) : (chunk ? chunk_splits(kv, Ms, W.pairs) : wide_splits(kv, Ms, W.pairs));
+    const bool mid = !chunk && !narrow && Ms <= kv->opt_mid_rows;
+    const int S = narrow ? narrow_splits(kv, Ms, W.pairs) : mid ? mid_splits(kv, Ms, W.pairs) : (chunk ? chunk_splits(kv, Ms, W.pairs) : wide_splits(kv, Ms, W.pairs));
     AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * kD, d_pos, depth, Ms, s0, NH, S, wide_rows_per_block(Ms), W.pm, W.pl, W.pacc16,
                fuse_append ? k16 : nullptr, fuse_append ? v16 : nullptr};
     // option key 7, rows of at most 2 tokens: the last workgroup of each column merges the splits inside the attention launch
     const bool one_launch = narrow && mode == 0 && !kv->opt_unrot && kv->opt_merge_in_launch;
     if (one_launch) { A.tickets = W.tickets; A.out16 = out16 + (size_t)s0 * NH * kD; }
-    if (narrow) launch_attend_narrow(A, st); else launch_attend_wide(A, st);
+    if (narrow) launch_attend_narrow(A, st); else if (mid) launch_attend_mid(A, st); else launch_attend_wide(A, st);
     if (mode != 2 && !one_launch) launch_combine(CombineArgs{W.pm, W.pl, W.pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD, kv->opt_unrot}, st);
   }
 }
@@ -410,6 +422,8 @@ int yka_set_opt(yka_kv* kv, int key, int value) {
     case 5: if (value < 0) throw std::runtime_error("context hint must be >= 0"); kv->opt_ctx_hint = value; break;
     case 6: if (value < 0) throw std::runtime_error("profile layer must be >= 0"); kv->opt_profile_layer = value; break;
     case 7: kv->opt_merge_in_launch = value != 0; break;
+    case 8: if (value < 0 || value > kMaxSlice) throw std::runtime_error("widest window of the mid kernel must be in [0, 64]"); kv->opt_mid_rows = value; break;
+    case 9: if (value < 0 || value > kMaxSplits) throw std::runtime_error("splits must be in [0, 256]"); kv->opt_splits_mid = value; break;
     default: throw std::runtime_error("unknown option key");
   }
   YKA_CATCH_INT

@@ -124,7 +124,8 @@ void launch_tb_unpack(const uint8_t* blob, const int* grp, const int* pos, const
 // launchers (each checks nothing: the C layer validates shapes first)
 void launch_append(const AppendArgs&, hipStream_t);
 void launch_attend_narrow(const AttnArgs&, hipStream_t);   // 16-row tiles: 2 tokens x 6 heads per workgroup column
-void launch_attend_wide(const AttnArgs&, hipStream_t);     // 3..64 tokens
+void launch_attend_wide(const AttnArgs&, hipStream_t);     // 3..64 tokens, and prefill slices
+void launch_attend_mid(const AttnArgs&, hipStream_t);      // 3..16 tokens: a wave owns whole tiles, row tiles of 16 rows (wider: blocks of 16 tokens)
 void launch_combine(const CombineArgs&, hipStream_t);
 void launch_attn_post(const PostArgs&, hipStream_t);
 void launch_attn_post256(const PostArgs&, hipStream_t);    // the same step for 256-channel heads (attend256.hip)
