@@ -13,6 +13,7 @@ def _fill(native, oracle, seed, ctx, M, max_ctx=None, **kw):
     max_ctx = max_ctx or ((ctx + M + 255) // 256) * 256
     oc = oracle.Cache(max_ctx)
     kv = native.KvCache(max_ctx=max_ctx, **kw)
+    kv.set_opt(8, 16)              # every window of up to 16 rows through this kernel (by default the wide kernel takes over earlier)
     if ctx:
         oc.append(k, v, 0)
         kv.import_rows(0, 0, oc.kc[:, :ctx], oc.ks[:, :ctx], oc.vc[:, :ctx], oc.vs[:, :ctx])
@@ -109,6 +110,7 @@ def test_paged_is_bit_identical_to_contiguous(native, oracle):
     outs = []
     for paged in (False, True):
         with native.KvCache(max_ctx=2304, paged=paged) as kv:
+            kv.set_opt(8, 16)
             if paged:
                 kv.set_page_table(rng.permutation(9).astype(np.int32))
             kv.import_rows(0, 0, oc.kc[:, :ctx], oc.ks[:, :ctx], oc.vc[:, :ctx], oc.vs[:, :ctx])
@@ -144,6 +146,7 @@ def test_large_scores_raise_the_running_maximum(native, oracle):
     q = np.repeat(base, 6, axis=1).repeat(M, axis=0).astype(np.float16)       # aligned with the ramp direction
     oc = oracle.Cache(1280); oc.append(k[:ctx], v[:ctx], 0)
     with native.KvCache(max_ctx=1280) as kv:
+        kv.set_opt(8, 16)
         kv.import_rows(0, 0, oc.kc[:, :ctx], oc.ks[:, :ctx], oc.vc[:, :ctx], oc.vs[:, :ctx])
         out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx)
         oc.append(k[ctx:], v[ctx:], ctx)
