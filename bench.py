@@ -390,6 +390,8 @@ def main():
                     help="how the timed layer calls are issued: captured-pass replays, eager calls, or auto (eager for windows of 16+ rows)")
     ap.add_argument("--condition-ms", type=float, default=100.0,
                     help="untimed replays of the same workload before the warm-up steps, so that the timed steps run at sustained clocks")
+    ap.add_argument("--opt", action="append", default=[], metavar="KEY=VALUE",
+                    help="yka_set_opt on the headline handle before anything is timed (e.g. 8=16: windows of up to 16 rows on the mid kernel)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary decode / verify-16 / verify-32 lines")
     ap.add_argument("--batched-only", action="store_true",
@@ -427,6 +429,9 @@ def main():
     max_ctx = ((ctx + 64 + 255) // 256) * 256
     q, k, v = synth(2026, ctx, 64)
     kv = native.KvCache(n_layers=L, max_ctx=max_ctx, max_rows=64)
+    for kvp in args.opt:
+        key, val = kvp.split("=")
+        kv.set_opt(int(key), int(val))
     fill_cache(kv, k, v, ctx)
     layers = list(range(L))
     kn, vn = k[ctx:], v[ctx:]

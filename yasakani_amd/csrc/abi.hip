@@ -136,9 +136,9 @@ int wide_splits(const yka_kv* kv, int M, size_t ws_pairs = kWsPairs) {
 // Mid kernel (windows of 3..16 tokens; wider ones as blocks of 16 tokens): one workgroup of 4 waves per CU, every wave
 // at least one tile.
 int mid_splits(const yka_kv* kv, int M, size_t ws_pairs = kWsPairs) {
-  const int nb = (M + 15) / 16;
+  const int nb = (M + 15) / 16, wgs = 256;
   const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
-  int S = kv->opt_splits_mid > 0 ? kv->opt_splits_mid : std::min(256 / (kv->cfg.n_kv_heads * nb), ((ctx + 31) / 32) / 4);
+  int S = kv->opt_splits_mid > 0 ? kv->opt_splits_mid : std::min(wgs / (kv->cfg.n_kv_heads * nb), ((ctx + 31) / 32) / 4);
   S = std::max(1, std::min(kMaxSplits, S));
   return std::min(S, std::max(1, (int)(ws_pairs / (size_t)M)));
 }

@@ -43,6 +43,33 @@ constexpr int kAccPitch = kD + 4;              // floats per staged row of the w
 // the PV instructions read probabilities written a whole step earlier, operand_ready covers the one place where they
 // follow at once.  pv_done puts 16 idle slots between the last PV instruction and the epilogue's reads of a row tile's
 // accumulators (the compiler keeps 8).  Inside the loop an accumulator is next touched a whole tile later.
+// What a lane holds of a raw 32-key tile in this kernel.  The K group scales are those of the lane's OWN keys (16kt + i,
+// the rows of its K operand: 4 fp16 = one 8-byte load per key half), because here the scales go into the operand, not
+// onto the scores.  14 loads per tile.
+struct MidTile {
+  u32x4 kw[2];         // K codes: key 16*kt + i, dword m = channels 32m + 8g .. +7
+  u32x2 ksa[2];        // K scales of key 16*kt + i, groups 0..3
+  uint32_t vw[8];      // V codes: token tau(g, e), channels 8i .. +7
+  u32x2 vs[2];         // V scales, group i/4, tokens 16h + 4g .. +3
+};
+#define YKA_GL(width, dst, off, base, imm) asm volatile("global_load_" width " %0, %1, %2 offset:%3 nt" : "=v"(dst) : "v"(off), "s"(base), "n"(imm))
+__device__ __forceinline__ void load_mid_tile(const uint8_t* pg, int tp, const LaneOffs& L, uint32_t ksa_off, MidTile& R) {
+  const uint8_t* c64 = pg + (uint32_t)tp * 64u;     // code rows (K and V planes) of the tile
+  const uint8_t* s8 = pg + (uint32_t)tp * 8u;       // K scale rows
+  const uint8_t* s2 = pg + (uint32_t)tp * 2u;       // V scale columns
+  YKA_GL("dwordx4", R.kw[0], L.kc, c64, 0);      YKA_GL("dwordx4", R.kw[1], L.kc, c64, 1024);
+  YKA_GL("dwordx2", R.ksa[0], ksa_off, s8, 0);   YKA_GL("dwordx2", R.ksa[1], ksa_off, s8, 128);
+  YKA_GL("dwordx2", R.vs[0], L.vs, s2, 0);       YKA_GL("dwordx2", R.vs[1], L.vs, s2, 32);
+  YKA_GL("dword", R.vw[0], L.vc, c64, 0);    YKA_GL("dword", R.vw[1], L.vc, c64, 64);   YKA_GL("dword", R.vw[2], L.vc, c64, 128);  YKA_GL("dword", R.vw[3], L.vc, c64, 192);
+  YKA_GL("dword", R.vw[4], L.vc, c64, 1024); YKA_GL("dword", R.vw[5], L.vc, c64, 1088); YKA_GL("dword", R.vw[6], L.vc, c64, 1152); YKA_GL("dword", R.vw[7], L.vc, c64, 1216);
+}
+#undef YKA_GL
+__device__ __forceinline__ void wait_mid_tile(MidTile& R) {
+  asm volatile("s_waitcnt vmcnt(0)"
+               : "+v"(R.kw[0]), "+v"(R.kw[1]), "+v"(R.ksa[0]), "+v"(R.ksa[1]), "+v"(R.vs[0]), "+v"(R.vs[1]),
+                 "+v"(R.vw[0]), "+v"(R.vw[1]), "+v"(R.vw[2]), "+v"(R.vw[3]), "+v"(R.vw[4]), "+v"(R.vw[5]), "+v"(R.vw[6]), "+v"(R.vw[7]));
+}
+
 __device__ __forceinline__ void operand_ready(h8& p) {
   asm volatile("s_nop 2" : "+v"(p));
 }
@@ -55,6 +82,11 @@ __device__ __forceinline__ void pv_done(f4 (&o)[8]) {
 }  // namespace
 
 // grid (S, n_kv, row blocks), block 256.  Row R = 16 rt + i of a block is (token tokb + R / 6, head kvh * 6 + R % 6).
+// One wave per SIMD for every instantiation.  (Two waves per SIMD were tried for NRT = 2, whose registers nearly fit:
+// the compiler then spills under pressure, and what it spilled were the destination registers of tile loads still in
+// flight - copied to the accumulator file right behind the load instruction and reused as the next load's address.
+// The static check in tests/test_isa_inflight_loads.py reports exactly that; it has to pass before this file runs on
+// a GPU.)
 template <int NRT>
 __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
   constexpr int TB = (16 * NRT) / kG;          // tokens per row block
@@ -67,8 +99,20 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
   const int lane = tid & 63, i = lane & 15, g = lane >> 4;
   const int tokb = rb * TB, ntok = min(TB, A.M - tokb), nrows = kG * ntok;
 
-  // ---- one trip to memory: the position, the depth entries and the query rows (wave w stages scale group w of every
-  //      row tile).  Odd channels carry 1/16: the odd nibble of a byte dequantizes to 16 (n - 8). ----
+  // The tiles of a row block are dealt out to ALL waves of its workgroups round robin: wave gw = 4 split + wave takes the
+  // tiles gw, gw + W, gw + 2 W, ... (W = 4 S waves).  Which tile a wave starts with therefore does not depend on the
+  // position, and its loads go out before anything else: the position, the query rows and the first tile arrive in ONE
+  // trip to memory.  (The tile exists whatever the position is: it lies inside the container.  If it turns out to be
+  // beyond the keys this pass sees, or to hold rows this pass is about to store, what was loaded is dropped.)
+  const int W = 4 * A.S, gw = 4 * split + wave;
+  const LaneOffs offs = lane_offs(i, g);
+  const uint32_t ksa_off = kPageKs + 8u * i;       // K scales of key i of a key half: [token][4] fp16
+  auto request = [&](int T, MidTile& r) __attribute__((always_inline)) { load_mid_tile(kv_page_uniform(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, ksa_off, r); };
+  MidTile raw;
+  request(min(gw, A.kv.max_ctx / 32 - 1), raw);
+
+  // ---- the same trip: the position, the depth entries and the query rows (wave w stages scale group w of every
+  //      row tile) ----
   uint4 qraw[NRT];
   int dep[NRT];
 #pragma unroll
@@ -84,8 +128,7 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
 #pragma unroll
   for (int rt = 0; rt < NRT; ++rt) {
     const h8 c = __builtin_bit_cast(h8, qraw[rt]);
-    const _Float16 sx = (_Float16)0.0625f;
-    const h8 f = h8{c[0], c[4], c[1] * sx, c[5] * sx, c[2], c[6], c[3] * sx, c[7] * sx};
+    const h8 f = h8{c[0], c[4], c[1], c[5], c[2], c[6], c[3], c[7]};       // the element order the K dequantization produces
     s_q[(rt * 4 + wave) * 64 + lane] = __builtin_bit_cast(uint4, f);
   }
   int lenr[NRT];
@@ -100,31 +143,33 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
   for (int o = 1; o < 16; o <<= 1) { maxlen = max(maxlen, __shfl_xor(maxlen, o, 64)); minlen = min(minlen, __shfl_xor(minlen, o, 64)); }
   maxlen = __builtin_amdgcn_readfirstlane(maxlen); minlen = __builtin_amdgcn_readfirstlane(minlen);
 
-  // The grid is sized for the context the caller expects; how many of its splits the block uses follows from the length
-  // found on the device: at least four tiles (one per wave) per workgroup.  The tiles are cut evenly (sizes differ by
-  // at most one).  The other workgroups leave the "no keys" marker and exit.
+  // The grid is sized for the context the caller expects.  A workgroup none of whose waves has a tile (short contexts)
+  // leaves the "no keys" marker and exits; the others hold tile counts that differ by at most one.
   const int ntiles = (maxlen + 31) >> 5;
-  const int s_used = min(A.S, max(1, ntiles >> 2));
-  if (split >= s_used) {
+  auto owned = [&](int T) { return (T % W) >> 2 == split; };         // does a wave of this workgroup own tile T
+  if (4 * split >= ntiles) {
     if (tid < nrows) {
       const size_t p = ((size_t)(tokb + tid / kG) * A.S + split) * A.n_heads + kvh * kG + tid % kG;
       A.pm[p] = -1e30f; A.pl[p] = 0.f;
     }
+    wait_mid_tile(raw);                            // the loads are answered before their registers are given up
     return;
   }
-  const int tile0 = (int)(((long long)split * ntiles) / s_used), tile1 = (int)(((long long)(split + 1) * ntiles) / s_used);
 
   // ---- fused quantize-on-append.  A block reads rows of the pass up to its own last token; it stores those of them that
   //      lie in its tiles before it loads the tiles (writer and readers are waves of one CU and one write-through L1:
   //      workgroup-scope fences around the barrier).  Row blocks of one kv head write identical bytes.  A row no query
-  //      row can see (a depth table may say so) lies past the last tile when it opens a new one: the last split in use
-  //      of the last row block stores it. ----
+  //      row can see (a depth table may say so) lies past the last tile when it opens a new one: the workgroup of the
+  //      last row block that would own that tile stores it. ----
+  bool stale = false;                                          // this wave's first tile holds rows this workgroup stores below
   if (A.k16) {
     const int nvis = min(A.M, tokb + ntok);                    // rows of the slice this block may read
     const int nst = rb == (int)gridDim.z - 1 ? A.M : nvis;     // rows it stores if they are its own
     const int r_lo = pos + A.tok0, r_hi = r_lo + nst - 1;
-    const bool last = rb == (int)gridDim.z - 1 && split == s_used - 1;
-    const bool any_mine = ((r_hi >> 5) >= tile0 && (r_lo >> 5) < tile1) || (last && (r_hi >> 5) >= ntiles);   // uniform over the workgroup
+    const bool lastb = rb == (int)gridDim.z - 1;
+    bool any_mine = false;                                     // uniform over the workgroup; a slice spans at most 3 tiles
+    for (int T = r_lo >> 5; T <= r_hi >> 5; ++T) any_mine |= owned(T);
+    stale = any_mine && gw >= (r_lo >> 5) && gw <= (r_hi >> 5);
     if (any_mine) {
       const int c = tid & 15, slot = tid >> 4;                 // 16 lanes per 128-channel row, 16 rows (K and V of 8 tokens) per step
       for (int h0 = 0; h0 < 2 * nst; h0 += 32) {
@@ -138,8 +183,9 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
 #pragma unroll
         for (int it = 0; it < 2; ++it) {
           const int hh = h0 + it * 16 + slot, t = hh >> 1, r = pos + A.tok0 + t;
-          const bool held = (r >> 5) >= tile0 && (r >> 5) < tile1 && t < nvis, unseen = last && (r >> 5) >= ntiles;
-          if (t < nst && r >= 0 && r < A.kv.max_ctx && (held || unseen)) quant_store_chunk8(A.kv, kvh, r, hh & 1, rawv[it], c);
+          // rows this block may read; the last block also stores the rows nobody reads (past every visible tile)
+          const bool mine = owned(r >> 5) && (t < nvis || (lastb && (r >> 5) >= ntiles));
+          if (t < nst && r >= 0 && r < A.kv.max_ctx && mine) quant_store_chunk8(A.kv, kvh, r, hh & 1, rawv[it], c);
         }
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
@@ -151,7 +197,7 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
     __syncthreads();                             // the query fragments are in LDS
   }
 
-  const float sc_log2 = kLog2e / sqrtf((float)kD), inv_sc = sqrtf((float)kD) / kLog2e;
+  const float sc_log2 = kLog2e / sqrtf((float)kD);
   float m_run[NRT], l_run[NRT];
   f4 o[NRT][8];
 #pragma unroll
@@ -160,25 +206,43 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
 #pragma unroll
     for (int b = 0; b < 8; ++b) { o[rt][b] = f4{0.f, 0.f, 0.f, 0.f}; asm("" : "+a"(o[rt][b])); }
   }
-  const LaneOffs offs = lane_offs(i, g);
   uint32_t magic = kMagic;
   asm volatile("" : "+v"(magic));
 
   // one 32-key tile against every row tile of the block
-  auto tile = [&](const int T, RawTile& cur, auto&& request_next) __attribute__((always_inline)) {
+  auto tile = [&](const int T, MidTile& cur, auto&& request_next) __attribute__((always_inline)) {
     const int t0 = T << 5;
     const bool need_mask = t0 + 32 > minlen;     // uniform: only the last tiles hold keys past a row's length
     // ---- the tile's MFMA operands, once: K codes as exact integers (A operand of S^T = K Q^T: key 16kt + i, channels
     //      32m + 8g ..), V scaled (A operand of O^T += V^T P^T: channel 8i + b, tokens tau(g, .)) ----
-    h8 kf[2][4];
+    // K: code x scale, exact, as the sum of two fp16 images.  The fp16 group scale s (11 significant bits) is cut into
+    // hi = its upper 8 bits and lo = s - hi (3 bits): (n - 8) has 3 bits, so (n - 8) * hi and (n - 8) * lo are both
+    // exact in fp16 (lo's last bit is s's last bit: no underflow that s itself does not have), and the score MFMAs, which
+    // accumulate in fp32, add the two products of every channel without rounding either.  All eight MFMAs of a key half
+    // (4 groups x hi, lo) chain into ONE accumulator: a score leaves the matrix pipe finished but for the softmax scale -
+    // no multiply-add per score and scale group on the vector unit, a quarter of the partial-sum registers.
+    h8 kf[2][2][4];                              // [key half][hi | lo][scale group]
 #pragma unroll
-    for (int kt = 0; kt < 2; ++kt)
+    for (int kt = 0; kt < 2; ++kt) {
+      const uint32_t sw[2] = {cur.ksa[kt][0], cur.ksa[kt][1]};
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
-        h2 k4[4];
-        dq_dword_int(cur.kw[kt][m], k4, magic);
-        kf[kt][m] = h8{k4[0][0], k4[0][1], k4[1][0], k4[1][1], k4[2][0], k4[2][1], k4[3][0], k4[3][1]};
+        const uint32_t pair = sw[m >> 1];
+        const uint32_t hi_pair = pair & 0xfff8fff8u;
+        const h2 lo_pair = as_h2(pair) - as_h2(hi_pair);
+        const _Float16 sh = as_h2(hi_pair)[m & 1], sl = lo_pair[m & 1];
+        const h2 sh2 = {sh, sh}, sl2 = {sl, sl};
+        const h2 c1032 = {(_Float16)1032.f, (_Float16)1032.f};
+        const uint32_t w = cur.kw[kt][m];
+        // codes n0,n4 | n1,n5 | n2,n6 | n3,n7 as n - 8 (every nibble shifted down to bit 0 / 16: no factor 16 on the odd ones)
+        const h2 c0 = as_h2(nib(w, 0x000f000fu, magic)) - c1032, c1 = as_h2(nib(w >> 4, 0x000f000fu, magic)) - c1032;
+        const h2 c2 = as_h2(nib(w >> 8, 0x000f000fu, magic)) - c1032, c3 = as_h2(nib(w >> 12, 0x000f000fu, magic)) - c1032;
+        const h2 a0 = c0 * sh2, a1 = c1 * sh2, a2 = c2 * sh2, a3 = c3 * sh2;
+        const h2 b0 = c0 * sl2, b1 = c1 * sl2, b2 = c2 * sl2, b3 = c3 * sl2;
+        kf[kt][0][m] = h8{a0[0], a0[1], a1[0], a1[1], a2[0], a2[1], a3[0], a3[1]};
+        kf[kt][1][m] = h8{b0[0], b0[1], b1[0], b1[1], b2[0], b2[1], b3[0], b3[1]};
       }
+    }
     h8 vf[8];
     {
       h2 va[8][4];
@@ -199,22 +263,15 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
       for (int b = 0; b < 8; ++b)
         vf[b] = h8{va[b][0][0], va[b][0][1], va[b][1][0], va[b][1][1], va[b][2][0], va[b][2][1], va[b][3][0], va[b][3][1]};
     }
-    // K group scales of the lane's 8 keys (tau(g, e)): 16 words of two fp16 each, [key half][2 r + (groups 0,1 | 2,3)].
-    // They are COPIED out of the raw tile before the next tile is requested: nothing of the raw tile is live when its
-    // registers are loaded again, so the register set that is waited for at the top of the loop is the one the request
-    // writes (a value kept alive across the request would make the compiler move the whole set with copies placed in
-    // front of the wait, i.e. copies of registers whose loads are still in flight).
-    uint32_t ksw[2][8];
+    // Everything derived from the raw tile exists before the next tile is requested, and nothing of the raw tile is
+    // live when its registers are loaded again: the register set that is waited for at the top of the loop is then the
+    // one the request writes (a value kept alive across the request makes the compiler move the whole set with copies
+    // placed in front of the wait, i.e. copies of registers whose loads are still in flight; code sunk towards its first
+    // use does the same).
 #pragma unroll
     for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-      for (int w = 0; w < 8; ++w) {
-        const uint32_t x = cur.ks[kt][w >> 2][w & 3];
-        asm volatile("v_mov_b32 %0, %1" : "=v"(ksw[kt][w]) : "v"(x));
-      }
-    // everything derived from the raw tile exists before the request (nothing is sunk past it towards its first use)
-#pragma unroll
-    for (int kt = 0; kt < 2; ++kt) asm volatile("" : "+v"(kf[kt][0]), "+v"(kf[kt][1]), "+v"(kf[kt][2]), "+v"(kf[kt][3]));
+      for (int hl = 0; hl < 2; ++hl) asm volatile("" : "+v"(kf[kt][hl][0]), "+v"(kf[kt][hl][1]), "+v"(kf[kt][hl][2]), "+v"(kf[kt][hl][3]));
     asm volatile("" : "+v"(vf[0]), "+v"(vf[1]), "+v"(vf[2]), "+v"(vf[3]), "+v"(vf[4]), "+v"(vf[5]), "+v"(vf[6]), "+v"(vf[7]));
     __builtin_amdgcn_sched_barrier(0);
     request_next();                              // the raw registers are free: the next tile's loads run under the row tiles
@@ -226,17 +283,21 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
     //      which it waits for its own matrix results; here every MFMA result is consumed one step after it was asked for.
     //      Scheduling barriers keep the steps apart: the registers hold two sets of partial sums, not six. ----
     h8 qf[2][4];
-    f4 part[2][2][4];                            // [set][key half][scale group]
+    f4 part[2][2];                               // [set][key half]: finished dot products q . (code x scale)
     h8 pf[2];
     auto load_q = [&](int rt, h8 (&q)[4]) __attribute__((always_inline)) {
 #pragma unroll
       for (int m = 0; m < 4; ++m) q[m] = __builtin_bit_cast(h8, s_q[(rt * 4 + m) * 64 + lane]);
     };
-    auto scores = [&](const h8 (&q)[4], f4 (&pp)[2][4]) __attribute__((always_inline)) {
+    auto scores = [&](const h8 (&q)[4], f4 (&pp)[2]) __attribute__((always_inline)) {
+      pp[0] = f4{0.f, 0.f, 0.f, 0.f}; pp[1] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int kt = 0; kt < 2; ++kt)
+      for (int m = 0; m < 4; ++m)
 #pragma unroll
-        for (int m = 0; m < 4; ++m) pp[kt][m] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kt][m], q[m], f4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+        for (int hl = 0; hl < 2; ++hl)
+#pragma unroll
+          for (int kt = 0; kt < 2; ++kt)           // the two chains alternate: an MFMA never waits for the one before it
+            pp[kt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(kf[kt][hl][m], q[m], pp[kt], 0, 0, 0);
     };
     load_q(0, qf[0]);
     scores(qf[0], part[0]);
@@ -247,22 +308,14 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
       const int cs = rt & 1, ns = cs ^ 1;
       if (rt + 1 < NRT) scores(qf[ns], part[ns]);                  // asked for now, consumed in the next step
       if (rt + 2 < NRT) load_q(rt + 2, qf[cs]);                    // the fragments of row tile rt were last read one step ago
-      // part[cs][kt][m][r] = sum over group m of q * code for key t0 + 16kt + 4g + r and row i of row tile rt
+      // part[cs][kt][r] = q . k for key t0 + 16kt + 4g + r and row i of row tile rt
       const bool first = m_run[rt] < -1e29f;     // the row has seen no key yet
       const float msub = first ? 0.f : m_run[rt];
-      const float c0 = -msub * inv_sc;           // the chain of scale multiply-adds starts from minus the running maximum (raw units)
       float e[8];
 #pragma unroll
       for (int kt = 0; kt < 2; ++kt)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const h2 s01 = as_h2(ksw[kt][2 * r]), s23 = as_h2(ksw[kt][2 * r + 1]);
-          float dot = __builtin_fmaf(part[cs][kt][0][r], (float)s01[0], c0);
-          dot = __builtin_fmaf(part[cs][kt][1][r], (float)s01[1], dot);
-          dot = __builtin_fmaf(part[cs][kt][2][r], (float)s23[0], dot);
-          dot = __builtin_fmaf(part[cs][kt][3][r], (float)s23[1], dot);
-          e[4 * kt + r] = dot * sc_log2;             // exponent of the probability, relative to the running maximum
-        }
+        for (int r = 0; r < 4; ++r) e[4 * kt + r] = __builtin_fmaf(part[cs][kt][r], sc_log2, -msub);   // exponent of the probability, relative to the running maximum
       if (need_mask) {
 #pragma unroll
         for (int k = 0; k < 8; ++k) { const int key = t0 + tau(g, k); e[k] = key < lenr[rt] ? e[k] : -INFINITY; }
@@ -311,20 +364,25 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
     __builtin_amdgcn_sched_barrier(0);
   };
 
-  // The wave's tiles are T0, T0 + 4, ...  One register set: the request for the next tile goes out as soon as the
+  // The wave's tiles are gw, gw + W, ...  One register set: the request for the next tile goes out as soon as the
   // current one has been turned into operands, and is in flight during the whole walk over the row tiles.  It is always
-  // issued (past the end: the current tile again) so that the number of loads in flight at the one wait site is static.
-  {
-    RawTile raw;
-    auto request = [&](int T, RawTile& r) __attribute__((always_inline)) { load_tile(kv_page_uniform(A.kv, kvh, T << 5), (T << 5) % kPageTok, offs, r); };
-    const int T0 = tile0 + wave;
-    if (T0 < tile1) {
-      request(T0, raw);
-      for (int T = T0; T < tile1; T += 4) {
-        wait_tile<0>(raw);
-        tile(T, raw, [&]() __attribute__((always_inline)) { request(T + 4 < tile1 ? T + 4 : T, raw); });
-      }
-      wait_tile<0>(raw);                         // the last request is answered before its registers are given up
+  // issued (past the end: the current tile again) so that the number of loads in flight at a wait is static.  The first
+  // tile was requested at the top of the kernel; a wave whose first tile holds rows that this workgroup has just stored
+  // asks for it again (short contexts only: the first W tiles).  Every value of the register set that reaches the loop
+  // has passed a wait.
+  wait_mid_tile(raw);
+  if (stale) {                                     // wave uniform
+    MidTile again;
+    request(gw, again);
+    wait_mid_tile(again);
+    raw = again;
+  }
+  if (gw < ntiles) {
+    for (int T = gw;;) {
+      tile(T, raw, [&]() __attribute__((always_inline)) { request(T + W < ntiles ? T + W : T, raw); });
+      wait_mid_tile(raw);
+      T += W;
+      if (T >= ntiles) break;
     }
   }
 #pragma unroll
