@@ -8,10 +8,13 @@ absolute bar is taken against the oracle's fp32 result rounded to fp16: what the
     short contexts reach (a row dominated by one V row): there the bar is 2e-3 * |ref| - the "scaled" bar, counted and
     reported separately;
   * relative L2 is always taken against the unrounded fp32 result.
-Between 2 and 4 the plain bar is exactly one fp16 spacing (2^-9 = 1.95e-3).  A row that one key dominates returns that
-key's V row, which the kernels hold as fp16(code * scale) - up to half a spacing off the exact product - before the
-output is rounded again: two spacings (3.9e-3) are possible there.  The committed cases do not hit it; a randomized sweep
-of 300 shapes found one such value (a 1025-row chunk on 64 cached tokens, a row near the start of the chunk).
+Between 2 and 4 the plain bar is exactly one fp16 spacing (2^-9 = 1.95e-3).  The kernels hold V as fp16(code * scale),
+up to half a spacing OF THE VALUE'S OWN BINADE off the exact product; a row made of a few keys whose V values lie in
+[4, 8) but whose output lies in [2, 4) carries up to one output spacing of such error before the output itself is
+rounded, and lands two spacings (3.9e-3) from the oracle's rounded value when the oracle's fp32 result sits next to a
+rounding boundary.  This EXCEEDS the plain 2e-3 bar.  It needs very short contexts (a row of a handful of keys); two
+shapes of a randomized sweep hit it (tests/test_gpu_sweep.py keeps both), each in one output value.  Those tests, and only
+those, use `two_spacings=True`: values with |ref| in [2, 4] may be two fp16 spacings off, everything else as above.
 """
 import numpy as np
 
@@ -41,7 +44,15 @@ def attn_report(out, ref):
     return plain, scaled, rl, int((~small).sum())
 
 
-def assert_attn_close(out, ref, what=""):
+def assert_attn_close(out, ref, what="", two_spacings=False):
+    if two_spacings:
+        a = np.asarray(out, np.float64)
+        b = np.asarray(ref, np.float64)
+        b16 = np.asarray(ref, np.float32).astype(np.float16).astype(np.float64)
+        mid = (np.abs(b) >= 2.0) & (np.abs(b) <= PLAIN_UP_TO)
+        d = np.abs(a - b16)
+        assert not mid.any() or d[mid].max() <= 2 * 2.0 ** -9, f"{what}: {d[mid].max():.3e} on a value in [2, 4]: more than two fp16 spacings"
+        out = np.where(mid, b16, a)              # the rest of the comparison runs with those values taken as met
     plain, scaled, rl, n_big = attn_report(out, ref)
     assert plain <= MAX_ABS and scaled <= MAX_ABS and rl <= REL_L2, (
         f"{what}: max-abs {plain:.3e} (plain bar {MAX_ABS}, |ref| <= {PLAIN_UP_TO}), scaled max-abs {scaled:.3e} over {n_big} "
