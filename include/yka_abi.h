@@ -76,7 +76,18 @@ YKA_API const char* yka_build_info(void);
  *        splits inside the attention launch: the workgroup that finishes a column last combines it.  0 (default) = a
  *        second launch combines.  Same results to within the summation order.  On MI355X the second launch is the faster
  *        form (12.0 against 18.9 us per layer call at 32k tokens): the hand-over between XCDs costs three dependent
- *        trips to memory (store acknowledged, ticket, loads), more than the gap between two kernels. */
+ *        trips to memory (store acknowledged, ticket, loads), more than the gap between two kernels;
+ * key 8: widest window (rows) that runs on the kernel for small windows (a wave owns whole tiles and walks the window's row
+ *        tiles; 128-channel rows only).  0 = never, at most 64 (wider windows than 16 rows then run as blocks of 16
+ *        tokens).  Default 10: measured faster than the 128-row workgroups of the wide kernel up to there;
+ * key 9: split count of that kernel (0 = automatic);
+ * key 10: tokens per prefill slice (passes wider than 64 rows), 0 = 1024; 128 .. 4096;
+ * key 11: 16-bit row type at the boundary: 0 = fp16 (default), 1 = bf16, the type of the reference's activations
+ *        (q35_kernels.cu:1048,1062: Q, gate and attention outputs are bf16 there).  With 1, d_q16 / d_k16 / d_v16 of every
+ *        entry point are bf16 and are converted to fp16 by one extra launch per call (round to nearest; exact for
+ *        magnitudes between 2^-14 and 65504, i.e. for normalised activations), attention outputs are rounded once from
+ *        their fp32 value to bf16, and yka_attn_post writes q16 / gate16 as bf16.  Setting it to 1 the first time reserves
+ *        the staging rows (max_rows of Q, K and V): do that before capturing passes; the call is not on the launch path. */
 YKA_API int yka_set_opt(yka_kv* kv, int key, int value);
 
 /* Paged mode: logical page p of `layer` (-1 = every layer) lives in physical page h_table[p]; n_pages = max_ctx/256
@@ -103,8 +114,9 @@ YKA_API int yka_attend(yka_kv* kv, int layer, const uint16_t* d_q16, int M, cons
 /* One layer call = the effect of yka_append followed by yka_attend on the same stream: the sequence of
  * Engine35::attn_block (engine35.cpp:911-934).  The rows are quantized inside the attention launches (each 64-row
  * slice stores its own rows before it reads them; bit-identical to yka_append), so a layer call is two launches:
- * attention and the split combiner.  M may be as large as max_rows; passes wider than 64 rows are cut into 64-row
- * slices inside, as attn_block does (engine35.cpp:935-947). */
+ * attention and the split combiner.  M may be as large as max_rows; a pass wider than 64 rows is a prefill chunk: its rows
+ * are appended by one launch, then slices of up to 1024 tokens (option key 10) run through the wide kernel, one attention
+ * and one combiner launch per slice (attn_block cuts such passes into 64-row slices, engine35.cpp:935-947). */
 YKA_API int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16_t* d_k16,
                               const uint16_t* d_v16, int M, const int* d_pos, const uint8_t* d_depth,
                               uint16_t* d_out16, void* hip_stream);
@@ -183,6 +195,10 @@ typedef struct yka_post_params {
   int32_t rope_dims;         /* even, 0..head_dim; 0 = no rotary step (the reference rotates 64 of 256 channels, q35.hpp:13) */
   int32_t rope_rows;         /* rows whose position is not below rope_rows are dropped */
   int32_t rotate;            /* 0 / 1 */
+  const float* d_xgate;      /* the gate half of the Q projection, [M][n_heads][head_dim] fp32, or NULL (the reference's Q
+                              * projection carries query and gate side by side, q35_kernels.cu:1017,1048) */
+  uint16_t* d_gate16;        /* [M][n_heads][head_dim]: the gate rows rounded to the handle's 16-bit row type, the operand
+                              * yka_attn_out256 later takes (q35_kernels.cu:1048); NULL together with d_xgate */
 } yka_post_params;
 YKA_API int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float* d_xk, const float* d_xv, int M,
                           const int* d_pos, const yka_post_params* params, uint16_t* d_q16, void* hip_stream);
@@ -202,10 +218,11 @@ YKA_API int yka_attn_out256_lo_host(const uint16_t* y16, const uint16_t* gate16,
 YKA_API int yka_append256_f32_host(yka_kv* kv, int layer, const float* k32, const float* v32, int M, int pos, int rotate);
 YKA_API int yka_rotate_q256_host(const float* x32, int rows, uint16_t* q16);
 
-/* Host-pointer form of yka_attn_post: uploads everything, sets the device position to `pos`, runs, downloads q16. */
+/* Host-pointer form of yka_attn_post: uploads everything, sets the device position to `pos`, runs, downloads q16 (and
+ * gate16 if xgate / gate16 are given; both NULL = no gate rows). */
 YKA_API int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, const float* xv, int M, int pos,
                                const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope,
-                               int rope_dims, int rope_rows, int rotate, uint16_t* q16);
+                               int rope_dims, int rope_rows, int rotate, uint16_t* q16, const float* xgate, uint16_t* gate16);
 
 /* Codec round trip on the GPU, replaces yskn_kvx_probe (kvx_probe.cu:22-36): x16 [rows][128] fp16 ->
  * codes [rows][64], scales [rows][4] fp16, y [rows][128] fp32 dequantized. */

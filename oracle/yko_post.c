@@ -11,7 +11,8 @@
  *                  d <  rd/2: f16( f16(xn[d] * cos) + f16(-xn[d + rd/2] * sin) )
  *                  d >= rd/2: f16( f16(xn[d] * cos) + f16( xn[d - rd/2] * sin) )   with (cos, sin) of channel d - rd/2
  *                then [rotation] -> fp16
- * Two deliberate differences from the reference's kernel (so this restates its algorithm, not its bit pattern; parity
+ * Two deliberate differences from the reference's kernel in this 128-channel form (the 256-channel form further down
+ * follows the reference's order exactly) (so this restates its algorithm, not its bit pattern; parity
  * with the reference's own outputs for this step is UNPINNED - its rsqrtf puts bit equality out of reach anyway - and
  * the functions here are pinned by the independent fp64 / closed-form checks of tests/test_oracle_post.py): the
  * reference rounds the projected value to its 16-bit type first (y = rbf(buf[tid]), :1030) and uses that everywhere,
@@ -110,28 +111,33 @@ void yko_unrotate_out(const float* y32, int rows, uint16_t* out16) {
   }
 }
 
-/* ---- the same step for 256-channel heads (the reference's own head size, src/q35_kernels.cu:1037-1065) ----
- * Q and K: ss = sum y^2 - inside each quarter of 64 channels the butterfly a[i] += a[i ^ o], o = 32 .. 1, then
- * ((q0 + q1) + q2) + q3; r = 1 / sqrt(ss / 256 + eps); xn = f16(y * r * (1 + w[d])); rotary on the first rd channels as
- * above; then [the 256-point signed rotation x 1/16, yko_kvx_rotate256].  Q rows leave as fp16.  K rows (and V rows,
- * which skip normalisation and the rotary step) leave as the fp32 values the row quantizer (yko_flat4_encode256) takes:
- * fp16-valued when the rotation is off, the rotation's fp32 result when it is on. */
+/* ---- the same step for 256-channel heads (the reference's own head size, src/q35_kernels.cu:1030-1065) ----
+ * In the reference's own order of operations (only its 16-bit type, bf16 there and fp16 here, and its approximate
+ * reciprocal square root differ):
+ *   y = f16(projected value) first, for Q, K, V and gate rows alike (:1030); gate rows leave as that value (:1048);
+ *   Q and K: ss = sum y^2 - inside each run of 32 channels the butterfly a[i] += a[i ^ o], o = 16 .. 1 (:1051), then the
+ *   8 run sums folded in sequence from 0 (:1055-1056); r = 1 / sqrt(ss / 256 + eps); xn = f16(y * r * (1 + w[d]));
+ *   rotary on the first rd channels as above; then [the 256-point signed rotation x 1/16, yko_kvx_rotate256].
+ * Q rows leave as fp16.  K rows (and V rows, which skip normalisation and the rotary step) leave as the fp32 values the
+ * row quantizer (yko_flat4_encode256) takes: fp16-valued when the rotation is off, the rotation's fp32 result when on. */
 static float sumsq256(const float* y) {
-  float q[4];
-  for (int w = 0; w < 4; ++w) {
-    float a[64], b[64];
-    for (int i = 0; i < 64; ++i) a[i] = y[64 * w + i] * y[64 * w + i];
-    for (int o = 32; o; o >>= 1) {
-      for (int i = 0; i < 64; ++i) b[i] = a[i] + a[i ^ o];
+  float tot = 0.f;
+  for (int w = 0; w < 8; ++w) {
+    float a[32], b[32];
+    for (int i = 0; i < 32; ++i) a[i] = y[32 * w + i] * y[32 * w + i];
+    for (int o = 16; o; o >>= 1) {
+      for (int i = 0; i < 32; ++i) b[i] = a[i] + a[i ^ o];
       memcpy(a, b, sizeof a);
     }
-    q[w] = a[0];
+    tot = tot + a[0];
   }
-  return ((q[0] + q[1]) + q[2]) + q[3];
+  return tot;
 }
 
 /* one Q or K head row: y[256] -> o32[256] (before the final rounding of Q rows / the row quantizer of K rows) */
-void yko_post256_qk_row(const float* y, const uint16_t* w16, float eps, const float* cs, int rd, int rot, float* o32) {
+void yko_post256_qk_row(const float* yin, const uint16_t* w16, float eps, const float* cs, int rd, int rot, float* o32) {
+  float y[256];
+  for (int d = 0; d < 256; ++d) y[d] = f16r(yin[d]);
   const float tot = sumsq256(y);
   const float r = 1.f / sqrtf(tot / 256.f + eps);
   float xn[256], o[256];
@@ -159,7 +165,8 @@ void yko_attn_post256(const float* xq, const float* xk, const float* xv, int M, 
     }
     for (int h = 0; h < n_kv; ++h) {
       yko_post256_qk_row(xk + ((size_t)t * n_kv + h) * 256, kn_w16, eps, cs, rd, rot, k32 + ((size_t)t * n_kv + h) * 256);
-      const float* y = xv + ((size_t)t * n_kv + h) * 256;
+      float y[256];
+      for (int d = 0; d < 256; ++d) y[d] = f16r(xv[((size_t)t * n_kv + h) * 256 + d]);
       float* o = v32 + ((size_t)t * n_kv + h) * 256;
       if (rot) yko_kvx_rotate256(y, o, 0); else memcpy(o, y, 256 * sizeof(float));
     }

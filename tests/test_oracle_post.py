@@ -133,26 +133,28 @@ def test_post256_rows_match_fp64_forms_and_rotation():
     kw = (rng.standard_normal(256) * 0.1).astype(np.float16).view(np.uint16)
     rope = yko.rope_table(32, rd)
     q16, k32, v32 = yko.attn_post256(xq, xk, xv, qw, kw, 1e-6, rope, rd, pos, rot=0)
+    # the projected value is rounded to the 16-bit type before anything else (src/q35_kernels.cu:1030)
+    r16 = lambda a: a.astype(np.float16).astype(np.float32)
     for t in range(M):
         cs = rope[pos + t].astype(np.float64)
         for h in range(H):
-            ref = _post_numpy_d(xq[t, h], qw, 1e-6, cs, rd)
+            ref = _post_numpy_d(r16(xq[t, h]), qw, 1e-6, cs, rd)
             assert np.abs(_h(q16[t, h]) - ref).max() <= 2.5e-3 * max(1.0, np.abs(ref).max())
         for h in range(KVH):
-            ref = _post_numpy_d(xk[t, h], kw, 1e-6, cs, rd)
+            ref = _post_numpy_d(r16(xk[t, h]), kw, 1e-6, cs, rd)
             assert np.abs(k32[t, h] - ref).max() <= 2.5e-3 * max(1.0, np.abs(ref).max())
-    # K rows without rotation are fp16 valued; V rows pass through untouched
+    # K rows without rotation are fp16 valued; V rows are the rounded projection
     assert np.array_equal(k32, k32.astype(np.float16).astype(np.float32))
-    assert np.array_equal(v32, xv)
-    # channels past rd carry no rotary change: one rounding only
-    ref = _post_numpy_d(xq[0, 0], qw, 1e-6, rope[pos].astype(np.float64), rd)
-    assert np.array_equal(q16[0, 0, rd:], ref[rd:].astype(np.float16).view(np.uint16))
+    assert np.array_equal(v32, r16(xv))
+    # channels past rd carry no rotary change: one more rounding only
+    ref = _post_numpy_d(r16(xq[0, 0]), qw, 1e-6, rope[pos].astype(np.float64), rd)
+    assert np.abs(_h(q16[0, 0, rd:]) - ref[rd:]).max() <= 1.0e-3 * max(1.0, np.abs(ref).max())
     # with the rotation on: exactly the pinned 256-point rotation of the un-rotated rows (Q rounded to fp16 after it)
     q16r, k32r, v32r = yko.attn_post256(xq, xk, xv, qw, kw, 1e-6, rope, rd, pos, rot=1)
     qf = q16.view(np.float16).astype(np.float32).reshape(-1, 256)
     assert np.array_equal(q16r.reshape(-1, 256), yko.kvx_rotate256(qf).astype(np.float16).view(np.uint16))
     assert np.array_equal(k32r.reshape(-1, 256), yko.kvx_rotate256(k32.reshape(-1, 256)))
-    assert np.array_equal(v32r.reshape(-1, 256), yko.kvx_rotate256(xv.reshape(-1, 256)))
+    assert np.array_equal(v32r.reshape(-1, 256), yko.kvx_rotate256(r16(xv).reshape(-1, 256)))
 
 
 def test_post256_structure():
@@ -170,8 +172,34 @@ def test_post256_structure():
     assert np.array_equal(a[rd:], b[rd:]) and not np.array_equal(a[:rd], b[:rd])
     qc, _, _ = yko.attn_post256(x * 4, x[:, :1], x[:, :1], zero_w, zero_w, 0.0, rope, rd, 7, 0)
     assert np.array_equal(qb, qc)                                            # power-of-two scale invariance: exact
-    # the sum of squares is exact on small integers whatever the order: r = 1 / sqrt(ss / 256)
+    # the sum of squares is exact on small integers whatever the order (so the order of the reference, 32-channel runs
+    # folded in sequence, src/q35_kernels.cu:1051-1056, cannot show here): r = 1 / sqrt(ss / 256)
     xi = rng.integers(-3, 4, size=(1, 1, 256)).astype(np.float32)
     qi, _, _ = yko.attn_post256(xi, xi[:, :1], xi[:, :1], zero_w, zero_w, 0.0, rope, 0, 0, 0)
     r = np.float32(1.0) / np.sqrt(np.float32((xi.astype(np.float64) ** 2).sum() / 256.0))
     assert np.array_equal(qi[0, 0], (xi[0, 0] * r).astype(np.float16).view(np.uint16))
+
+
+def test_post256_sum_of_squares_follows_the_reference_order():
+    """ss = the 8 sums of 32-channel runs (each a butterfly a[i] += a[i ^ o], o = 16 .. 1) folded in sequence from 0
+    (src/q35_kernels.cu:1050-1056).  With one large square per run and tiny ones beside it the fp32 result depends on
+    the association; the row's normalisation factor must be the one this order gives."""
+    rng = np.random.default_rng(15)
+    zero_w = np.zeros(256, np.uint16)
+    rope = yko.rope_table(4, 0) if False else np.zeros((1, 1, 2), np.float32)
+    for trial in range(20):
+        x = (rng.standard_normal(256) * 10.0 ** rng.integers(-3, 3, size=256)).astype(np.float16).astype(np.float32)
+        sq = (x * x).astype(np.float32)
+        runs = []
+        for w in range(8):
+            a = sq[32 * w:32 * w + 32].copy()
+            for o in (16, 8, 4, 2, 1):
+                a = (a + a[np.arange(32) ^ o]).astype(np.float32)
+            runs.append(a[0])
+        tot = np.float32(0.0)
+        for r_ in runs:
+            tot = np.float32(tot + r_)
+        r = np.float32(1.0) / np.sqrt(np.float32(tot / np.float32(256.0)))
+        q16, _, _ = yko.attn_post256(x.reshape(1, 1, 256), x.reshape(1, 1, 256), x.reshape(1, 1, 256), zero_w, zero_w, 0.0, rope, 0, 0, 0)
+        expect = (x * r).astype(np.float32).astype(np.float16).view(np.uint16)
+        assert np.array_equal(q16[0, 0], expect), trial

@@ -35,6 +35,9 @@ struct yka_kv {
   int* d_pos = nullptr;            // position used by the host-pointer hooks
   hipStream_t stream = nullptr;    // stream of the host-pointer hooks
   int opt_splits_narrow = 0, opt_splits_wide = 0, opt_force_narrow = 0, opt_unrot = 0, opt_ctx_hint = 0, opt_profile_layer = 0, opt_merge_in_launch = 0;
+  int opt_chunk_slice = 0;                     // tokens per prefill slice (0: kChunkSlice)
+  int opt_io_bf16 = 0;                         // 16-bit rows at the boundary (Q, new K / V, gate, outputs) are bf16, not fp16
+  uint16_t *stage_q = nullptr, *stage_k = nullptr, *stage_v = nullptr;   // fp16 images of bf16 inputs (allocated when option key 11 is set)
   int opt_mid_rows = 10, opt_splits_mid = 0;   // widest window the mid kernel takes (0: none; measured faster than the wide kernel up to 10 rows), its split count (0: automatic)
   // trellis-coded rows (set by yka_kv_set_profile; head_dim 256 only): rows as the reference lays them out, per layer
   // [K payload n_kv * max_ctx * stride][V payload][K scales n_kv * max_ctx fp32][V scales]
@@ -200,7 +203,19 @@ void no_trellis(const yka_kv* kv) {
   if (kv->tb) throw std::runtime_error("this entry point does not work on trellis-coded rows");
 }
 
+// bf16 rows at the boundary: one launch turns the pass's Q / new K / new V rows into the fp16 rows the kernels read
+// (either group may be absent); outputs are written as bf16 by the combiners themselves.
+void rows_to_f16(yka_kv* kv, const uint16_t*& q16, const uint16_t*& k16, const uint16_t*& v16, int M, hipStream_t st) {
+  if (!kv->opt_io_bf16) return;
+  if (M < 1 || M > kv->cfg.max_rows) throw std::runtime_error("bf16 rows: the staging rows hold max_rows rows per pass");
+  const size_t nq = (size_t)M * kv->cfg.n_heads * kv->D(), nk = (size_t)M * kv->cfg.n_kv_heads * kv->D();
+  launch_bf16_to_f16(q16, kv->stage_q, q16 ? nq : 0, k16, kv->stage_k, v16, kv->stage_v, nk, st);
+  if (q16) q16 = kv->stage_q;
+  if (k16) { k16 = kv->stage_k; v16 = kv->stage_v; }
+}
+
 void do_append(yka_kv* kv, int layer, const uint16_t* k16, const uint16_t* v16, int M, const int* d_pos, hipStream_t st) {
+  { const uint16_t* none = nullptr; rows_to_f16(kv, none, k16, v16, M, st); }
   if (kv->tb) tb_append(kv, layer, nullptr, nullptr, k16, v16, M, d_pos, 0, st);
   else if (kv->r256()) launch_append256(AppendArgs{kv->view(layer), k16, v16, d_pos, M}, st);
   else launch_append(AppendArgs{kv->view(layer), k16, v16, d_pos, M}, st);
@@ -216,6 +231,10 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
                hipStream_t st, int mode = 0, const uint16_t* k16 = nullptr, const uint16_t* v16 = nullptr, const Workspace* ws = nullptr) {
   const int NH = kv->cfg.n_heads;
   const Workspace W = ws ? *ws : Workspace{kv->pm, kv->pl, kv->pacc16, kWsPairs, kv->tickets};
+  rows_to_f16(kv, q16, k16, v16, M, st);
+  const int io_was = kv->opt_io_bf16;
+  struct Restore { yka_kv* kv; int v; ~Restore() { kv->opt_io_bf16 = v; } } restore{kv, io_was};
+  kv->opt_io_bf16 = 0;                             // the rows are fp16 from here on (nested do_append calls must not convert again)
   if (kv->tb) {
     // trellis-coded rows: the encoder runs first (two launches); rows of at most 2 tokens (or option key 3) run on row
     // tiles of 2 tokens x 6 heads, wider slices on 128-row workgroups that decode every tile once into LDS
@@ -233,7 +252,7 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
                          T.pairs, T.gfac, T.has_mu ? T.mu : nullptr, layer, q16 + (size_t)s0 * NH * 256, d_pos, depth, Ms, s0, NH, S,
                          kv->pm, kv->pl, kv->pacc16};
       if (narrow) launch_attend_tb(A, T.kb, st); else launch_attend_tb_wide(A, T.kb, st);
-      if (mode != 2) launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, kv->opt_unrot}, st);
+      if (mode != 2) launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, kv->opt_unrot, io_was}, st);
     }
     return;
   }
@@ -252,7 +271,7 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
       AttnArgs A{kv->view(layer), q16 + (size_t)s0 * NH * 256, d_pos, depth, Ms, s0, NH, S, 0, kv->pm, kv->pl, kv->pacc16,
                  fuse256 ? k16 : nullptr, fuse256 ? v16 : nullptr};
       if (narrow) launch_attend256(A, st); else launch_attend256_wide(A, st);
-      if (mode != 2) launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, kv->opt_unrot}, st);
+      if (mode != 2) launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, kv->opt_unrot, io_was}, st);
     }
     return;
   }
@@ -266,7 +285,7 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
   const bool chunk = M > kMaxSlice && !kv->opt_force_narrow && !ws;
   const bool fuse_append = k16 && !chunk && (M <= 2 || !kv->opt_force_narrow);
   if (k16 && !fuse_append) do_append(kv, layer, k16, v16, M, d_pos, st);
-  const int slice = chunk ? kChunkSlice : kMaxSlice;
+  const int slice = chunk ? (kv->opt_chunk_slice > 0 ? kv->opt_chunk_slice : kChunkSlice) : kMaxSlice;
   for (int s0 = 0; s0 < M; s0 += slice) {
     const int Ms = std::min(slice, M - s0);
     const bool narrow = !chunk && (Ms <= 2 || kv->opt_force_narrow);
@@ -276,9 +295,9 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
                fuse_append ? k16 : nullptr, fuse_append ? v16 : nullptr};
     // option key 7, rows of at most 2 tokens: the last workgroup of each column merges the splits inside the attention launch
     const bool one_launch = narrow && mode == 0 && !kv->opt_unrot && kv->opt_merge_in_launch;
-    if (one_launch) { A.tickets = W.tickets; A.out16 = out16 + (size_t)s0 * NH * kD; }
+    if (one_launch) { A.tickets = W.tickets; A.out16 = out16 + (size_t)s0 * NH * kD; A.out_bf16 = io_was; }
     if (narrow) launch_attend_narrow(A, st); else if (mid) launch_attend_mid(A, st); else launch_attend_wide(A, st);
-    if (mode != 2 && !one_launch) launch_combine(CombineArgs{W.pm, W.pl, W.pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD, kv->opt_unrot}, st);
+    if (mode != 2 && !one_launch) launch_combine(CombineArgs{W.pm, W.pl, W.pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD, kv->opt_unrot, io_was}, st);
   }
 }
 
@@ -288,6 +307,8 @@ void do_attend_ms(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const ui
                   const int* row_slot, uint16_t* out16, hipStream_t st) {
   const int NH = kv->cfg.n_heads, D = kv->D();
   const bool r256 = kv->r256();
+  rows_to_f16(kv, q16, k16, v16, M, st);
+  const int io_was = kv->opt_io_bf16;
   if (kv->tb) {
     // trellis-coded rows: every container is a stream of the layer option key 6 names; its groups code and decode the rows
     const yka_kv::Tb& T = *kv->tb;
@@ -304,7 +325,7 @@ void do_attend_ms(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const ui
                          T.pairs, T.gfac, T.has_mu ? T.mu : nullptr, pl, q16 + (size_t)s0 * NH * 256, nullptr, nullptr, Ms, s0, NH, S,
                          kv->pm, kv->pl, kv->pacc16, Rs};
       launch_attend_tb(A, T.kb, st);
-      launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, kv->opt_unrot}, st);
+      launch_combine256(CombineArgs{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * 256, kv->opt_unrot, io_was}, st);
     }
     return;
   }
@@ -316,9 +337,9 @@ void do_attend_ms(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const ui
     S = std::min(std::max(2, std::min(kMaxSplits, S)), (int)(kWsPairs / (size_t)Ms));
     RowMap Rs = R; Rs.pos += s0; Rs.slot += s0;
     AttnArgs A{kv->view(0), q16 + (size_t)s0 * NH * D, nullptr, nullptr, Ms, s0, NH, S, 128, kv->pm, kv->pl, kv->pacc16, nullptr, nullptr, Rs};
-    const CombineArgs C{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * D, kv->opt_unrot};
+    const CombineArgs C{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * D, kv->opt_unrot, io_was};
     if (r256) { launch_attend256(A, st); launch_combine256(C, st); }
-    else if (!kv->opt_unrot && kv->opt_merge_in_launch) { A.tickets = kv->tickets; A.out16 = C.out16; launch_attend_narrow(A, st); }
+    else if (!kv->opt_unrot && kv->opt_merge_in_launch) { A.tickets = kv->tickets; A.out16 = C.out16; A.out_bf16 = io_was; launch_attend_narrow(A, st); }
     else { launch_attend_narrow(A, st); launch_combine(C, st); }
   }
 }
@@ -407,6 +428,7 @@ void yka_kv_close(yka_kv* kv) {
     (void)hipFree(kv->tb->scr); (void)hipFree(kv->tb->stage);
     delete kv->tb;
   }
+  (void)hipFree(kv->stage_q); (void)hipFree(kv->stage_k); (void)hipFree(kv->stage_v);
   (void)hipFree(kv->pool); (void)hipFree(kv->tables); (void)hipFree(kv->pm); (void)hipFree(kv->pl); (void)hipFree(kv->pacc16); (void)hipFree(kv->d_pos); (void)hipFree(kv->tickets);
   delete kv;
 }
@@ -424,6 +446,19 @@ int yka_set_opt(yka_kv* kv, int key, int value) {
     case 7: kv->opt_merge_in_launch = value != 0; break;
     case 8: if (value < 0 || value > kMaxSlice) throw std::runtime_error("widest window of the mid kernel must be in [0, 64]"); kv->opt_mid_rows = value; break;
     case 9: if (value < 0 || value > kMaxSplits) throw std::runtime_error("splits must be in [0, 256]"); kv->opt_splits_mid = value; break;
+    case 11: {
+      if (value != 0 && value != 1) throw std::runtime_error("row type must be 0 (fp16) or 1 (bf16)");
+      if (value && !kv->stage_q) {                 // not on the launch path: the staging rows are reserved here, once
+        HIPCHK(hipSetDevice(kv->cfg.device));
+        const size_t nq = (size_t)kv->cfg.max_rows * kv->cfg.n_heads * kv->D(), nk = (size_t)kv->cfg.max_rows * kv->cfg.n_kv_heads * kv->D();
+        HIPCHK(hipMalloc((void**)&kv->stage_q, nq * 2));
+        HIPCHK(hipMalloc((void**)&kv->stage_k, nk * 2));
+        HIPCHK(hipMalloc((void**)&kv->stage_v, nk * 2));
+      }
+      kv->opt_io_bf16 = value;
+      break;
+    }
+    case 10: if (value != 0 && (value < 128 || value > 4096)) throw std::runtime_error("prefill slice must be 0 or in [128, 4096] tokens"); kv->opt_chunk_slice = value; break;
     default: throw std::runtime_error("unknown option key");
   }
   YKA_CATCH_INT
@@ -550,8 +585,10 @@ int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float* d_xk, c
   YKA_TRY
   on_device(kv); check_layer(kv, layer); check_rows(kv, M); check_post(kv, P);
   if (!d_xq || !d_xk || !d_xv || !d_pos || !d_q16) throw std::runtime_error("null pointer");
+  if ((P->d_xgate == nullptr) != (P->d_gate16 == nullptr)) throw std::runtime_error("the gate projection and its output come together or not at all");
   PostArgs A{kv->view(layer), d_xq, d_xk, d_xv, M, kv->cfg.n_heads, d_pos, P->d_qn_w16, P->d_kn_w16, P->eps,
              P->d_rope, P->rope_dims, P->rope_rows, P->rotate != 0, d_q16};
+  A.xgate = P->d_xgate; A.gate16 = P->d_gate16; A.io_bf16 = kv->opt_io_bf16;
   post_launch(kv, layer, A, (hipStream_t)hip_stream);
   HIPCHK(hipGetLastError());
   YKA_CATCH_INT
@@ -559,7 +596,7 @@ int yka_attn_post(yka_kv* kv, int layer, const float* d_xq, const float* d_xk, c
 
 int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, const float* xv, int M, int pos,
                        const uint16_t* qn_w16, const uint16_t* kn_w16, float eps, const float* rope, int rope_dims,
-                       int rope_rows, int rotate, uint16_t* q16) {
+                       int rope_rows, int rotate, uint16_t* q16, const float* xgate, uint16_t* gate16) {
   YKA_TRY
   on_device(kv); check_layer(kv, layer); check_rows(kv, M);
   if (!xq || !xk || !xv || !qn_w16 || !kn_w16 || !q16) throw std::runtime_error("null pointer");
@@ -569,22 +606,27 @@ int yka_attn_post_host(yka_kv* kv, int layer, const float* xq, const float* xk, 
   if (rope_dims > 0 && (!rope || rope_rows < pos + M)) throw std::runtime_error("rotary table shorter than pos + M");
   const size_t nq = (size_t)M * kv->cfg.n_heads * kD, nk = (size_t)M * kv->cfg.n_kv_heads * kD;
   const size_t nr = rope_dims > 0 ? (size_t)rope_rows * rope_dims : 1;
-  DevBuf dq(nq * 4), dk(nk * 4), dv(nk * 4), dqw((size_t)kD * 2), dkw((size_t)kD * 2), dr(nr * 4), dq16(nq * 2);
+  if ((xgate == nullptr) != (gate16 == nullptr)) throw std::runtime_error("the gate projection and its output come together or not at all");
+  DevBuf dq(nq * 4), dk(nk * 4), dv(nk * 4), dqw((size_t)kD * 2), dkw((size_t)kD * 2), dr(nr * 4), dq16(nq * 2), dg(xgate ? nq * 4 : 4), dg16(xgate ? nq * 2 : 4);
+  if (xgate) HIPCHK(hipMemcpy(dg.p, xgate, nq * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dq.p, xq, nq * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dk.p, xk, nk * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dv.p, xv, nk * 4, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dqw.p, qn_w16, kD * 2, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dkw.p, kn_w16, kD * 2, hipMemcpyHostToDevice));
   if (rope_dims > 0) HIPCHK(hipMemcpy(dr.p, rope, nr * 4, hipMemcpyHostToDevice));
-  yka_post_params P{dqw.as<uint16_t>(), dkw.as<uint16_t>(), eps, dr.as<float>(), rope_dims, rope_rows, rotate};
+  yka_post_params P{dqw.as<uint16_t>(), dkw.as<uint16_t>(), eps, dr.as<float>(), rope_dims, rope_rows, rotate, nullptr, nullptr};
   check_post(kv, &P);
   launch_set_int(kv->d_pos, pos, kv->stream);
   PostArgs A{kv->view(layer), dq.as<float>(), dk.as<float>(), dv.as<float>(), M, kv->cfg.n_heads, kv->d_pos,
              P.d_qn_w16, P.d_kn_w16, eps, P.d_rope, rope_dims, rope_rows, rotate != 0, dq16.as<uint16_t>()};
+  if (xgate) { A.xgate = dg.as<float>(); A.gate16 = dg16.as<uint16_t>(); }
+  A.io_bf16 = kv->opt_io_bf16;
   post_launch(kv, layer, A, kv->stream);
   HIPCHK(hipGetLastError());
   HIPCHK(hipStreamSynchronize(kv->stream));
   HIPCHK(hipMemcpy(q16, dq16.p, nq * 2, hipMemcpyDeviceToHost));
+  if (xgate) HIPCHK(hipMemcpy(gate16, dg16.p, nq * 2, hipMemcpyDeviceToHost));
   YKA_CATCH_INT
 }
 
@@ -1082,8 +1124,13 @@ int yka_append_host(yka_kv* kv, int layer, const uint16_t* k16, const uint16_t* 
   HIPCHK(hipMemcpy(dk.p, k16, nk * 2, hipMemcpyHostToDevice));
   HIPCHK(hipMemcpy(dv.p, v16, nk * 2, hipMemcpyHostToDevice));
   HIPCHK(hipDeviceSynchronize());
-  launch_set_int(kv->d_pos, pos, kv->stream);
-  do_append(kv, layer, dk.as<uint16_t>(), dv.as<uint16_t>(), M, kv->d_pos, kv->stream);
+  // bf16 rows pass through staging rows that hold max_rows rows: such a handle takes the rows in pieces of that many
+  const int piece = kv->opt_io_bf16 ? kv->cfg.max_rows : M;
+  const size_t per_row = (size_t)kv->cfg.n_kv_heads * kv->D();
+  for (int r0 = 0; r0 < M; r0 += piece) {
+    launch_set_int(kv->d_pos, pos + r0, kv->stream);
+    do_append(kv, layer, dk.as<uint16_t>() + r0 * per_row, dv.as<uint16_t>() + r0 * per_row, std::min(piece, M - r0), kv->d_pos, kv->stream);
+  }
   HIPCHK(hipGetLastError());
   HIPCHK(hipStreamSynchronize(kv->stream));
   YKA_CATCH_INT

@@ -90,32 +90,41 @@ __global__ void __launch_bounds__(256) append256_kernel(AppendArgs A) {
 }
 
 // ---- the step between the QKV projection and the cache for 256-channel heads, fused with quantize-on-append
-//      (src/q35_kernels.cu:1037-1065 with fp16 in the place of the reference's bf16 roundings): per-head RMS normalisation
-//      (sum of squares: butterfly inside each wave, then ((w0 + w1) + w2) + w3), partial rotary embedding with the
-//      rotate-half pairing, optional 256-point signed rotation; Q rows leave as fp16, K and V rows go through the row
-//      quantizer as fp32 values.  grid (n_heads + 2 n_kv, M), block 256 = one head row. ----
+//      (src/q35_kernels.cu:1030-1065 in the reference's own order of operations, with fp16 in the place of its bf16
+//      roundings): the projected value is rounded to 16 bits first (:1030); per-head RMS normalisation (sum of squares:
+//      butterfly inside each run of 32 channels, then the 8 run sums folded in sequence, :1051-1056), partial rotary
+//      embedding with the rotate-half pairing, optional 256-point signed rotation; Q rows leave as fp16, K and V rows go
+//      through the row quantizer as fp32 values; gate rows (if given) leave as the rounded projection (:1048).
+//      grid (n_heads + 2 n_kv [+ n_heads gate rows], M), block 256 = one head row. ----
 __device__ __forceinline__ float f16r256(float x) { asm volatile("" : "+v"(x)); return __half2float(__float2half_rn(x)); }
 __global__ void __launch_bounds__(256) attn_post256_kernel(PostArgs A) {
   __shared__ float buf[256];
-  __shared__ float red[4];
+  __shared__ float red[8];
   __shared__ uint8_t fld[256];
   const int blk = blockIdx.x, tok = blockIdx.y, d = threadIdx.x;
   const int NH = A.n_heads, KVH = A.kv.n_kv;
   const int pos = *A.d_pos + tok;
   if (pos < 0 || pos >= A.kv.max_ctx || (A.rd > 0 && pos >= A.rope_rows)) return;   // rows outside the container are dropped
+  if (blk >= NH + 2 * KVH) {                       // gate rows: the projection rounded to the 16-bit type
+    const size_t e = ((size_t)tok * NH + (blk - NH - 2 * KVH)) * kD2 + d;
+    A.gate16[e] = A.io_bf16 ? f2bf_bits(A.xgate[e]) : __half_as_ushort(__float2half_rn(A.xgate[e]));
+    return;
+  }
   const bool isq = blk < NH, isk = !isq && blk < NH + KVH;
   const int head = isq ? blk : (isk ? blk - NH : blk - NH - KVH);
   const float* src = isq ? A.xq + ((size_t)tok * NH + head) * kD2
                          : (isk ? A.xk : A.xv) + ((size_t)tok * KVH + head) * kD2;
-  const float y = src[d];
+  const float y = f16r256(src[d]);
   float out;
   if (isq || isk) {
     float ss = __fmul_rn(y, y);
 #pragma unroll
-    for (int o = 32; o; o >>= 1) ss = __fadd_rn(ss, __shfl_xor(ss, o, 64));
-    if ((d & 63) == 0) red[d >> 6] = ss;
+    for (int o = 16; o; o >>= 1) ss = __fadd_rn(ss, __shfl_xor(ss, o, 64));
+    if ((d & 31) == 0) red[d >> 5] = ss;
     __syncthreads();
-    const float tot = __fadd_rn(__fadd_rn(__fadd_rn(red[0], red[1]), red[2]), red[3]);
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) tot = __fadd_rn(tot, red[w]);
     // sqrtf, not __fsqrt_rn: only the former is correctly rounded on this target
     const float r = __fdiv_rn(1.f, sqrtf(__fadd_rn(__fdiv_rn(tot, 256.f), A.eps)));
     const float w = __half2float(__ushort_as_half((isq ? A.qn_w16 : A.kn_w16)[d]));
@@ -138,7 +147,7 @@ __global__ void __launch_bounds__(256) attn_post256_kernel(PostArgs A) {
   }
   if (isq) {
     asm volatile("" : "+v"(out));                  // the rotation's last multiply is rounded to fp32 before the fp16 rounding
-    A.q16[((size_t)tok * NH + head) * kD2 + d] = __half_as_ushort(__float2half_rn(out));
+    A.q16[((size_t)tok * NH + head) * kD2 + d] = A.io_bf16 ? f2bf_bits(out) : __half_as_ushort(__float2half_rn(out));
   } else if (A.k32_out) {
     (isk ? A.k32_out : A.v32_out)[((size_t)tok * KVH + head) * kD2 + d] = out;
   } else {
@@ -453,11 +462,11 @@ __global__ void __launch_bounds__(256) combine256_kernel(CombineArgs A) {
   for (int k = 0; k < 8; ++k) { o += s_o[k][tid]; L += s_wsum[k]; }
   float y = L > 0.f ? __fdiv_rn(o, L) : 0.f;
   if (A.unrot) y = rotate256(y, s_w, true);        // inverse of the rotation of the V rows (src/q35_kernels.cu:1421); s_w is free again
-  A.out16[((size_t)tok * A.n_heads + head) * kD2 + tid] = __half_as_ushort(__float2half_rn(y));
+  A.out16[((size_t)tok * A.n_heads + head) * kD2 + tid] = A.out_bf16 ? f2bf_bits(y) : __half_as_ushort(__float2half_rn(y));
 }
 
 void launch_attn_post256(const PostArgs& A, hipStream_t st) {
-  hipLaunchKernelGGL(attn_post256_kernel, dim3(A.n_heads + 2 * A.kv.n_kv, A.M), dim3(256), 0, st, A);
+  hipLaunchKernelGGL(attn_post256_kernel, dim3(A.n_heads + 2 * A.kv.n_kv + (A.gate16 ? A.n_heads : 0), A.M), dim3(256), 0, st, A);
 }
 void launch_append256(const AppendArgs& A, hipStream_t st) {
   hipLaunchKernelGGL(append256_kernel, dim3(A.M, A.kv.n_kv * 2), dim3(256), 0, st, A);

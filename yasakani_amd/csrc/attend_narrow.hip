@@ -166,13 +166,13 @@ __device__ __forceinline__ void combine_column(const AttnArgs& A, int kvh, int r
       const int h = tid >> 4;
       const float L = s_red[h] + s_red[kG + h] + s_red[2 * kG + h] + s_red[3 * kG + h];
       const float inv = L > 0.f ? 1.f / L : 0.f;       // a row that saw no key at all (a rejected row of a multi-stream pass)
-      h8 v;
+      float yv[8];
 #pragma unroll
       for (int c = 0; c < 8; ++c) {
         const float o = s_o[(0 * kG + h) * kD + c8 + c] + s_o[(1 * kG + h) * kD + c8 + c] + s_o[(2 * kG + h) * kD + c8 + c] + s_o[(3 * kG + h) * kD + c8 + c];
-        v[c] = (_Float16)(o * inv);
+        yv[c] = o * inv;
       }
-      *reinterpret_cast<uint4*>(A.out16 + ((size_t)tj * A.n_heads + kvh * kG + h) * kD + c8) = __builtin_bit_cast(uint4, v);
+      *reinterpret_cast<uint4*>(A.out16 + ((size_t)tj * A.n_heads + kvh * kG + h) * kD + c8) = pack_out8(yv, A.out_bf16);
     }
   }
 }
@@ -549,7 +549,7 @@ __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
       y = y * 0.0625f * channel_sign(tid);         // signs last on the way back (src/kvx_codec.cuh:28-32)
     }
   }
-  if (tid < kD) A.out16[((size_t)tok * A.n_heads + head) * kD + tid] = __half_as_ushort(__float2half_rn(y));
+  if (tid < kD) A.out16[((size_t)tok * A.n_heads + head) * kD + tid] = A.out_bf16 ? f2bf_bits(y) : __half_as_ushort(__float2half_rn(y));
 }
 // The combiner for wide passes (many rows, at most 32 splits, no un-rotation): one wave per (token, head) row, four
 // waves per workgroup, no LDS and no barrier.  Lane = (split lane 0..3, 8 channels); a split lane takes splits sl, sl + 4,
@@ -591,10 +591,10 @@ __global__ void __launch_bounds__(256) combine_rows_kernel(CombineArgs A) {
   wsum += __shfl_xor(wsum, 16, 64); wsum += __shfl_xor(wsum, 32, 64);
   if (sl == 0) {
     const float inv = wsum > 0.f ? 1.f / wsum : 0.f;
-    h8 v;
+    float yv[8];
 #pragma unroll
-    for (int c = 0; c < 8; ++c) v[c] = (_Float16)(acc[c] * inv);
-    *reinterpret_cast<uint4*>(A.out16 + (size_t)row * kD + c8) = __builtin_bit_cast(uint4, v);
+    for (int c = 0; c < 8; ++c) yv[c] = acc[c] * inv;
+    *reinterpret_cast<uint4*>(A.out16 + (size_t)row * kD + c8) = pack_out8(yv, A.out_bf16);
   }
 }
 void launch_combine(const CombineArgs& A, hipStream_t st) {

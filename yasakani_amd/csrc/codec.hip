@@ -1,6 +1,7 @@
 // Quantize-on-append and the codec probes.  Compiled with -ffp-contract=off: the codec is bit-exact by contract,
 // and the reference builds with --fmad=false (CMakeLists.txt:60-63).
 // The quantizer itself lives in codec_device.h (shared with the fused decode kernel).
+#include <algorithm>
 #include "codec_device.h"
 
 namespace yka {
@@ -84,6 +85,31 @@ void launch_dequant_rows(const KvView& kv, int pos0, int n, float* k, float* v, 
 }
 
 __global__ void set_int_kernel(int* p, int v) { *p = v; }
+// bf16 -> fp16 for the rows a caller hands over in bf16 (handles opened for bf16 rows): 8 values per thread; blockIdx.y
+// selects the array.  The fp32 value of every bf16 is rounded to fp16 (exact for magnitudes between 2^-14 and 65504).
+__global__ void __launch_bounds__(256) bf16_to_f16_kernel(const uint16_t* a, uint16_t* a16, size_t na, const uint16_t* b, uint16_t* b16,
+                                                          const uint16_t* c, uint16_t* c16, size_t nbc) {
+  const uint16_t* src = blockIdx.y == 0 ? a : blockIdx.y == 1 ? b : c;
+  uint16_t* dst = blockIdx.y == 0 ? a16 : blockIdx.y == 1 ? b16 : c16;
+  const size_t n = blockIdx.y == 0 ? na : nbc;
+  const size_t e = ((size_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (!src || e >= n) return;
+  const uint4 r = *reinterpret_cast<const uint4*>(src + e);
+  const uint32_t w[4] = {r.x, r.y, r.z, r.w};
+  uint32_t o[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint16_t lo = __half_as_ushort(__float2half_rn(bf_bits2f((uint16_t)w[k]))), hi = __half_as_ushort(__float2half_rn(bf_bits2f((uint16_t)(w[k] >> 16))));
+    o[k] = (uint32_t)lo | ((uint32_t)hi << 16);
+  }
+  *reinterpret_cast<uint4*>(dst + e) = make_uint4(o[0], o[1], o[2], o[3]);
+}
+void launch_bf16_to_f16(const uint16_t* a, uint16_t* a16, size_t na, const uint16_t* b, uint16_t* b16, const uint16_t* c, uint16_t* c16, size_t nbc,
+                        hipStream_t st) {
+  const size_t n = std::max(na, b ? nbc : (size_t)0);
+  hipLaunchKernelGGL(bf16_to_f16_kernel, dim3((unsigned)((n / 8 + 255) / 256), b ? 3 : 1), dim3(256), 0, st, a, a16, na, b, b16, c, c16, nbc);
+}
+
 void launch_set_int(int* p, int v, hipStream_t st) { hipLaunchKernelGGL(set_int_kernel, dim3(1), dim3(1), 0, st, p, v); }
 
 }  // namespace yka

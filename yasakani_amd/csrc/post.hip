@@ -45,7 +45,8 @@ __device__ __forceinline__ float rotate128_fwd(float x, float* buf, float factor
 
 }  // namespace
 
-// grid (n_heads + 2 n_kv, M), block 128: blocks [0, n_heads) are Q heads, then the K heads, then the V heads
+// grid (n_heads + 2 n_kv [+ n_heads], M), block 128: blocks [0, n_heads) are Q heads, then the K heads, then the V heads,
+// then (if the caller hands over the gate half of the Q projection) the gate rows
 __global__ void __launch_bounds__(128) attn_post_kernel(PostArgs A) {
   __shared__ float buf[128];
   __shared__ float red[2];
@@ -53,6 +54,11 @@ __global__ void __launch_bounds__(128) attn_post_kernel(PostArgs A) {
   const int NH = A.n_heads, KVH = A.kv.n_kv;
   const int pos = *A.d_pos + tok;
   if (pos < 0 || pos >= A.kv.max_ctx || (A.rd > 0 && pos >= A.rope_rows)) return;   // same rule as the append kernel: rows outside the container are dropped
+  if (blk >= NH + 2 * KVH) {                       // gate rows (src/q35_kernels.cu:1048): the projection rounded to the 16-bit type
+    const size_t e = ((size_t)tok * NH + (blk - NH - 2 * KVH)) * kD + d;
+    A.gate16[e] = A.io_bf16 ? f2bf_bits(A.xgate[e]) : __half_as_ushort(__float2half_rn(A.xgate[e]));
+    return;
+  }
   const bool isq = blk < NH, isk = !isq && blk < NH + KVH;
   const int head = isq ? blk : (isk ? blk - NH : blk - NH - KVH);
   const float* src = isq ? A.xq + ((size_t)tok * NH + head) * kD
@@ -88,12 +94,12 @@ __global__ void __launch_bounds__(128) attn_post_kernel(PostArgs A) {
   }
   asm volatile("" : "+v"(out));                    // as in f16r: the rotation's last multiply is rounded to fp32 first
   const __half o16 = __float2half_rn(out);
-  if (isq) A.q16[((size_t)tok * NH + head) * kD + d] = __half_as_ushort(o16);
+  if (isq) A.q16[((size_t)tok * NH + head) * kD + d] = A.io_bf16 ? f2bf_bits(out) : __half_as_ushort(o16);
   else quant_store_value(A.kv, head, pos, !isk, __half2float(o16), d);
 }
 
 void launch_attn_post(const PostArgs& A, hipStream_t st) {
-  hipLaunchKernelGGL(attn_post_kernel, dim3(A.n_heads + 2 * A.kv.n_kv, A.M), dim3(128), 0, st, A);
+  hipLaunchKernelGGL(attn_post_kernel, dim3(A.n_heads + 2 * A.kv.n_kv + (A.gate16 ? A.n_heads : 0), A.M), dim3(128), 0, st, A);
 }
 
 }  // namespace yka

@@ -1,6 +1,7 @@
 // Internal declarations shared by the translation units of libyka.so (gfx950 only).
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
 #include <stdint.h>
 
 namespace yka {
@@ -68,11 +69,12 @@ struct AttnArgs {
   // narrow kernel only: tickets != nullptr folds the split combine into the launch - every workgroup of a (kv head, row
   // tile) column takes a ticket from tickets[kv head * gridDim.z + row tile] once its partials are out, and the one that
   // draws the last ticket merges the column's partials into out16 and puts the counter back to zero
-  int* tickets = nullptr; uint16_t* out16 = nullptr;
+  int* tickets = nullptr; uint16_t* out16 = nullptr; int out_bf16 = 0;
 };
 // unrot != 0: the output row gets the inverse signed Hadamard rotation (7 butterfly stages, x 1/16, signs) before it is
 // rounded to fp16 - the counterpart of rotating V rows on their way into the cache (src/q35_kernels.cu:1421)
-struct CombineArgs { const float* pm; const float* pl; const uint16_t* pacc16; int S; int M; int n_heads; uint16_t* out16; int unrot; };
+struct CombineArgs { const float* pm; const float* pl; const uint16_t* pacc16; int S; int M; int n_heads; uint16_t* out16; int unrot;
+                     int out_bf16 = 0; };   // outputs leave as bf16 (rounded once from the fp32 result) instead of fp16
 // projection outputs xq [M][n_heads][128], xk / xv [M][n_kv][128] fp32 -> q16 and the cache rows at *d_pos + t
 struct PostArgs {
   KvView kv; const float* xq; const float* xk; const float* xv; int M; int n_heads; const int* d_pos;
@@ -82,6 +84,9 @@ struct PostArgs {
   // 256-channel heads only: if set, the finished K / V rows are written here as fp32 [M][n_kv][256] instead of being
   // quantized into kv (a handle with trellis-coded rows runs its encoder on them afterwards)
   float* k32_out = nullptr; float* v32_out = nullptr;
+  // the gate half of the Q projection [M][n_heads][head_dim] fp32 -> gate16 (same shape, 16-bit), or nullptr
+  const float* xgate = nullptr; uint16_t* gate16 = nullptr;
+  int io_bf16 = 0;   // 16-bit rows that leave (q16, gate16) are bf16 instead of fp16
 };
 
 // Trellis-coded rows (trellis.hip; reference TbFastArgs, src/kvq_fast.hpp:16-37).  Probe form (yin != nullptr): rows
@@ -143,6 +148,8 @@ void launch_import_rows(const KvView&, int pos0, int n, const uint8_t* kc, const
 void launch_dequant_rows(const KvView&, int pos0, int n, float* k, float* v, hipStream_t);
 void launch_codec_probe(const uint16_t* x16, int rows, uint8_t* codes, uint16_t* scales, float* y, hipStream_t);
 void launch_set_int(int* p, int v, hipStream_t);
+// bf16 rows -> fp16 rows (round to nearest even; exact for magnitudes fp16 holds), n values each; any pointer pair may be null
+void launch_bf16_to_f16(const uint16_t* a, uint16_t* a16, size_t na, const uint16_t* b, uint16_t* b16, const uint16_t* c, uint16_t* c16, size_t nbc, hipStream_t);
 // the reference's own 256-channel row format (row256.hip): mode 0 = int8 rows, 1 = flat int4 (32 MSB-first words per row)
 void launch_row256_encode(const float* x, int rows, int mode, int rot, int8_t* q8, uint32_t* words, float* scales, hipStream_t);
 void launch_row256_decode(int rows, int mode, int rot, const int8_t* q8, const uint32_t* words, const float* scales, float* y, hipStream_t);
@@ -155,6 +162,24 @@ void launch_probe_mfma16(float* sink, unsigned long long* rec, int iters, int bl
 void launch_probe_valu(int op, float* sink, unsigned long long* rec, int iters, int blocks, int threads, hipStream_t);
 void launch_probe_cross(int op, float* sink, unsigned long long* rec, int iters, int iters_b, int blocks, hipStream_t);
 void launch_probe_read(bool nt, const void* src, size_t bytes, float* sink, int blocks, hipStream_t);
+
+// fp32 -> bf16 bit pattern, round to nearest even (finite inputs)
+__device__ __forceinline__ uint16_t f2bf_bits(float x) {
+  const uint32_t u = __float_as_uint(x);
+  return (uint16_t)((u + 0x7fffu + ((u >> 16) & 1u)) >> 16);
+}
+__device__ __forceinline__ float bf_bits2f(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+// 8 fp32 results -> 16 bytes of fp16 or bf16
+__device__ __forceinline__ uint4 pack_out8(const float* y, int bf16) {
+  uint32_t w[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    const uint16_t lo = bf16 ? f2bf_bits(y[2 * k]) : __half_as_ushort(__float2half_rn(y[2 * k]));
+    const uint16_t hi = bf16 ? f2bf_bits(y[2 * k + 1]) : __half_as_ushort(__float2half_rn(y[2 * k + 1]));
+    w[k] = (uint32_t)lo | ((uint32_t)hi << 16);
+  }
+  return make_uint4(w[0], w[1], w[2], w[3]);
+}
 
 // start of the (page, kv head) block that holds token t
 __device__ __forceinline__ uint8_t* kv_page(const KvView& kv, int kvh, int t) {

@@ -30,7 +30,8 @@ class PostParams(C.Structure):
     """yka_post_params: device pointers of the norm weights and of the rotary table, and the switches of the step
     between the QKV projection and the cache."""
     _fields_ = [("d_qn_w16", C.c_void_p), ("d_kn_w16", C.c_void_p), ("eps", C.c_float), ("d_rope", C.c_void_p),
-                ("rope_dims", C.c_int32), ("rope_rows", C.c_int32), ("rotate", C.c_int32)]
+                ("rope_dims", C.c_int32), ("rope_rows", C.c_int32), ("rotate", C.c_int32),
+                ("d_xgate", C.c_void_p), ("d_gate16", C.c_void_p)]
 
 
 def _load():
@@ -70,7 +71,7 @@ def _load():
         "yka_kv_import_rows256": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_append_attend_ms": (i32, [vp, vp, vp, vp, i32, vp, vp, vp, vp]),
         "yka_ms_call_host": (i32, [vp, vp, vp, vp, i32, vp, vp, vp]),
-        "yka_attn_post_host": (i32, [vp, i32, vp, vp, vp, i32, i32, vp, vp, C.c_float, vp, i32, i32, i32, vp]),
+        "yka_attn_post_host": (i32, [vp, i32, vp, vp, vp, i32, i32, vp, vp, C.c_float, vp, i32, i32, i32, vp, vp, vp]),
         "yka_kv_export_rows": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_kv_import_rows": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_kv_dequant_rows": (i32, [vp, i32, i32, i32, vp, vp]),
@@ -122,6 +123,17 @@ def _u16(a, shape):
     if a.dtype != np.uint16 or a.shape != tuple(shape):
         raise ValueError(f"expected fp16/uint16 array of shape {tuple(shape)}, got {a.dtype} {a.shape}")
     return a
+
+
+def bf16_bits(x):
+    """fp32 array -> bf16 bit patterns (uint16), round to nearest even (finite values)."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32)
+    return ((u + np.uint32(0x7fff) + ((u >> np.uint32(16)) & np.uint32(1))) >> np.uint32(16)).astype(np.uint16)
+
+
+def bf16_to_f32(b):
+    """bf16 bit patterns (uint16) -> fp32."""
+    return (np.ascontiguousarray(b, np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
 
 
 def build_info() -> str:
@@ -223,6 +235,7 @@ class KvCache:
 
     def __init__(self, n_layers=1, n_heads=24, n_kv_heads=4, head_dim=D, max_ctx=4096, max_rows=64, paged=False, device=0):
         self.cfg = KvConfig(n_layers, n_heads, n_kv_heads, head_dim, max_ctx, max_rows, int(bool(paged)), device)
+        self._bf16 = False          # option key 11: the boundary's 16-bit rows are bf16 (passed and returned as raw uint16 bit patterns)
         self._h = lib().yka_kv_open(C.byref(self.cfg))
         if not self._h:
             raise YkaError(lib().yka_last_error().decode("utf-8", "replace"))
@@ -260,6 +273,8 @@ class KvCache:
     # -- options / layout --
     def set_opt(self, key, value):
         _chk(lib().yka_set_opt(self._h, key, value))
+        if key == 11:
+            self._bf16 = bool(value)
 
     def set_page_table(self, table, layer=-1):
         t = np.ascontiguousarray(table, dtype=np.int32)
@@ -367,7 +382,7 @@ class KvCache:
         dep = None if depth is None else np.ascontiguousarray(depth, np.uint8)
         out = np.empty((M, self.cfg.n_heads, self.cfg.head_dim), np.uint16)
         _chk(lib().yka_layer_call_host(self._h, layer, _ptr(q), _ptr(k), _ptr(v), M, pos, _ptr(dep), _ptr(out)))
-        return out.view(np.float16)
+        return out if self._bf16 else out.view(np.float16)
 
     def append_host(self, layer, k16, v16, pos):
         """Quantize host rows k16/v16 [M,n_kv_heads,128] into rows pos..pos+M-1."""
@@ -375,9 +390,11 @@ class KvCache:
         k = _u16(k16, (M, self.cfg.n_kv_heads, self.cfg.head_dim)); v = _u16(v16, (M, self.cfg.n_kv_heads, self.cfg.head_dim))
         _chk(lib().yka_append_host(self._h, layer, _ptr(k), _ptr(v), M, pos))
 
-    def attn_post_host(self, layer, xq, xk, xv, pos, qn_w16, kn_w16, eps, rope, rope_dims, rotate=False):
+    def attn_post_host(self, layer, xq, xk, xv, pos, qn_w16, kn_w16, eps, rope, rope_dims, rotate=False, xgate=None):
         """Projection outputs (fp32; xq [M,n_heads,head_dim], xk/xv [M,n_kv_heads,head_dim]) -> RMS norm, rotary,
-        optional rotation; K/V rows are quantized into rows pos..pos+M-1, the Q rows come back as fp16."""
+        optional rotation; K/V rows are quantized into rows pos..pos+M-1, the Q rows come back as 16-bit rows (fp16; raw
+        bf16 bit patterns as uint16 if option key 11 is set).  With xgate (the gate half of the Q projection) the gate rows
+        come back too: returns (q, gate)."""
         M = xq.shape[0]
         D = self.cfg.head_dim
         xq = np.ascontiguousarray(xq, np.float32).reshape(M, self.cfg.n_heads, D)
@@ -389,9 +406,16 @@ class KvCache:
             rope = np.ascontiguousarray(rope, np.float32).reshape(-1, rope_dims // 2, 2)
             rows = rope.shape[0]
         q16 = np.empty((M, self.cfg.n_heads, D), np.uint16)
+        g16 = None
+        if xgate is not None:
+            xgate = np.ascontiguousarray(xgate, np.float32).reshape(M, self.cfg.n_heads, D)
+            g16 = np.empty((M, self.cfg.n_heads, D), np.uint16)
         _chk(lib().yka_attn_post_host(self._h, layer, _ptr(xq), _ptr(xk), _ptr(xv), M, pos, _ptr(qw), _ptr(kw), float(eps),
-                                      _ptr(rope) if rope_dims > 0 else None, int(rope_dims), rows, int(bool(rotate)), _ptr(q16)))
-        return q16.view(np.float16)
+                                      _ptr(rope) if rope_dims > 0 else None, int(rope_dims), rows, int(bool(rotate)), _ptr(q16),
+                                      _ptr(xgate) if xgate is not None else None, _ptr(g16) if g16 is not None else None))
+        if self._bf16:
+            return q16 if g16 is None else (q16, g16)
+        return q16.view(np.float16) if g16 is None else (q16.view(np.float16), g16.view(np.float16))
 
     def capture_pass(self, layers, d_q16, d_k16, d_v16, M, d_pos, d_out16, d_depth=None, mode=0):
         """Records one layer call per listed layer into a graph (device addresses); returns a Pass."""
