@@ -205,12 +205,14 @@ def trellis_figures(native, ctx=32768, L=16, bits=5, torch=None):
     return out
 
 
-def prefill_chunk(native, reps=5):
+def prefill_chunk(native, reps=5, opts=()):
     """A 2048-row prefill chunk on 131072 cached tokens: one append launch, then two 1024-token slices through the wide
     kernel (128 rows per workgroup) and their combiner launches.  4 containers x 76.7 MB."""
     ctx, M, L = 131072, 2048, 4
     q, k, v = synth(31, ctx, M)
     kv = native.KvCache(n_layers=L, max_ctx=ctx + M, max_rows=M)
+    for key, val in opts:
+        kv.set_opt(key, val)
     fill_cache(kv, k, v, ctx, chunk=16384)
     ms, _ = kv.bench(q, k[ctx:], v[ctx:], ctx, mode=0, use_graph=True, reps=reps)
     us = float(np.median(ms)) * 1e3 / L
@@ -331,14 +333,30 @@ def cpu_baseline(kv, q, ctx, M, budget_s=10.0):
             if el > budget and calls >= least:
                 return el / calls, calls, el, r
 
+    def sample_scalar(qq, pos, budget):
+        calls, t0 = 0, time.perf_counter()
+        while True:
+            oc.attend_f32(qq, pos, threads=1, scalar_build=True)
+            calls += 1
+            el = time.perf_counter() - t0
+            if el > budget:
+                return el / calls, calls, el
+
     per_call, calls, el, ref16 = sample(q, ctx, threads, budget_s)
     base = {"value": algorithmic_bytes(ctx, M) / per_call / 1e9, "unit": "GB/s", "cores": threads, "kind": "port",
-            "us_per_layer": per_call * 1e6, "build": "gcc -O3 -mavx2 -fopenmp (vectorised inner loops)",
+            "us_per_layer": per_call * 1e6, "build": yko.BUILD_FLAGS,
             "sample": f"{calls} whole layer calls (attention + combine, no append) of the same workload, {el:.1f} s"}
     other = {}
     one, c1, e1, _ = sample(q, ctx, 1, 3.0, least=1)
     other["headline_one_thread"] = {"us_per_layer": one * 1e6, "value_GBs": algorithmic_bytes(ctx, M) / one / 1e9, "cores": 1,
-                                    "sample": f"{c1} calls, {e1:.1f} s"}
+                                    "build": yko.BUILD_FLAGS, "sample": f"{c1} calls, {e1:.1f} s"}
+    # the plain scalar build of the same sources on one thread: what a straightforward CPU port of the path does
+    sc, cs, es = sample_scalar(q, ctx, 3.0)
+    other["headline_scalar_build_one_thread"] = {"us_per_layer": sc * 1e6, "value_GBs": algorithmic_bytes(ctx, M) / sc / 1e9, "cores": 1,
+                                                 "build": yko.BUILD_FLAGS_SCALAR, "sample": f"{cs} calls, {es:.1f} s"}
+    sd, cd, ed = sample_scalar(q[:1], min(32768, ctx), 1.0)
+    other["decode_32768_scalar_build_one_thread"] = {"us_per_layer": sd * 1e6, "value_GBs": algorithmic_bytes(min(32768, ctx), 1) / sd / 1e9,
+                                                     "cores": 1, "build": yko.BUILD_FLAGS_SCALAR, "sample": f"{cd} calls, {ed:.1f} s"}
     for name, pos in (("decode_4096", min(4096, ctx)), ("decode_32768", min(32768, ctx))):
         for thr in (threads, 1):
             t, c, e, _ = sample(q[:1], pos, thr, 1.0)
@@ -381,7 +399,7 @@ def machine_figures(native):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=640)
+    ap.add_argument("--steps", type=int, default=320)
     ap.add_argument("--warmup", type=int, default=64)
     ap.add_argument("--layers", type=int, default=32, help="distinct KV containers the steps rotate over")
     ap.add_argument("--ctx", type=int, default=32768)
@@ -417,7 +435,7 @@ def main():
         print(json.dumps({"machine": machine_figures(native)}))
         return
     if args.prefill_only:
-        print(json.dumps({"prefill_2048_at_131072": prefill_chunk(native, reps=8)}))
+        print(json.dumps({"prefill_2048_at_131072": prefill_chunk(native, reps=8, opts=[tuple(int(x) for x in o.split("=")) for o in args.opt])}))
         return
     if args.r256_only:
         print(json.dumps({"reference_rows_head_dim_256": r256_figures(native, args.ctx)}))
@@ -473,6 +491,9 @@ def main():
                    f"\u00b5s/layer + effective KV GB/s (% HBM peak), int4-KV GQA decode at {ctx} ctx"),
         "value": gbs, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "conditioning_ms": args.condition_ms,
         "ms_per_step": us / 1e3, "us_per_layer": us, "hbm_peak_frac": gbs / HBM_PEAK_GBS,
+        # value / ms_per_step / us_per_layer come from GPU events on the stream the calls are issued on; the host's clock
+        # around the same region (issue + synchronize included) is given beside them
+        "clock": "GPU events on the launch stream", "host_clock_us_per_layer": roof["host_clock_us_per_layer"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": f"verify window of {M} rows over {ctx} cached int4 tokens (one layer call = append + attention + combine)",
                    "n_heads": NH, "n_kv_heads": KVH, "head_dim": D, "kv_format": "int4 group-32, fp16 scales",
@@ -482,7 +503,7 @@ def main():
     }
     if not args.no_extra:
         extra = {}
-        for rows in (1, 16, 32):
+        for rows in (1, 4, 8, 16, 32):
             if rows == M:
                 continue
             u, g, r, _ = measure(rows, max(L, args.steps // 2), args.warmup)

@@ -15,10 +15,15 @@ D, GROUP = 128, 32
 NG = D // GROUP
 
 
+_SO_SCALAR = os.path.join(_HERE, "libyko_scalar.so")
+BUILD_FLAGS = "gcc -O3 -mavx2 -ffp-contract=off -fopenmp (inner loops written for the vectoriser)"
+BUILD_FLAGS_SCALAR = "gcc -O2 -fno-tree-vectorize -fno-tree-slp-vectorize -ffp-contract=off (plain scalar code)"
+
+
 def build(force=False):
     if force:
         subprocess.run(["make", "-C", _HERE, "clean"], check=True, stdout=subprocess.DEVNULL)
-    p = subprocess.run(["make", "-C", _HERE], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    p = subprocess.run(["make", "-C", _HERE, "all"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if p.returncode != 0:
         raise RuntimeError("building libyko.so failed:\n" + p.stdout[-4000:])
     return _SO
@@ -72,6 +77,21 @@ def lib():
         L.yko_tb_encode_rows.argtypes = [vp, vp, vp, C.c_int, vp, vp, vp, C.c_int, vp, vp, vp, vp]
         _lib = L
     return _lib
+
+
+_lib_scalar = None
+
+
+def scalar_lib():
+    """The attention oracle built as plain scalar code (timing baseline only; same sources, same results)."""
+    global _lib_scalar
+    if _lib_scalar is None:
+        if not os.path.exists(_SO_SCALAR):
+            build()
+        L = C.CDLL(_SO_SCALAR)
+        L.yko_attend_f32.argtypes = [C.POINTER(_Cache), C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]
+        _lib_scalar = L
+    return _lib_scalar
 
 
 def _p(a):
@@ -156,7 +176,7 @@ class Cache:
         c = self._c()
         lib().yko_append(C.byref(c), _p(k), _p(v), M, pos)
 
-    def attend_f32(self, q16, pos, depth=None, splits=0, threads=1, want_f32=False):
+    def attend_f32(self, q16, pos, depth=None, splits=0, threads=1, want_f32=False, scalar_build=False):
         q = _as_u16(q16)
         M = q.shape[0]
         assert q.shape == (M, self.n_heads, self.head_dim)
@@ -164,7 +184,7 @@ class Cache:
         out = np.empty(q.shape, np.uint16)
         o32 = np.empty(q.shape, np.float32) if want_f32 else None
         c = self._c()
-        lib().yko_attend_f32(C.byref(c), _p(q), M, pos, _p(dep), splits, threads, _p(out), _p(o32))
+        (scalar_lib() if scalar_build else lib()).yko_attend_f32(C.byref(c), _p(q), M, pos, _p(dep), splits, threads, _p(out), _p(o32))
         return (out.view(np.float16), o32) if want_f32 else out.view(np.float16)
 
     def attend_f64(self, q16, pos, depth=None):

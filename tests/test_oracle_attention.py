@@ -65,6 +65,14 @@ def test_split_count_and_threads_do_not_matter(oracle):
     assert (a.view(np.uint16) == b.view(np.uint16)).all()
 
 
+def test_scalar_build_gives_the_same_bits(oracle):
+    """The benchmark's second CPU baseline (the same sources without the vectoriser) computes the same values."""
+    c, q = _setup(oracle, 9, 3000, 5)
+    a, a32 = c.attend_f32(q, 3000, want_f32=True)
+    b, b32 = c.attend_f32(q, 3000, want_f32=True, scalar_build=True)
+    assert (a.view(np.uint16) == b.view(np.uint16)).all() and (a32.view(np.uint32) == b32.view(np.uint32)).all()
+
+
 def test_reference_split_policy_switches_at_4096(oracle):
     # rows below 4096 keys use 31 splits, rows at or above use 42 (src/q35_atxpk.cu:404-409): a window that straddles must still be right
     c, q = _setup(oracle, 8, 4090, 16)
