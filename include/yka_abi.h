@@ -130,12 +130,16 @@ YKA_API int yka_append_attend(yka_kv* kv, int layer, const uint16_t* d_q16, cons
  * 24 query heads; anything else returns -1 with a message.  The call allocates nothing, frees nothing, synchronises
  * nothing.  Every call on one GPU uses that GPU's one array: calls that overlap on a GPU (two streams, two handles) race
  * on it; calls on one stream, or otherwise ordered, are safe.  No partial has to start at zero: every launch writes
- * every partial it later reads.  The last kilobyte holds the split tickets option key 7 uses: zero when the library is
- * loaded, and put back to zero by the workgroup that draws a column's last ticket, so every launch finds them zero (a
- * launch that was aborted half way would not: reload the library, or keep option key 7 off, after a GPU fault). */
+ * every partial it later reads.  The last kilobyte holds the split tickets option key 7 uses: a fill kernel in front of
+ * every launch that uses them puts them to zero, so a launch that ended half way cannot disturb a later one. */
 YKA_API int yka_append_attend_static(yka_kv* kv, int layer, const uint16_t* d_q16, const uint16_t* d_k16,
                                      const uint16_t* d_v16, int M, const int* d_pos, const uint8_t* d_depth,
                                      uint16_t* d_out16, void* hip_stream);
+
+/* Test hook, no counterpart in the reference: overwrites the handle's OWN split workspace (the one yka_append_attend and
+ * yka_attend use) with NaN bit patterns, synchronously.  A call that gives right results afterwards did not read it
+ * without writing it first - in particular yka_append_attend_static, which must not touch it at all. */
+YKA_API int yka_kv_poison_workspace(yka_kv* kv);
 
 /* Multi-stream pass (batched decode): row t of the pass belongs to the stream whose KV container is d_row_slot[t]
  * (a container index in [0, n_layers): the handle's containers are then one per stream of the layer being run) and sits

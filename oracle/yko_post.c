@@ -11,15 +11,13 @@
  *                  d <  rd/2: f16( f16(xn[d] * cos) + f16(-xn[d + rd/2] * sin) )
  *                  d >= rd/2: f16( f16(xn[d] * cos) + f16( xn[d - rd/2] * sin) )   with (cos, sin) of channel d - rd/2
  *                then [rotation] -> fp16
- * Two deliberate differences from the reference's kernel in this 128-channel form (the 256-channel form further down
- * follows the reference's order exactly) (so this restates its algorithm, not its bit pattern; parity
- * with the reference's own outputs for this step is UNPINNED - its rsqrtf puts bit equality out of reach anyway - and
- * the functions here are pinned by the independent fp64 / closed-form checks of tests/test_oracle_post.py): the
- * reference rounds the projected value to its 16-bit type first (y = rbf(buf[tid]), :1030) and uses that everywhere,
- * here y stays fp32; and the reference folds 8 warp sums of 32-lane butterflies in sequence (:1050-1056), here the
- * order is the one below.
- * Sum order of ss (fixed so that every implementation can match it bit for bit): inside each half of 64 channels the
- * butterfly a[i] += a[i ^ o], o = 32, 16, 8, 4, 2, 1; then half 0 + half 1.
+ * The order of operations is the reference's own: the projected value is rounded to the 16-bit type first
+ * (y = rbf(buf[tid]), :1030) and that value is used everywhere; the sum of squares runs a butterfly a[i] += a[i ^ o],
+ * o = 16 .. 1, inside each run of 32 channels (:1051) and folds the run sums in sequence from 0 (:1055-1056) - 4 runs for
+ * these 128-channel heads, 8 for the reference's 256.  What still differs from the reference's bit pattern is its 16-bit
+ * type (bf16 there) and its approximate reciprocal square root (rsqrtf, not correctly rounded on its hardware): parity
+ * with the reference's own outputs for this step is therefore UNPINNED, and the functions here are pinned by the
+ * independent fp64 / closed-form checks of tests/test_oracle_post.py.
  * Rotation for 128 channels: signs from the same integer hash as the 256-channel form (src/kvx_codec.cuh:28-32),
  * 7 butterfly stages as src/kvx_codec.cuh:40-45, then a power-of-two factor: 1/8 for K and V rows, 1/16 for Q rows and
  * for the inverse applied to attention outputs.  (1/8)(1/16) 128 = 1, so q.k is unchanged by rotating both, and the
@@ -49,22 +47,24 @@ void yko_rotate128(const float* x, float* y, int inverse, float factor) {
 static float f16r(float x) { return yko_h2f(yko_f2h(x)); }
 
 static float sumsq128(const float* y) {
-  float half[2];
-  for (int w = 0; w < 2; ++w) {
-    float a[64], b[64];
-    for (int i = 0; i < 64; ++i) a[i] = y[64 * w + i] * y[64 * w + i];
-    for (int o = 32; o; o >>= 1) {
-      for (int i = 0; i < 64; ++i) b[i] = a[i] + a[i ^ o];
+  float tot = 0.f;
+  for (int w = 0; w < 4; ++w) {
+    float a[32], b[32];
+    for (int i = 0; i < 32; ++i) a[i] = y[32 * w + i] * y[32 * w + i];
+    for (int o = 16; o; o >>= 1) {
+      for (int i = 0; i < 32; ++i) b[i] = a[i] + a[i ^ o];
       memcpy(a, b, sizeof a);
     }
-    half[w] = a[0];
+    tot = tot + a[0];
   }
-  return half[0] + half[1];
+  return tot;
 }
 
 /* one Q or K head row: y[128] -> out16[128] */
-void yko_post_qk_row(const float* y, const uint16_t* w16, float eps, const float* cs /* [rd/2][2] of this position */,
+void yko_post_qk_row(const float* yin, const uint16_t* w16, float eps, const float* cs /* [rd/2][2] of this position */,
                      int rd, int rot, float rot_factor, uint16_t* out16) {
+  float y[128];
+  for (int d = 0; d < 128; ++d) y[d] = f16r(yin[d]);
   const float tot = sumsq128(y);
   const float r = 1.f / sqrtf(tot / 128.f + eps);
   float xn[128], o[128];
@@ -79,8 +79,9 @@ void yko_post_qk_row(const float* y, const uint16_t* w16, float eps, const float
   for (int d = 0; d < 128; ++d) out16[d] = yko_f2h(o[d]);
 }
 
-void yko_post_v_row(const float* y, int rot, uint16_t* out16) {
-  float o[128];
+void yko_post_v_row(const float* yin, int rot, uint16_t* out16) {
+  float y[128], o[128];
+  for (int d = 0; d < 128; ++d) y[d] = f16r(yin[d]);
   if (rot) yko_rotate128(y, o, 0, 0.125f); else memcpy(o, y, sizeof o);
   for (int d = 0; d < 128; ++d) out16[d] = yko_f2h(o[d]);
 }

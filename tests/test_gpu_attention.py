@@ -167,8 +167,8 @@ def test_multi_layer_containers_are_independent(native, oracle):
 
 @pytest.mark.parametrize("M", [65, 66])
 def test_tail_slice_of_one_or_two_rows(native, oracle, M):
-    # 64 rows on the wide kernel, then a slice of 1 or 2 rows on the decode kernel that starts at row 64 of the pass and
-    # stores its own rows
+    # a pass of 65 or 66 rows is a prefill chunk: one append launch for all its rows, then one slice (up to 1024 tokens)
+    # on the wide kernel whose last 128-row workgroup holds only the 6 or 12 rows beyond row 384
     ctx = 700
     kv, oc, q, kn, vn = _fill(native, oracle, 600 + M, ctx, M, max_rows=128)
     with kv:
@@ -181,14 +181,34 @@ def test_tail_slice_of_one_or_two_rows(native, oracle, M):
 
 
 def test_wide_pass_is_cut_into_slices(native, oracle):
-    # passes wider than 64 rows are cut into 64-row slices (src/engine35.cpp:935-947)
+    # the reference cuts passes wider than 64 rows into 64-row slices (src/engine35.cpp:935-947); here such a pass is a
+    # prefill chunk: its rows are appended by one launch, then slices of up to 1024 tokens run on the wide kernel
     ctx, M = 300, 150
     kv, oc, q, kn, vn = _fill(native, oracle, 507, ctx, M, max_rows=256)
     with kv:
         out = kv.layer_call(0, q, kn, vn, ctx)
         oc.append(kn, vn, ctx)
         assert_attn_close(out, oc.attend_f32(q, ctx, threads=8, want_f32=True)[1], "150-row pass")
-        # every slice stored its own rows (quantize-on-append rides in the attention launches), bit-exact
+        # the rows the append launch stored, bit-exact
+        got = kv.export_rows(0, ctx, M)
+        for a, b in zip(got, (oc.kc, oc.ks, oc.vc, oc.vs)):
+            assert (a == b[:, ctx:ctx + M]).all()
+
+
+@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("merge_in_launch", [0, 1])
+def test_decode_waves_with_many_few_and_no_tiles_in_one_launch(native, oracle, M, merge_in_launch):
+    """8 splits over 73 tiles: splits 0..6 hold 10 tiles each (waves 0 and 1 take three tiles - the double-buffered loop -,
+    waves 2 and 3 two - the branch without a loop), split 7 holds 3 (waves 0..2 one tile, wave 3 none): every way a wave of
+    the decode kernel waits for its query rows runs in the same launch."""
+    ctx = 73 * 32 - 20 - (M - 1)
+    kv, oc, q, kn, vn = _fill(native, oracle, 650 + M, ctx, M)
+    with kv:
+        kv.set_opt(1, 8)
+        kv.set_opt(7, merge_in_launch)
+        out = kv.layer_call(0, q, kn, vn, ctx)
+        oc.append(kn, vn, ctx)
+        assert_attn_close(out, oc.attend_f32(q, ctx, threads=8, want_f32=True)[1], f"8 splits over 73 tiles, M={M}")
         got = kv.export_rows(0, ctx, M)
         for a, b in zip(got, (oc.kc, oc.ks, oc.vc, oc.vs)):
             assert (a == b[:, ctx:ctx + M]).all()

@@ -27,6 +27,16 @@ def _fill(kv, k, v, ctx, chunk=8192):
         kv.append_host(0, k[p:p + n], v[p:p + n], p)
 
 
+def _planes_match_the_oracle_quantizer(oracle, oc, k, v, spans):
+    """The cache the GPU built (exported into oc) is what the oracle's own quantizer gives for the same fp16 rows: all four
+    planes, bit for bit, over each (first row, count) span."""
+    for lo, n in spans:
+        chk = oracle.Cache(((n + 255) // 256) * 256)
+        chk.append(k[lo:lo + n], v[lo:lo + n], 0)
+        for name, plane_chk, plane_gpu in (("K codes", chk.kc, oc.kc), ("K scales", chk.ks, oc.ks), ("V codes", chk.vc, oc.vc), ("V scales", chk.vs, oc.vs)):
+            assert (plane_chk[:, :n] == plane_gpu[:, lo:lo + n]).all(), f"{name} differ in rows {lo}..{lo + n - 1}"
+
+
 def _oracle_cache(oracle, kv, n, max_ctx):
     oc = oracle.Cache(max_ctx)
     oc.kc[:, :n], oc.ks[:, :n], oc.vc[:, :n], oc.vs[:, :n] = kv.export_rows(0, 0, n)
@@ -43,11 +53,7 @@ def test_config_1_2_decode_and_verify_at_32k(native, oracle, M):
         oc = _oracle_cache(oracle, kv, ctx + M, 33024)
         # the cache the GPU built is what the oracle's quantizer gives: all four planes of the first 2048 rows, of the last
         # 2048 cached rows and of the rows this call appended
-        for lo, n in ((0, 2048), (ctx - 2048, 2048 + M)):
-            chk = oracle.Cache(2304)
-            chk.append(k[lo:lo + n], v[lo:lo + n], 0)
-            for plane_chk, plane_gpu in ((chk.kc, oc.kc), (chk.ks, oc.ks), (chk.vc, oc.vc), (chk.vs, oc.vs)):
-                assert (plane_chk[:, :n] == plane_gpu[:, lo:lo + n]).all()
+        _planes_match_the_oracle_quantizer(oracle, oc, k, v, ((0, 2048), (ctx - 2048, 2048 + M)))
         ref16, ref32 = oc.attend_f32(q, ctx, threads=16, want_f32=True)
         assert_attn_close(out, ref32, f"32k M={M}")
         assert np.abs(out.astype(np.float64) - ref32).max() <= 2e-3   # at the measured size the plain absolute bar holds against the unrounded result too
@@ -61,6 +67,9 @@ def test_config_3_prefill_chunk_2048_on_131072(native, oracle):
         _fill(kv, k, v, ctx)
         out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx)      # quantizes the chunk into the cache
         oc = _oracle_cache(oracle, kv, ctx + M, max_ctx)
+        # the rows the chunk appended (all 2048) and 2048 cached rows from the middle of the context, against the oracle's
+        # own quantizer
+        _planes_match_the_oracle_quantizer(oracle, oc, k, v, ((ctx, M), (65536 - 1024, 2048)))
         # every 16th row of the chunk plus the first and the last row of every 64-row group: the rows of one group are one
         # oracle call (a window at position ctx + 64 g whose depth table names the sampled rows)
         for g in range(M // 64):
@@ -91,6 +100,8 @@ def test_config_4_paged_262144(native, oracle):
             outs[paged, 64] = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx)
             if paged:
                 oc = _oracle_cache(oracle, kv, ctx + 64, max_ctx)
+                # the rows the window appended and 2048 cached rows that straddle pages, read back through the page table
+                _planes_match_the_oracle_quantizer(oracle, oc, k, v, ((ctx, 64), (131072 - 1000, 2048)))
     for M in (1, 64):
         assert (outs[False, M].view(np.uint16) == outs[True, M].view(np.uint16)).all(), f"paged != contiguous at M={M}"
     ref32 = oc.attend_f32(q[:1], ctx, threads=16, want_f32=True)[1]
@@ -98,3 +109,7 @@ def test_config_4_paged_262144(native, oracle):
     assert_attn_close(outs[True, 1], ref32, "262144 decode")
     ref64 = oc.attend_f32(q[60:64], ctx + 60, depth=np.arange(4, dtype=np.uint8), threads=16, want_f32=True)[1]
     assert_attn_close(outs[True, 64][60:64], ref64, "262144 verify rows 60..63")
+    # rows from all four 16-row quarters of the window (one oracle call: a window at ctx whose depth table names them)
+    sel = np.array([0, 21, 42, 63], dtype=np.uint8)
+    ref_sel = oc.attend_f32(q[sel.astype(np.int64)], ctx, depth=sel, threads=16, want_f32=True)[1]
+    assert_attn_close(outs[True, 64][sel.astype(np.int64)], ref_sel, "262144 verify rows 0, 21, 42, 63")

@@ -151,3 +151,28 @@ def test_large_scores_raise_the_running_maximum(native, oracle):
         out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx)
         oc.append(k[ctx:], v[ctx:], ctx)
         assert_attn_close(out, oc.attend_f32(q, ctx, threads=8, want_f32=True)[1], "growing scores")
+
+
+@pytest.mark.parametrize("M", [4, 8, 16])
+def test_windows_at_32k(native, oracle, M):
+    """The measured size: 32768 cached tokens (1025 tiles over 256 waves), rows quantized by the library itself."""
+    ctx = 32768
+    ch = oracle.outlier_channels(7900 + M)
+    q = oracle.fill_normal_f16(7901 + M, M * 24).reshape(M, 24, 128)
+    k = oracle.fill_normal_f16(7902 + M, (ctx + M) * 4, 128, ch, 8.0).reshape(ctx + M, 4, 128)
+    v = oracle.fill_normal_f16(7903 + M, (ctx + M) * 4).reshape(ctx + M, 4, 128)
+    with native.KvCache(max_ctx=33024) as kv:
+        kv.set_opt(8, 16)
+        for p in range(0, ctx, 8192):
+            kv.append_host(0, k[p:p + 8192], v[p:p + 8192], p)
+        out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx)
+        oc = oracle.Cache(33024)
+        n = ctx + M
+        oc.kc[:, :n], oc.ks[:, :n], oc.vc[:, :n], oc.vs[:, :n] = kv.export_rows(0, 0, n)
+        chk = oracle.Cache(256)
+        chk.append(k[ctx:], v[ctx:], 0)
+        for a, b in zip((chk.kc, chk.ks, chk.vc, chk.vs), (oc.kc, oc.ks, oc.vc, oc.vs)):
+            assert (a[:, :M] == b[:, ctx:ctx + M]).all()                     # the rows the kernel stored: the oracle's quantizer, bit for bit
+        ref32 = oc.attend_f32(q, ctx, threads=16, want_f32=True)[1]
+        assert_attn_close(out, ref32, f"32k M={M}")
+        assert np.abs(out.astype(np.float64) - ref32).max() <= 2e-3

@@ -1,6 +1,7 @@
 """Pins the oracle's restatement of the step between the QKV projection and the cache (RMS normalisation, partial
 rotary embedding, 128-point signed Hadamard rotation) against numpy fp64 forms and structural properties.  CPU only."""
 import numpy as np
+import pytest
 from scipy.linalg import hadamard
 
 from oracle import yko
@@ -64,9 +65,10 @@ def test_post_rows_match_fp64_forms():
             assert np.abs(_h(k16[t, h]) - ref).max() <= 2.5e-3 * max(1.0, np.abs(ref).max())
     # V rows: plain rounding to fp16
     assert np.array_equal(v16, xv.astype(np.float16).view(np.uint16))
-    # channels past rd carry no rotary change: one rounding only
-    ref = _post_numpy(xq[0, 0], qw, 1e-6, rope[pos].astype(np.float64), rd)
-    assert np.array_equal(q16[0, 0, rd:], ref[rd:].astype(np.float16).view(np.uint16))
+    # channels past rd carry no rotary change: the entry rounding and one more
+    r16 = lambda a: a.astype(np.float16).astype(np.float32)
+    ref = _post_numpy(r16(xq[0, 0]), qw, 1e-6, rope[pos].astype(np.float64), rd)
+    assert np.abs(_h(q16[0, 0, rd:]) - ref[rd:]).max() <= 1.0e-3 * max(1.0, np.abs(ref).max())
 
 
 def test_post_structure():
@@ -102,7 +104,8 @@ def test_post_with_rotation_equals_rotation_of_post():
     f = lambda u: u.view(np.float16).astype(np.float32).reshape(-1, 128)
     assert np.array_equal(q1.reshape(-1, 128), yko.rotate128(f(q0), False, 0.0625).astype(np.float16).view(np.uint16))
     assert np.array_equal(k1.reshape(-1, 128), yko.rotate128(f(k0), False, 0.125).astype(np.float16).view(np.uint16))
-    assert np.array_equal(v1.reshape(-1, 128), yko.rotate128(xv.reshape(-1, 128), False, 0.125).astype(np.float16).view(np.uint16))
+    xv16 = xv.astype(np.float16).astype(np.float32)                    # the projection is rounded on entry
+    assert np.array_equal(v1.reshape(-1, 128), yko.rotate128(xv16.reshape(-1, 128), False, 0.125).astype(np.float16).view(np.uint16))
     # scores survive the rotation up to the fp16 rounding of the rotated rows
     s0 = (f(q0)[:24].astype(np.float64) * f(k0)[0]).sum(1)
     s1 = (f(q1)[:24].astype(np.float64) * f(k1)[0]).sum(1)
@@ -180,18 +183,20 @@ def test_post256_structure():
     assert np.array_equal(qi[0, 0], (xi[0, 0] * r).astype(np.float16).view(np.uint16))
 
 
-def test_post256_sum_of_squares_follows_the_reference_order():
-    """ss = the 8 sums of 32-channel runs (each a butterfly a[i] += a[i ^ o], o = 16 .. 1) folded in sequence from 0
+@pytest.mark.parametrize("D", [128, 256])
+def test_sum_of_squares_follows_the_reference_order(D):
+    """ss = the sums of 32-channel runs (each a butterfly a[i] += a[i ^ o], o = 16 .. 1) folded in sequence from 0
     (src/q35_kernels.cu:1050-1056).  With one large square per run and tiny ones beside it the fp32 result depends on
     the association; the row's normalisation factor must be the one this order gives."""
-    rng = np.random.default_rng(15)
-    zero_w = np.zeros(256, np.uint16)
-    rope = yko.rope_table(4, 0) if False else np.zeros((1, 1, 2), np.float32)
+    rng = np.random.default_rng(15 + D)
+    zero_w = np.zeros(D, np.uint16)
+    rope = np.zeros((1, 1, 2), np.float32)
+    post = yko.attn_post256 if D == 256 else yko.attn_post
     for trial in range(20):
-        x = (rng.standard_normal(256) * 10.0 ** rng.integers(-3, 3, size=256)).astype(np.float16).astype(np.float32)
+        x = (rng.standard_normal(D) * 10.0 ** rng.integers(-3, 3, size=D)).astype(np.float16).astype(np.float32)
         sq = (x * x).astype(np.float32)
         runs = []
-        for w in range(8):
+        for w in range(D // 32):
             a = sq[32 * w:32 * w + 32].copy()
             for o in (16, 8, 4, 2, 1):
                 a = (a + a[np.arange(32) ^ o]).astype(np.float32)
@@ -199,7 +204,7 @@ def test_post256_sum_of_squares_follows_the_reference_order():
         tot = np.float32(0.0)
         for r_ in runs:
             tot = np.float32(tot + r_)
-        r = np.float32(1.0) / np.sqrt(np.float32(tot / np.float32(256.0)))
-        q16, _, _ = yko.attn_post256(x.reshape(1, 1, 256), x.reshape(1, 1, 256), x.reshape(1, 1, 256), zero_w, zero_w, 0.0, rope, 0, 0, 0)
+        r = np.float32(1.0) / np.sqrt(np.float32(tot / np.float32(D)))
+        q16, _, _ = post(x.reshape(1, 1, D), x.reshape(1, 1, D), x.reshape(1, 1, D), zero_w, zero_w, 0.0, rope, 0, 0, 0)
         expect = (x * r).astype(np.float32).astype(np.float16).view(np.uint16)
         assert np.array_equal(q16[0, 0], expect), trial

@@ -1,6 +1,8 @@
 """The allocation-free layer call (yka_append_attend_static) against yka_append_attend: same kernels, same split
 counts, so outputs and appended rows must agree bit for bit.  Two calls in a row share the GPU's one static workspace;
-the second is smaller than the first, so stale partials of the first lie next to the ones it writes."""
+the second is smaller than the first, so stale partials of the first lie next to the ones it writes.  The handle's own
+workspace holds NaN patterns while the static calls run (they must not read it), free device memory is the same before
+and after them, and the call is also issued under stream capture - where an allocation is refused - and replayed."""
 import ctypes
 
 import numpy as np
@@ -15,7 +17,22 @@ class _Hip:
         self.rt.hipMalloc.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_size_t]
         self.rt.hipMemcpy.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int]
         self.rt.hipFree.argtypes = [ctypes.c_void_p]
+        self.rt.hipMemGetInfo.argtypes = [ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+        self.rt.hipStreamCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.rt.hipStreamDestroy.argtypes = [ctypes.c_void_p]
+        self.rt.hipStreamSynchronize.argtypes = [ctypes.c_void_p]
+        self.rt.hipStreamBeginCapture.argtypes = [ctypes.c_void_p, ctypes.c_int]
+        self.rt.hipStreamEndCapture.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_void_p)]
+        self.rt.hipGraphInstantiate.argtypes = [ctypes.POINTER(ctypes.c_void_p), ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t]
+        self.rt.hipGraphLaunch.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        self.rt.hipGraphExecDestroy.argtypes = [ctypes.c_void_p]
+        self.rt.hipGraphDestroy.argtypes = [ctypes.c_void_p]
         self.bufs = []
+
+    def free_bytes(self):
+        free, total = ctypes.c_size_t(), ctypes.c_size_t()
+        self._ok(self.rt.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)))
+        return free.value
 
     def _ok(self, rc):
         assert rc == 0, f"HIP error {rc}"
@@ -60,11 +77,16 @@ def test_static_workspace_call_equals_the_allocating_one(native, oracle):
             dq, dk, dv, dpos = hip.alloc(nq), hip.alloc(nk), hip.alloc(nk), hip.alloc(4)
             dout_a, dout_b = hip.alloc(nq), hip.alloc(nq)
             pos = ctx
+            free_before = None
             for M, off in calls:
                 q = q_all[off:off + M]
                 hip.upload(dq, q.view(np.uint16)); hip.upload(dk, k_new[off:off + M].view(np.uint16)); hip.upload(dv, v_new[off:off + M].view(np.uint16))
                 hip.upload(dpos, np.array([pos], np.int32))
                 kv.append_attend(0, dq, dk, dv, M, dpos, dout_a)
+                hip.sync()
+                kv.poison_workspace()                    # the handle's own partials: NaN while the static call runs
+                if free_before is None:
+                    free_before = hip.free_bytes()
                 kv.append_attend_static(1, dq, dk, dv, M, dpos, dout_b)
                 hip.sync()
                 a = np.empty((M, 24, 128), np.uint16); b = np.empty((M, 24, 128), np.uint16)
@@ -73,6 +95,41 @@ def test_static_workspace_call_equals_the_allocating_one(native, oracle):
                 for x, y in zip(kv.export_rows(0, pos, M), kv.export_rows(1, pos, M)):
                     assert (x == y).all(), f"appended rows differ at M={M}"
                 pos += M
+            # a workspace allocated behind the caller's back would be 26 MB (the handle's) or 9.7 MB (the static array's size);
+            # the runtime's own pools (kernel arguments, signals) may grow by a page or two
+            assert free_before - hip.free_bytes() < (2 << 20), "free device memory shrank over the static calls"
+            # the same call recorded under stream capture (an allocation there is refused) and replayed twice, with eager
+            # work in between; layer 1 holds the rows already, the replays store the same rows again
+            M, off = calls[1]
+            pos_c = ctx + calls[0][0]
+            hip.upload(dq, q_all[off:off + M].view(np.uint16)); hip.upload(dk, k_new[off:off + M].view(np.uint16)); hip.upload(dv, v_new[off:off + M].view(np.uint16))
+            hip.upload(dpos, np.array([pos_c], np.int32))
+            kv.append_attend(0, dq, dk, dv, M, dpos, dout_a)
+            hip.sync()
+            want = np.empty((M, 24, 128), np.uint16); hip.download(dout_a, want)
+            st, graph, gexec = ctypes.c_void_p(), ctypes.c_void_p(), ctypes.c_void_p()
+            hip._ok(hip.rt.hipStreamCreate(ctypes.byref(st)))
+            try:
+                kv.poison_workspace()
+                hip._ok(hip.rt.hipStreamBeginCapture(st, 0))                 # global mode: unsafe calls (allocations) fail
+                try:
+                    kv.append_attend_static(1, dq, dk, dv, M, dpos, dout_b, None, st.value)
+                finally:
+                    rc_end = hip.rt.hipStreamEndCapture(st, ctypes.byref(graph))
+                hip._ok(rc_end)
+                hip._ok(hip.rt.hipGraphInstantiate(ctypes.byref(gexec), graph, None, None, 0))
+                for replay in range(2):
+                    hip.upload(dout_b, np.zeros((M, 24, 128), np.uint16))
+                    hip._ok(hip.rt.hipGraphLaunch(gexec, st))
+                    hip._ok(hip.rt.hipStreamSynchronize(st))
+                    got = np.empty((M, 24, 128), np.uint16); hip.download(dout_b, got)
+                    assert (got == want).all(), f"replay {replay} of the captured static call differs"
+                    kv.append_attend_static(1, dq, dk, dv, M, dpos, dout_b)      # eager work between the replays
+                    hip.sync()
+            finally:
+                if gexec: hip.rt.hipGraphExecDestroy(gexec)
+                if graph: hip.rt.hipGraphDestroy(graph)
+                hip.rt.hipStreamDestroy(st)
             # and the allocating call is what the oracle says (so both are)
             from tests.tolerances import assert_attn_close
             oc = oracle.Cache(2304)

@@ -295,7 +295,12 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
                fuse_append ? k16 : nullptr, fuse_append ? v16 : nullptr};
     // option key 7, rows of at most 2 tokens: the last workgroup of each column merges the splits inside the attention launch
     const bool one_launch = narrow && mode == 0 && !kv->opt_unrot && kv->opt_merge_in_launch;
-    if (one_launch) { A.tickets = W.tickets; A.out16 = out16 + (size_t)s0 * NH * kD; A.out_bf16 = io_was; }
+    if (one_launch) {
+      // the counters are put back to zero by a fill kernel in front of every such launch: a launch that ended half way
+      // (or anything else that left one non-zero) cannot make a later call skip its merge
+      launch_zero_ints(W.tickets, kv->cfg.n_kv_heads * kMaxSlice, st);
+      A.tickets = W.tickets; A.out16 = out16 + (size_t)s0 * NH * kD; A.out_bf16 = io_was;
+    }
     if (narrow) launch_attend_narrow(A, st); else if (mid) launch_attend_mid(A, st); else launch_attend_wide(A, st);
     if (mode != 2 && !one_launch) launch_combine(CombineArgs{W.pm, W.pl, W.pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * kD, kv->opt_unrot, io_was}, st);
   }
@@ -339,7 +344,10 @@ void do_attend_ms(yka_kv* kv, const uint16_t* q16, const uint16_t* k16, const ui
     AttnArgs A{kv->view(0), q16 + (size_t)s0 * NH * D, nullptr, nullptr, Ms, s0, NH, S, 128, kv->pm, kv->pl, kv->pacc16, nullptr, nullptr, Rs};
     const CombineArgs C{kv->pm, kv->pl, kv->pacc16, S, Ms, NH, out16 + (size_t)s0 * NH * D, kv->opt_unrot, io_was};
     if (r256) { launch_attend256(A, st); launch_combine256(C, st); }
-    else if (!kv->opt_unrot && kv->opt_merge_in_launch) { A.tickets = kv->tickets; A.out16 = C.out16; A.out_bf16 = io_was; launch_attend_narrow(A, st); }
+    else if (!kv->opt_unrot && kv->opt_merge_in_launch) {
+      launch_zero_ints(kv->tickets, kv->cfg.n_kv_heads * kMaxSlice, st);
+      A.tickets = kv->tickets; A.out16 = C.out16; A.out_bf16 = io_was; launch_attend_narrow(A, st);
+    }
     else { launch_attend_narrow(A, st); launch_combine(C, st); }
   }
 }
@@ -524,6 +532,18 @@ int yka_append_attend_static(yka_kv* kv, int layer, const uint16_t* d_q16, const
                     reinterpret_cast<int*>(base + kStaticWsBytes - kStaticTicketBytes)};   // 24 heads = 4 kv heads x 64 row tiles of tickets at most
   do_attend(kv, layer, d_q16, M, d_pos, d_depth, d_out16, (hipStream_t)hip_stream, 0, d_k16, d_v16, &W);
   HIPCHK(hipGetLastError());
+  YKA_CATCH_INT
+}
+
+int yka_kv_poison_workspace(yka_kv* kv) {
+  YKA_TRY
+  on_device(kv);
+  HIPCHK(hipDeviceSynchronize());
+  const size_t rows = kWsPairs * (size_t)kv->cfg.n_heads;
+  HIPCHK(hipMemset(kv->pm, 0xff, rows * 4));
+  HIPCHK(hipMemset(kv->pl, 0xff, rows * 4));
+  HIPCHK(hipMemset(kv->pacc16, 0xff, rows * (size_t)kv->D() * 2));
+  HIPCHK(hipDeviceSynchronize());
   YKA_CATCH_INT
 }
 
@@ -1148,6 +1168,8 @@ int yka_machine_probe(int kind, int p0, int iters, int blocks, int threads, doub
     if (kind == 5 && (p0 < 0 || p0 > 7)) throw std::runtime_error("kind 5: p0 = opcode 0..7");
     if (kind == 5) threads = 512;
     if (kind == 4 && iters > 4096) throw std::runtime_error("kind 4: iters = MiB to read, at most 4096");
+    // a probe loop cannot be stopped once launched: a million iterations (about a second) is the most a call may ask for
+    if (iters > 1000000 || (kind == 3 && p0 > 1000000)) throw std::runtime_error("iters (and p0 of kind 3) must be at most 1000000");
     if (kind == 1) threads = 256;
     const int waves = blocks * (threads / 64);
     const size_t nbytes = kind == 4 ? (size_t)iters << 20 : 16;

@@ -60,13 +60,15 @@ __device__ __forceinline__ uint4 ld_agent16(const uint16_t* p) {
 
 // The workgroup's partials are out (or its "no keys" markers): wait until the stores are acknowledged, take a ticket of
 // the column.  True for the workgroup that drew the last one: every partial of the column is then visible to agent-scope
-// loads.  It also puts the counter back to zero for the next launch.
+// loads.  The ticket is an acquire-release operation at agent scope behind a workgroup barrier, so the order "partials,
+// then ticket" (writers) and "ticket, then partials" (the merging workgroup) holds by the memory model and not only by
+// the explicit wait.  The counter is also put back to zero; the host zeroes it in front of every launch regardless.
 __device__ __forceinline__ bool last_of_column(const AttnArgs& A, int* s_ticket) {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   int* t = A.tickets + blockIdx.y * gridDim.z + blockIdx.z;
   if (threadIdx.x == 0) {
-    const int old = __hip_atomic_fetch_add(t, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const int old = __hip_atomic_fetch_add(t, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
     if (old == A.S - 1) __hip_atomic_store(t, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     *s_ticket = old;
   }

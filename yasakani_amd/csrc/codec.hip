@@ -110,6 +110,8 @@ void launch_bf16_to_f16(const uint16_t* a, uint16_t* a16, size_t na, const uint1
   hipLaunchKernelGGL(bf16_to_f16_kernel, dim3((unsigned)((n / 8 + 255) / 256), b ? 3 : 1), dim3(256), 0, st, a, a16, na, b, b16, c, c16, nbc);
 }
 
+__global__ void zero_ints_kernel(int* p, int n) { const int i = blockIdx.x * 256 + threadIdx.x; if (i < n) p[i] = 0; }
+void launch_zero_ints(int* p, int n, hipStream_t st) { hipLaunchKernelGGL(zero_ints_kernel, dim3((n + 255) / 256), dim3(256), 0, st, p, n); }
 void launch_set_int(int* p, int v, hipStream_t st) { hipLaunchKernelGGL(set_int_kernel, dim3(1), dim3(1), 0, st, p, v); }
 
 }  // namespace yka

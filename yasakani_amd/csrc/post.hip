@@ -1,16 +1,13 @@
 // The step between the QKV projection and the cache for 128-channel heads, fused with quantize-on-append:
 // per-head RMS normalisation, partial rotary embedding, optional signed Walsh-Hadamard rotation; Q rows leave as fp16,
 // K and V rows go straight into the int4 cache without a round trip through HBM as fp16.
-// Follows q35_attn_post_kernel (src/q35_kernels.cu:1013-1065) with fp16 in the place of the reference's bf16 roundings.
-// Two deliberate differences from that kernel, so this step is the reference's ALGORITHM, not its bit pattern (which
-// its rsqrtf puts out of reach anyway: parity with the reference's own outputs for this step is unpinned, the kernel is
-// pinned bit for bit against a CPU restatement of the sequence below, kept with the tests):
-//   * the reference first rounds the projected value to its 16-bit type (y = rbf(buf[tid]), :1030) and forms V, the sum
-//     of squares and xn from that; here the projection's fp32 value is used unrounded (one rounding fewer);
-//   * the reference sums squares by a 32-lane butterfly and then folds its 8 warp sums in sequence (:1050-1056); here the
-//     butterfly runs over 64 lanes and the two wave sums are added.
+// Follows q35_attn_post_kernel (src/q35_kernels.cu:1013-1065) in its own order of operations, with fp16 in the place of
+// the reference's bf16 roundings and a correctly rounded 1/sqrt in the place of its rsqrtf (which puts its bit pattern
+// out of reach: the kernel is pinned bit for bit against a CPU restatement of the sequence below, kept with the tests).
 // Compiled with -ffp-contract=off; every value is a fixed sequence of single IEEE operations:
-//   ss = sum y^2: butterfly a += a[lane ^ o], o = 32..1, inside each wave (= 64-channel half), then half 0 + half 1
+//   y = f16(projected value), for Q, K, V and gate rows alike (:1030)
+//   ss = sum y^2: butterfly a += a[lane ^ o], o = 16..1, inside each run of 32 channels (:1051), then the 4 run sums
+//   folded in sequence from 0 (:1055-1056)
 //   r = 1 / sqrt(ss / 128 + eps);  xn = f16(y * r * (1 + w))
 //   rotary, pairing d <-> d + rd/2:  f16(f16(xn * cos) + f16(-+ partner * sin))
 //   rotation: signs (src/kvx_codec.cuh:28-32), 7 butterfly stages (src/kvx_codec.cuh:40-45), x 1/8 for K and V,
@@ -49,7 +46,7 @@ __device__ __forceinline__ float rotate128_fwd(float x, float* buf, float factor
 // then (if the caller hands over the gate half of the Q projection) the gate rows
 __global__ void __launch_bounds__(128) attn_post_kernel(PostArgs A) {
   __shared__ float buf[128];
-  __shared__ float red[2];
+  __shared__ float red[4];
   const int blk = blockIdx.x, tok = blockIdx.y, d = threadIdx.x;
   const int NH = A.n_heads, KVH = A.kv.n_kv;
   const int pos = *A.d_pos + tok;
@@ -63,15 +60,17 @@ __global__ void __launch_bounds__(128) attn_post_kernel(PostArgs A) {
   const int head = isq ? blk : (isk ? blk - NH : blk - NH - KVH);
   const float* src = isq ? A.xq + ((size_t)tok * NH + head) * kD
                          : (isk ? A.xk : A.xv) + ((size_t)tok * KVH + head) * kD;
-  const float y = src[d];
+  const float y = f16r(src[d]);
   float out;
   if (isq || isk) {
     float ss = __fmul_rn(y, y);
 #pragma unroll
-    for (int o = 32; o; o >>= 1) ss = __fadd_rn(ss, __shfl_xor(ss, o, 64));
-    if ((d & 63) == 0) red[d >> 6] = ss;
+    for (int o = 16; o; o >>= 1) ss = __fadd_rn(ss, __shfl_xor(ss, o, 64));
+    if ((d & 31) == 0) red[d >> 5] = ss;
     __syncthreads();
-    const float tot = __fadd_rn(red[0], red[1]);
+    float tot = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) tot = __fadd_rn(tot, red[w]);
     // sqrtf, not __fsqrt_rn: only the former is correctly rounded on this target (measured against IEEE on 2^20 inputs)
     const float r = __fdiv_rn(1.f, sqrtf(__fadd_rn(__fdiv_rn(tot, 128.f), A.eps)));
     const float w = h2f_bits((isq ? A.qn_w16 : A.kn_w16)[d]);

@@ -148,6 +148,7 @@ void launch_import_rows(const KvView&, int pos0, int n, const uint8_t* kc, const
 void launch_dequant_rows(const KvView&, int pos0, int n, float* k, float* v, hipStream_t);
 void launch_codec_probe(const uint16_t* x16, int rows, uint8_t* codes, uint16_t* scales, float* y, hipStream_t);
 void launch_set_int(int* p, int v, hipStream_t);
+void launch_zero_ints(int* p, int n, hipStream_t);   // a fill kernel (safe inside a captured graph, unlike a memset node)
 // bf16 rows -> fp16 rows (round to nearest even; exact for magnitudes fp16 holds), n values each; any pointer pair may be null
 void launch_bf16_to_f16(const uint16_t* a, uint16_t* a16, size_t na, const uint16_t* b, uint16_t* b16, const uint16_t* c, uint16_t* c16, size_t nbc, hipStream_t);
 // the reference's own 256-channel row format (row256.hip): mode 0 = int8 rows, 1 = flat int4 (32 MSB-first words per row)

@@ -52,6 +52,7 @@ def _load():
         "yka_attend": (i32, [vp, i32, vp, i32, vp, vp, vp, vp]),
         "yka_append_attend": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
         "yka_append_attend_static": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
+        "yka_kv_poison_workspace": (i32, [vp]),
         "yka_codec_probe": (i32, [vp, i32, vp, vp, vp]),
         "yka_kvx256_probe": (i32, [vp, i32, i32, i32, vp, vp, vp, vp]),
         "yka_attn_post": (i32, [vp, i32, vp, vp, vp, i32, vp, vp, vp, vp]),
@@ -91,7 +92,7 @@ def _load():
 
 
 EXPORTS = ("yka_kv_open", "yka_kv_close", "yka_last_error", "yka_build_info", "yka_set_opt", "yka_kv_set_page_table",
-           "yka_append", "yka_attend", "yka_append_attend", "yka_append_attend_static", "yka_codec_probe", "yka_kvx256_probe", "yka_tb_pack_unpack", "yka_kv_set_profile", "yka_kv_profile_bits", "yka_kv_export_rows_tb", "yka_attn_post", "yka_append_attend_ms", "yka_ms_call_host",
+           "yka_append", "yka_attend", "yka_append_attend", "yka_append_attend_static", "yka_kv_poison_workspace", "yka_codec_probe", "yka_kvx256_probe", "yka_tb_pack_unpack", "yka_kv_set_profile", "yka_kv_profile_bits", "yka_kv_export_rows_tb", "yka_attn_post", "yka_append_attend_ms", "yka_ms_call_host",
            "yka_attn_post_host", "yka_kv_export_rows", "yka_kv_export_rows256", "yka_kv_import_rows256",
            "yka_attn_out256", "yka_attn_out256_host", "yka_attn_out256_lo", "yka_attn_out256_lo_host", "yka_append256_f32", "yka_rotate_q256", "yka_append256_f32_host", "yka_rotate_q256_host",
            "yka_kv_import_rows", "yka_kv_dequant_rows", "yka_kv_replicate_layer", "yka_layer_call_host",
@@ -322,6 +323,10 @@ class KvCache:
     def append_attend_static(self, layer, d_q16, d_k16, d_v16, M, d_pos, d_out16, d_depth=None, stream=0):
         """yka_append_attend with the split partials in the library's static device workspace (allocation-free form)."""
         _chk(lib().yka_append_attend_static(self._h, layer, d_q16, d_k16, d_v16, M, d_pos, d_depth, d_out16, stream))
+
+    def poison_workspace(self):
+        """test hook: NaN patterns over the handle's own split workspace"""
+        _chk(lib().yka_kv_poison_workspace(self._h))
 
     def set_profile(self, blob):
         """switch a head_dim-256 handle to trellis-coded rows under a KVQP profile blob (see yasakani_amd.kvqp)"""
