@@ -222,6 +222,85 @@ def prefill_chunk(native, reps=5, opts=()):
     return {"us_per_layer": us, "tflops": fl / (us * 1e-6) / 1e12, "mfma_peak_frac": fl / (us * 1e-6) / 1e12 / MFMA_F16_PEAK_TFLOPS}
 
 
+def sweep(native, which=("verify", "decode", "paged", "prefill"), reps=8, out=sys.stdout):
+    """Launch-geometry sweep: every workload below is timed as whole layer calls (append + attention + combine, replayed
+    from a graph over all containers of the handle, median of `reps` sweeps) under each value of the option keys that
+    shape its grid.  Key 0 / value 0 is the library's own choice.  Prints a table; returns the rows.  Any error ends the
+    sweep at once (the exception propagates): nothing is retried."""
+    rows_out = []
+
+    warmed = set()
+
+    def timed(kv, L, q, kn, vn, ctx, opts):
+        if id(kv) not in warmed:                             # the first sweeps on a fresh handle run at ramping clocks
+            warmed.add(id(kv))
+            t0 = time.perf_counter()
+            while time.perf_counter() - t0 < 0.2:
+                kv.bench(q, kn, vn, ctx, mode=0, use_graph=True, reps=reps)
+        for key, val in opts:
+            kv.set_opt(key, val)
+        ms, _ = kv.bench(q, kn, vn, ctx, mode=0, use_graph=True, reps=reps)
+        for key, _ in opts:
+            kv.set_opt(key, 0 if key != 8 else 10)           # back to the defaults
+        return float(np.median(ms)) * 1e3 / L
+
+    def emit(workload, opts, us, note=""):
+        label = " ".join(f"{k}={v}" for k, v in opts) or "defaults"
+        rows_out.append({"workload": workload, "options": label, "us_per_layer": us, "note": note})
+        print(f"| {workload} | {label} | {us:.2f} | {note} |", file=out, flush=True)
+
+    print("| workload | option keys | us per layer call | note |\n|---|---|---|---|", file=out, flush=True)
+    if "verify" in which or "decode" in which:
+        ctx, L = 32768, 32
+        q, k, v = synth(2026, ctx, 64)
+        kv = native.KvCache(n_layers=L, max_ctx=((ctx + 64 + 255) // 256) * 256, max_rows=64)
+        fill_cache(kv, k, v, ctx)
+        kn, vn = k[ctx:], v[ctx:]
+        if "verify" in which:
+            for M in (4, 8, 16, 32, 64):
+                name = f"verify-{M} at 32768"
+                emit(name, (), timed(kv, L, q[:M], kn[:M], vn[:M], ctx, ()))
+                if M <= 16:
+                    for S in (0, 8, 16, 32, 64):
+                        emit(name, ((8, 16), (9, S)), timed(kv, L, q[:M], kn[:M], vn[:M], ctx, ((8, 16), (9, S))), "mid kernel")
+                for S in (0, 2, 3, 4, 5, 6, 8, 10, 12, 16, 21, 32, 64):
+                    emit(name, ((8, 0), (2, S)), timed(kv, L, q[:M], kn[:M], vn[:M], ctx, ((8, 0), (2, S))), "wide kernel")
+        if "decode" in which:
+            for M in (1, 2):
+                for pos in (4096, 32768):
+                    name = f"decode ({M} row{'s' if M > 1 else ''}) at {pos}"
+                    for hint in ((0, pos) if pos < ctx else (0,)):
+                        for S in (0, 8, 16, 32, 48, 64, 96, 128, 192, 256):
+                            for fuse in (0, 1):
+                                opts = ((5, hint), (1, S), (7, fuse))
+                                emit(name, opts, timed(kv, L, q[:M], kn[:M], vn[:M], pos, opts), "32 containers of 32768 tokens; 4096: the first 4096 of each")
+        kv.close()
+    if "paged" in which:
+        ctx, L = 262144, 3
+        q, k, v = synth(32, ctx, 64)
+        kv = native.KvCache(n_layers=L, max_ctx=ctx + 256, max_rows=64, paged=True)
+        kv.set_page_table(np.random.default_rng(32).permutation((ctx + 256) // 256).astype(np.int32))
+        fill_cache(kv, k, v, ctx, chunk=16384)
+        for S in (0, 64, 96, 128, 192, 256):
+            emit("decode at 262144, shuffled pages", ((1, S),), timed(kv, L, q[:1], k[ctx:ctx + 1], v[ctx:ctx + 1], ctx, ((1, S),)))
+        for S in (0, 8, 12, 16, 21, 32, 42, 64):
+            emit("verify-64 at 262144, shuffled pages", ((2, S),), timed(kv, L, q, k[ctx:], v[ctx:], ctx, ((2, S),)))
+        kv.close()
+    if "prefill" in which:
+        ctx, M, L = 131072, 2048, 4
+        q, k, v = synth(31, ctx, M)
+        kv = native.KvCache(n_layers=L, max_ctx=ctx + M, max_rows=M)
+        fill_cache(kv, k, v, ctx, chunk=16384)
+        for slice_len in (0, 512, 683, 1024, 1366, 2048):
+            for S in (0, 1, 2, 3, 4, 6, 8):
+                if slice_len * S > 4096 or (slice_len == 0 and 1024 * S > 4096):
+                    continue                                  # more (token, split) pairs than the partial workspace holds
+                opts = ((10, slice_len), (2, S))
+                emit("prefill chunk 2048 rows at 131072", opts, timed(kv, L, q, k[ctx:], v[ctx:], ctx, opts))
+        kv.close()
+    return rows_out
+
+
 def big_configs(native):
     """Secondary figures for the two large configurations: the prefill chunk above and decode / verify-64 on 262144 tokens
     in shuffled 256-token pages."""
@@ -419,6 +498,9 @@ def main():
     ap.add_argument("--trellis-only", action="store_true",
                     help="run only the passes over trellis-coded rows (5 and 4 bits per element) and print their figures")
     ap.add_argument("--prefill-only", action="store_true", help="only run the 2048-row prefill chunk on 131072 cached tokens and print it")
+    ap.add_argument("--sweep", nargs="?", const="verify,decode,paged,prefill", default=None, metavar="GROUPS",
+                    help="time layer calls over the option keys that shape the launch (split counts, kernel choice, slice length, "
+                         "context hint) and print a table; GROUPS: comma-separated subset of verify,decode,paged,prefill")
     ap.add_argument("--machine", action="store_true", help="only run the machine probe (MFMA rate, read rate, overlap) and print it")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three device-to-device copies of 256 MiB (a kernel of known traffic, for scaling FETCH_SIZE / WRITE_SIZE)")
@@ -433,6 +515,9 @@ def main():
 
     if args.machine:
         print(json.dumps({"machine": machine_figures(native)}))
+        return
+    if args.sweep:
+        sweep(native, tuple(args.sweep.split(",")))
         return
     if args.prefill_only:
         print(json.dumps({"prefill_2048_at_131072": prefill_chunk(native, reps=8, opts=[tuple(int(x) for x in o.split("=")) for o in args.opt])}))
