@@ -66,3 +66,33 @@ def test_seeded_randomized_sweep(native, oracle):
             over.append((what, plain))
     # values two spacings off are possible (see the module docstring) but rare: none or a few of the 60 shapes
     assert len(over) <= 3, over
+
+
+@pytest.mark.parametrize("M", [1, 2, 8, 16, 64, 130])
+def test_large_magnitudes(native, oracle, M):
+    """Every kernel at the far end of the fp16 range: K rows of magnitude up to 6e4 (group scales up to 9e3), V rows of
+    magnitude up to 3e4, small queries so that the scores still discriminate.  The scaled K images of the mid kernel, the
+    exact codes x fp32 scales of the other two and the scaled V images all have to stay finite and exact."""
+    rng = np.random.default_rng(8800 + M)
+    ctx = 600
+    k = np.clip(rng.standard_normal((ctx + M, 4, 128)) * 9000.0, -60000, 60000).astype(np.float16)
+    v = np.clip(rng.standard_normal((ctx + M, 4, 128)) * 6000.0, -30000, 30000).astype(np.float16)
+    q = (rng.standard_normal((M, 24, 128)) * 1e-3).astype(np.float16)
+    max_ctx = 1024
+    oc = oracle.Cache(max_ctx)
+    with native.KvCache(max_ctx=max_ctx, max_rows=max(M, 64)) as kv:
+        kv.set_opt(8, 16)
+        kv.append_host(0, k[:ctx], v[:ctx], 0)
+        out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx)
+        oc.append(k, v, 0)
+        got = kv.export_rows(0, 0, ctx + M)
+        for a, b in zip(got, (oc.kc, oc.ks, oc.vc, oc.vs)):
+            assert (a == b[:, :ctx + M]).all()
+    ref32 = oc.attend_f32(q, ctx, threads=8, want_f32=True)[1]
+    assert np.isfinite(out.astype(np.float32)).all()
+    a, b = out.astype(np.float64), ref32.astype(np.float64)
+    assert np.linalg.norm(a - b) / np.linalg.norm(b) <= 1e-3
+    # a row is a weighted mean of V rows of magnitude ~1e4, each held as fp16(code x scale): the error of every channel
+    # scales with the magnitude of the row, not with the channel's own value
+    row_scale = np.abs(b).max(axis=2, keepdims=True)
+    assert (np.abs(a - b) <= 2e-3 * np.maximum(1.0, row_scale)).all(), (np.abs(a - b) / np.maximum(1.0, row_scale)).max()

@@ -261,7 +261,7 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
   }
 
   // Q fragments: B operand of S^T = K Q^T.  MFMA step m (= scale group m), lane (row i, lane group g), element e
-  // <-> channel 32m + 8g + pi(e), pi = [0,4,1,5,2,6,3,7] (the order dq_dword_int produces); odd channels carry 1/16.
+  // <-> channel 32m + 8g + pi(e), pi = [0,4,1,5,2,6,3,7] (the order dq_dword_int produces); odd channels carry 1/4, even ones 4.
   // The four loads are written as instructions and only requested here: the first tiles are requested right behind them
   // and q_ready<N> then waits for the query alone, leaving the N tile loads in flight - one trip to memory before the
   // first MFMA instead of two.  Padding lanes read row 0 of the slice (memory that exists) and drop it.
@@ -280,22 +280,25 @@ __global__ void __launch_bounds__(256, 2) attend_narrow_kernel(AttnArgs A) {
   auto q_ready = [&](auto n_younger) __attribute__((always_inline)) {
     uint32_t z;
     asm volatile("s_waitcnt vmcnt(%1)\n\tv_mov_b32 %0, 0" : "=v"(z) : "n"(decltype(n_younger)::value));
-    const _Float16 sx = (_Float16)0.0625f;
+    // the odd nibble of a byte enters the MFMA as 16 n: its query channels carry 1/4 and the others 4, so that both
+    // kinds of products are 4 q n and neither factor costs fp16 range at one end only (a plain 1/16 on the odd channels
+    // pushes queries below 1e-3 into the subnormals); the 4 leaves with the softmax scale
+    const _Float16 se = (_Float16)4.f, so = (_Float16)0.25f;
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
       const h8 c = __builtin_bit_cast(h8, vrow ? (qraw[m] | u32x4{z, z, z, z}) : u32x4{0u, 0u, 0u, 0u});
-      qf[m] = h8{c[0], c[4], c[1] * sx, c[5] * sx, c[2], c[6], c[3] * sx, c[7] * sx};
+      qf[m] = h8{c[0] * se, c[4] * se, c[1] * so, c[5] * so, c[2] * se, c[6] * se, c[3] * so, c[7] * so};
       // -8 * 2^-24 * (sum of the row's 32 query channels of group m): the lane's 8 channels, then its 3 sister lanes
       float qs = 0.f;
 #pragma unroll
       for (int e = 0; e < 8; ++e) qs += (float)c[e];
       qs += __shfl_xor(qs, 16, 64);
       qs += __shfl_xor(qs, 32, 64);
-      const float c0 = -8.f * kTwoM24 * qs;
+      const float c0 = -32.f * kTwoM24 * qs;       // -8 per code, in the units of the products: 4 q n 2^-24
       kinit[m] = f4{c0, c0, c0, c0};
     }
   };
-  const float sc_log2 = kTwo24 * kLog2e / sqrtf((float)kD);       // scores carry the 2^-24 of the subnormal codes
+  const float sc_log2 = 0.25f * kTwo24 * kLog2e / sqrtf((float)kD);   // scores carry the 2^-24 of the subnormal codes and the 4 of the query fragments
 
   float m_run = -1e30f, l_run = 0.f;
   f4 o[8];

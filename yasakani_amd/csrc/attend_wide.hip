@@ -198,12 +198,14 @@ __global__ void __launch_bounds__(NT) attend_wide_kernel(AttnArgs A) {
   h8 qf[8];
   {
     const uint16_t* qrow = A.q16 + ((size_t)tl * A.n_heads + head) * kD;
-    const _Float16 sx = (_Float16)0.0625f;
+    // the odd nibble of a byte is 16 (n - 8) in the K image: its query channels carry 1/4 and the others 4 (products 4 q n
+    // either way; a plain 1/16 would push small queries into the fp16 subnormals), the 4 leaves with the softmax scale
+    const _Float16 se = (_Float16)4.f, so = (_Float16)0.25f;
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       uint4 u = vrow ? *reinterpret_cast<const uint4*>(qrow + 32 * (ks >> 1) + 8 * (2 * (ks & 1) + h)) : make_uint4(0, 0, 0, 0);
       const h8 c = __builtin_bit_cast(h8, u);
-      qf[ks] = h8{c[0], c[4], c[1] * sx, c[5] * sx, c[2], c[6], c[3] * sx, c[7] * sx};
+      qf[ks] = h8{c[0] * se, c[4] * se, c[1] * so, c[5] * so, c[2] * se, c[6] * se, c[3] * so, c[7] * so};
     }
   }
   const bool has_rows = row0 < min(nrows, (rb + 1) * RPB);             // wave uniform
@@ -274,7 +276,7 @@ __global__ void __launch_bounds__(NT) attend_wide_kernel(AttnArgs A) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) o[dt][r] = 0.f;
 
-  const float sc_log2 = kLog2e / sqrtf((float)kD);
+  const float sc_log2 = 0.25f * kLog2e / sqrtf((float)kD);      // 1/4: the query fragments carry a factor 4
   Raw raw0{}, raw1{};                          // raw codes of the group's next two tiles: loads run two tiles ahead of their use
   const LaneOffs offs = lane_offs(gt, h);
   uint32_t magic = kMagic;
