@@ -5,14 +5,14 @@
 // and leaves (m, l, acc / l) partials for the combiner.  The shape of the work is the decode kernel's, not the wide
 // kernel's: a window of at most 16 tokens x 6 heads is at most six MFMA row tiles of 16 rows, few enough for ONE wave to
 // keep all their accumulators in registers (192 of the 512 a wave owns when it has its SIMD to itself).  So
-//   * a wave owns whole 32-key tiles, loads them with the decode kernel's loader (tile32_device.h: 16 explicit loads, the
-//     next tile in flight in a second register set) and dequantizes each tile ONCE into MFMA operands that stay in
-//     registers: K as exact integer codes, V scaled in fp16;
+//   * a wave owns whole 32-key tiles, loads them with 14 explicit loads (the next tile is in flight while the current one
+//     is worked on) and dequantizes each tile ONCE into MFMA operands that stay in registers: K as two exact scaled images
+//     (code x the upper 8 bits of the fp16 group scale, code x its lower 3 bits: both exact in fp16), V scaled in fp16;
 //   * it then walks the window's row tiles: query fragments come from LDS (staged once per workgroup in operand order:
-//     one conflict-free 16-byte read per lane and scale group), 8 score MFMAs, the K group scales applied to the fp32
-//     partial sums (K is never rounded), softmax with a lazily raised running maximum, 8 PV MFMAs into that row tile's
-//     accumulators.  Dequantization is paid once per tile instead of once per row tile, there is no LDS round trip
-//     for K / V and no barrier inside the loop;
+//     one conflict-free 16-byte read per lane and scale group), 16 score MFMAs chained over both images (the fp32
+//     accumulation adds them exactly: K is never rounded, and no multiply-add per score is left), softmax with a lazily
+//     raised running maximum, 8 PV MFMAs into that row tile's accumulators.  Dequantization is paid once per tile instead
+//     of once per row tile, there is no LDS round trip for K / V and no barrier inside the loop;
 //   * one workgroup (4 waves, one per SIMD) per compute unit; its waves take the tiles of the split round robin and are
 //     merged through LDS at the end, one row tile at a time (two buffers, one barrier per row tile);
 //   * the rows the pass appends are quantized and stored by the workgroups whose tiles hold them, before they load those
@@ -361,6 +361,10 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
     operand_ready(pf[(NRT - 1) & 1]);
 #pragma unroll
     for (int b = 0; b < 8; ++b) mfma_pv(o[NRT - 1][b], vf[b], pf[(NRT - 1) & 1]);
+    // The compiler may move accumulators between registers where control flow joins (it does at the loop's exit) and does
+    // not know that the instructions above are still writing them: their passes are drained here, once per tile.
+    asm volatile("s_nop 7" : "+a"(o[NRT - 1][0]), "+a"(o[NRT - 1][1]), "+a"(o[NRT - 1][2]), "+a"(o[NRT - 1][3]),
+                             "+a"(o[NRT - 1][4]), "+a"(o[NRT - 1][5]), "+a"(o[NRT - 1][6]), "+a"(o[NRT - 1][7]));
     __builtin_amdgcn_sched_barrier(0);
   };
 

@@ -4,7 +4,11 @@ The attention kernels keep tile loads in flight across loop iterations as hand-w
 counter waits, which the compiler does not know about.  Nothing may read or overwrite a register such a load will write
 until a `s_waitcnt vmcnt(N)` has retired the load: a register copy (or a spill) the compiler places between a load and its
 wait copies the register's previous contents, and the data that arrives later lands in a register that has been given
-to something else - an address, for instance.  `check_sources()` compiles each source it covers to assembly (device code
+to something else - an address, for instance.  The same kernels write out their PV matrix instructions by hand (so that the
+accumulators stay in the accumulator registers); the compiler does not know these are matrix instructions and keeps none
+of the wait states a vector instruction needs before it may read their results, so a register copy it places right behind
+one (where control flow joins, for instance) copies values the last passes have not written yet: `check_mfma_results`
+walks the instructions behind every hand-written matrix instruction for as many wait states as its passes need.  `check_sources()` compiles each source it covers to assembly (device code
 only, the flags of the library's Makefile) and walks every kernel along every path of its control flow.  It needs hipcc
 and no GPU.  Loads are assumed to return in the order issued.
 """
@@ -116,6 +120,109 @@ def check_kernel(lines):
     return [bad[k] for k in sorted(bad)]
 
 
+AREG = re.compile(r"\ba\[(\d+):(\d+)\]|\ba(\d+)\b")
+# wait states between a matrix instruction and a vector instruction that touches its result registers: 4-pass / 8-pass
+# instructions (one more than the hazard tables say)
+MFMA_WAIT = {"v_mfma_f32_16x16x32_f16": 8, "v_mfma_f32_32x32x16_f16": 12}
+
+
+def _aregs(text):
+    out = set()
+    for a, b, c in AREG.findall(text):
+        if c:
+            out.add(int(c))
+        else:
+            out.update(range(int(a), int(b) + 1))
+    return out
+
+
+def check_mfma_results(lines):
+    """For every hand-written matrix instruction: no other kind of instruction touches its result registers within the wait
+    states its passes need, along any path.  Returns (hand-written matrix instructions seen, violations)."""
+    ins, labels = _parse(lines)
+    bad, count = {}, 0
+    for p, (n, t, in_asm) in enumerate(ins):
+        op = t.split()[0]
+        if not (in_asm and op in MFMA_WAIT):
+            continue
+        count += 1
+        first = t.split(",")[0]
+        dst_a, dst_v = _aregs(first), _regs(first)         # the result lies in accumulator registers or in ordinary ones
+        work, seen = [(p + 1, MFMA_WAIT[op])], set()
+        while work:
+            pc, left = work.pop()
+            while pc < len(ins) and left > 0 and (pc, left) not in seen:
+                seen.add((pc, left))
+                n2, t2, _ = ins[pc]
+                op2 = t2.split()[0]
+                if op2 == "s_endpgm":
+                    break
+                if op2 == "s_nop":
+                    left -= int(t2.split()[1]) + 1
+                    pc += 1
+                    continue
+                if op2 == "s_branch":
+                    pc = labels[t2.split()[1]]
+                    left -= 1
+                    continue
+                if op2.startswith("s_cbranch"):
+                    work.append((labels[t2.split()[1]], left - 1))
+                elif not op2.startswith("v_mfma") and (_aregs(t2) & dst_a or _regs(t2) & dst_v):
+                    bad[(n, n2)] = (n2, t2, n, sorted(_aregs(t2) & dst_a) + sorted(_regs(t2) & dst_v))
+                left -= 1
+                pc += 1
+    return count, [bad[k] for k in sorted(bad)]
+
+
+def check_mfma_operands(lines):
+    """For every hand-written matrix instruction: none of the two instructions in front of it (wait states of `s_nop`
+    counted) is a vector instruction that writes one of its operands - a vector result is not forwarded to a matrix
+    instruction issued right behind it (the compiler keeps two wait states for its own).  Looks back in straight-line code
+    only: a label or a branch in between ends the search.  Returns the violations."""
+    bad = []
+    stream = []                                   # (kind, text, line) with labels kept, so that a join ends the look-back
+    in_asm = False
+    for n, raw in enumerate(lines):
+        t = raw.strip()
+        if t.startswith(";;#ASMSTART"):
+            in_asm = True
+            continue
+        if t.startswith(";;#ASMEND"):
+            in_asm = False
+            continue
+        if re.match(r"^\.L\w+:", t):
+            stream.append(("label", t, n + 1, False))
+            continue
+        if not t or t[0] in ";./" or t.endswith(":"):
+            continue
+        stream.append(("ins", t.split(";")[0].strip(), n + 1, in_asm))
+    for p, (kind, t, n, in_asm) in enumerate(stream):
+        if kind != "ins" or not in_asm or t.split()[0] not in MFMA_WAIT:
+            continue
+        ops = t.split(None, 1)[1].split(",")
+        srcs = set()
+        for o in ops[1:]:
+            srcs |= _regs(o)
+        left, q = 2, p - 1
+        while q >= 0 and left > 0:
+            k2, t2, n2, _ = stream[q]
+            if k2 == "label":
+                break
+            op2 = t2.split()[0]
+            if op2.startswith("s_cbranch") or op2 == "s_branch":
+                break
+            if op2 == "s_nop":
+                left -= int(t2.split()[1]) + 1
+            else:
+                if op2.startswith("v_") and not op2.startswith("v_mfma") and not op2.startswith("v_cmp"):
+                    w = _regs(t2.split(None, 1)[1].split(",")[0]) if " " in t2 else set()
+                    if w & srcs:
+                        bad.append((n, t, n2, t2, sorted(w & srcs)))
+                left -= 1
+            q -= 1
+    return bad
+
+
 def kernels_of(asm_text):
     """Splits an assembly file into (name, lines) per kernel."""
     out, name, cur = [], None, []
@@ -155,6 +262,11 @@ def check_sources(workdir, sources=SOURCES):
             seen += sum(1 for i, l in enumerate(lines) if "global_load" in l and i and "ASMSTART" in lines[i - 1])
             for n, t, regs in check_kernel(lines):
                 problems.append(f"{src} {name[:60]} line {n}: `{t[:80]}` touches v{regs} while their loads are in flight")
+            _, late = check_mfma_results(lines)
+            for n2, t2, n, regs in late:
+                problems.append(f"{src} {name[:60]} line {n2}: `{t2[:80]}` touches a{regs} before the matrix instruction of line {n} has written them")
+            for n, t, n2, t2, regs in check_mfma_operands(lines):
+                problems.append(f"{src} {name[:60]} line {n}: `{t[:70]}` reads v{regs} which `{t2[:60]}` (line {n2}) has only just written")
     return seen, problems
 
 
@@ -166,7 +278,8 @@ def main():
         problems.append(f"only {seen} hand-written loads found: the check looked at nothing")
     if problems:
         raise SystemExit("ISA check failed:\n" + "\n".join(problems[:40]))
-    print(f"ISA check: {seen} hand-written loads, no register touched while its load is in flight")
+    print(f"ISA check: {seen} hand-written loads, no register touched while its load is in flight; "
+          "no result of a hand-written matrix instruction touched before its passes are through")
 
 
 if __name__ == "__main__":
