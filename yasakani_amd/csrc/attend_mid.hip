@@ -91,7 +91,10 @@ template <int NRT>
 __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
   constexpr int TB = (16 * NRT) / kG;          // tokens per row block
   __shared__ __align__(16) uint4 s_q[NRT * 4 * 64];                 // [row tile][scale group][lane]: B operands of the score MFMAs
-  __shared__ __align__(16) float s_acc[2][4][16][kAccPitch];        // wave merge, ping-pong over row tiles
+  // wave merge: up to four row tiles are staged at once (one barrier for the whole merge), more go through two buffers
+  // in turn (one barrier per row tile)
+  constexpr int kStage = NRT <= 4 ? NRT : 2;
+  __shared__ __align__(16) float s_acc[kStage][4][16][kAccPitch];
   __shared__ float s_m[NRT][4][16], s_l[NRT][4][16];
   const int split = blockIdx.x, kvh = blockIdx.y, rb = blockIdx.z;
   const int tid = threadIdx.x;
@@ -392,23 +395,21 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
 #pragma unroll
   for (int rt = 0; rt < NRT; ++rt) pv_done(o[rt]);
 
-  // ---- merge the 4 waves row tile by row tile: every wave stages its accumulators, then thread (row j, 8 channels)
-  //      weighs the four and writes one normalised fp16 partial row piece.  o[rt][b][r] of lane (row i, group g) is
-  //      channel 8 (4g + r) + b. ----
-#pragma unroll
-  for (int rt = 0; rt < NRT; ++rt) {
-    if (16 * rt >= nrows) break;                   // uniform
+  // ---- merge the 4 waves: every wave stages its accumulators, then thread (row j, 8 channels) weighs the four and writes
+  //      one normalised fp16 partial row piece.  o[rt][b][r] of lane (row i, group g) is channel 8 (4g + r) + b. ----
+  auto stage = [&](int rt) __attribute__((always_inline)) {
     float l = l_run[rt];
     l += __shfl_xor(l, 16, 64);
     l += __shfl_xor(l, 32, 64);
     if (g == 0) { s_m[rt][wave][i] = m_run[rt]; s_l[rt][wave][i] = l; }
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
-      float* d = &s_acc[rt & 1][wave][i][8 * (4 * g + r)];
+      float* d = &s_acc[rt % kStage][wave][i][8 * (4 * g + r)];
       *reinterpret_cast<float4*>(d) = make_float4(o[rt][0][r], o[rt][1][r], o[rt][2][r], o[rt][3][r]);
       *reinterpret_cast<float4*>(d + 4) = make_float4(o[rt][4][r], o[rt][5][r], o[rt][6][r], o[rt][7][r]);
     }
-    __syncthreads();
+  };
+  auto reduce = [&](int rt) __attribute__((always_inline)) {
     const int j = tid >> 4, c8 = (tid & 15) * 8, R = 16 * rt + j;
     if (R < nrows) {
       const float m0 = s_m[rt][0][j], m1 = s_m[rt][1][j], m2 = s_m[rt][2][j], m3 = s_m[rt][3][j];
@@ -417,7 +418,7 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
       const float L = w[0] * s_l[rt][0][j] + w[1] * s_l[rt][1][j] + w[2] * s_l[rt][2][j] + w[3] * s_l[rt][3][j];
       float4 a0[4], a1[4];
 #pragma unroll
-      for (int wv = 0; wv < 4; ++wv) { a0[wv] = *reinterpret_cast<const float4*>(&s_acc[rt & 1][wv][j][c8]); a1[wv] = *reinterpret_cast<const float4*>(&s_acc[rt & 1][wv][j][c8 + 4]); }
+      for (int wv = 0; wv < 4; ++wv) { a0[wv] = *reinterpret_cast<const float4*>(&s_acc[rt % kStage][wv][j][c8]); a1[wv] = *reinterpret_cast<const float4*>(&s_acc[rt % kStage][wv][j][c8 + 4]); }
       float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int wv = 0; wv < 4; ++wv) {
@@ -431,6 +432,23 @@ __global__ void __launch_bounds__(256, 1) attend_mid_kernel(AttnArgs A) {
       const size_t p = ((size_t)(tokb + R / kG) * A.S + split) * A.n_heads + kvh * kG + R % kG;
       *reinterpret_cast<uint4*>(A.pacc16 + p * kD + c8) = __builtin_bit_cast(uint4, v);
       if (c8 == 0) { A.pm[p] = M2; A.pl[p] = L; }
+    }
+  };
+  if constexpr (NRT <= 4) {
+#pragma unroll
+    for (int rt = 0; rt < NRT; ++rt)
+      if (16 * rt < nrows) stage(rt);              // uniform
+    __syncthreads();
+#pragma unroll
+    for (int rt = 0; rt < NRT; ++rt)
+      if (16 * rt < nrows) reduce(rt);
+  } else {
+#pragma unroll
+    for (int rt = 0; rt < NRT; ++rt) {
+      if (16 * rt >= nrows) break;                 // uniform
+      stage(rt);
+      __syncthreads();
+      reduce(rt);
     }
   }
 }
