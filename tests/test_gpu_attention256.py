@@ -58,7 +58,7 @@ def test_attention_matches_oracle(native, oracle, ctx, M):
         out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx)
         got = kv.export_rows(0, ctx, M)
     ref.append(k[ctx:], v[ctx:], ctx)
-    # rows stored by the pass itself (inside the decode launch for M <= 2, by the append launch otherwise): bit-exact
+    # rows stored by the pass itself (inside the attention launch: by the workgroups whose key range holds them): bit-exact
     assert np.array_equal(got[0], ref.kc[:, ctx:ctx + M]) and np.array_equal(got[2], ref.vc[:, ctx:ctx + M])
     assert np.array_equal(got[1].view(np.uint32), ref.ks[:, ctx:ctx + M].view(np.uint32))
     assert np.array_equal(got[3].view(np.uint32), ref.vs[:, ctx:ctx + M].view(np.uint32))
@@ -107,6 +107,50 @@ def test_rows_no_query_row_sees_are_still_stored(native, oracle, ctx):
     assert np.array_equal(got[1].view(np.uint32), ref.ks[:, ctx:ctx + M].view(np.uint32))
     assert np.array_equal(got[3].view(np.uint32), ref.vs[:, ctx:ctx + M].view(np.uint32))
     assert_attn_close(out, ref.attend_f32(q, ctx, depth=depth), f"siblings at ctx={ctx}")
+
+
+def _rows_bit_exact(got, ref, ctx, M, what):
+    assert np.array_equal(got[0], ref.kc[:, ctx:ctx + M]) and np.array_equal(got[2], ref.vc[:, ctx:ctx + M]), what
+    assert np.array_equal(got[1].view(np.uint32), ref.ks[:, ctx:ctx + M].view(np.uint32)), what
+    assert np.array_equal(got[3].view(np.uint32), ref.vs[:, ctx:ctx + M].view(np.uint32)), what
+
+
+WINDOW_CASES = {
+    # a 64-row window that starts at an odd row of page 1 and ends in page 2 (rows of one wave lie in two pages)
+    "across a page, odd start": (2 * 256 - 21, 64, None),
+    # two row blocks
+    "two row blocks": (777, 40, None),
+    # siblings: no query row sees rows 1024..1028, which open a new tile past every key range
+    "unseen rows past the last tile": (1023, 6, [0] * 6),
+    # three row blocks, none of which sees past row 1000: rows 1024..1063 lie past the last tile of all of them
+    "64 siblings": (1000, 64, [0] * 64),
+    # the first row block reads further than the last one
+    "deep first block, shallow last": (900, 64, [63] * 32 + [0] * 32),
+}
+
+
+@pytest.mark.parametrize("paged", [False, True])
+@pytest.mark.parametrize("case", list(WINDOW_CASES))
+def test_windows_store_their_own_rows(native, oracle, case, paged):
+    """Passes of 3..64 rows quantize and store their rows inside the attention launch: every row bit-exact in the cache
+    afterwards, whichever workgroup held its tile, and the outputs as if the rows had been there before."""
+    ctx, M, dp = WINDOW_CASES[case]
+    depth = None if dp is None else np.array(dp, np.uint8)
+    q, k, v = _inputs(300 + ctx + M, ctx, M)
+    ref = oracle.Cache(1280, NH, KVH, D)
+    with native.KvCache(head_dim=D, max_ctx=1280, paged=paged) as kv:
+        if paged:
+            kv.set_page_table(np.array([3, 0, 4, 1, 2], np.int32))
+        _fill(kv, ref, k, v, ctx)
+        before = kv.export_rows(0, 0, ctx)
+        out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx, depth=depth)
+        got = kv.export_rows(0, ctx, M)
+        after = kv.export_rows(0, 0, ctx)
+    for a, b in zip(before, after):                       # nothing else was written
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), case
+    ref.append(k[ctx:], v[ctx:], ctx)
+    _rows_bit_exact(got, ref, ctx, M, case)
+    assert_attn_close(out, ref.attend_f32(q, ctx, depth=depth, threads=8), case)
 
 
 def test_entry_points_of_the_other_format_refuse(native):

@@ -224,8 +224,8 @@ void need_128(const yka_kv* kv) {
   if (kv->r256()) throw std::runtime_error("this entry point exists for head_dim 128 only");
 }
 
-// mode 0: attention + combine; 2: attention kernel alone.  k16/v16 != nullptr asks for quantize-on-append as well:
-// rows of at most 2 tokens fuse it into the attention launch, wider passes launch the append kernel first.
+// mode 0: attention + combine; 2: attention kernel alone.  k16/v16 != nullptr asks for quantize-on-append as well, which
+// rides in the attention launch wherever a kernel stores its own rows (see the branches below).
 struct Workspace { float* pm; float* pl; uint16_t* pacc16; size_t pairs; int* tickets; };
 void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_pos, const uint8_t* depth, uint16_t* out16,
                hipStream_t st, int mode = 0, const uint16_t* k16 = nullptr, const uint16_t* v16 = nullptr, const Workspace* ws = nullptr) {
@@ -257,9 +257,10 @@ void do_attend(yka_kv* kv, int layer, const uint16_t* q16, int M, const int* d_p
     return;
   }
   if (kv->r256()) {
-    // 256-channel rows: append first; rows of at most 2 tokens (or option key 3) run on row tiles of 2 tokens x 6 heads,
-    // two workgroups per CU; wider slices on 128-row workgroups of 8 waves, one per CU
-    const bool fuse256 = k16 && M <= 2;         // the decode kernel stores its own rows; wider passes launch the append first
+    // 256-channel rows: rows of at most 2 tokens (or option key 3) run on row tiles of 2 tokens x 6 heads, two workgroups
+    // per CU; wider slices on 128-row workgroups of 8 waves, one per CU.  Both kernels store the rows of a pass of one
+    // slice themselves; a wide pass forced through the decode kernel and a pass of several slices launch the append first.
+    const bool fuse256 = k16 && (M <= 2 || (M <= kMaxSlice && !kv->opt_force_narrow));
     if (k16 && !fuse256) do_append(kv, layer, k16, v16, M, d_pos, st);
     const int ctx = kv->opt_ctx_hint > 0 ? std::min(kv->opt_ctx_hint, kv->cfg.max_ctx) : kv->cfg.max_ctx;
     for (int s0 = 0; s0 < M; s0 += kMaxSlice) {

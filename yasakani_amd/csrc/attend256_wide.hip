@@ -9,7 +9,9 @@
 //   * a wave owns 16 rows (MFMA 16x16x32: 16 accumulator tiles of 4 registers cover the 256 output channels, the query
 //     fragments take 32 registers), so that two waves fit a SIMD;
 //   * LDS is double buffered: tile n+1 is dequantized while tile n is consumed; one barrier per tile; the tile loads are
-//     explicit instructions two tiles ahead with their own waits.
+//     explicit instructions two tiles ahead with their own waits;
+//   * quantize-on-append rides in the launch: a workgroup stores the rows of the pass that fall into the tiles of its own
+//     split before it reads them (32 lanes per row, a word of 8 channels each).
 // LDS image of one tile (42240 bytes):
 //   K  [32 keys][544 B]    chunk c (16 bytes) of a key = word c of its row = channels 8c + [7,3,6,2,5,1,4,0]
 //   V  [256 channels][96 B] key 16kb + 4g + r sits at slot 8g + 4kb + r: the 8 keys whose probabilities an MFMA lane of
@@ -117,6 +119,37 @@ __device__ __forceinline__ void dequant_to_lds(uint8_t* buf, int tid, const Raw&
   reinterpret_cast<uint32_t*>(buf + kLdsS)[tid & 63] = R.sc;      // waves repeat each other (no divergent branch)
 }
 
+// One 256-channel row by 32 lanes: lane c holds channels 8c .. 8c+7 as 8 fp16 in `raw` and builds word c.  Bit-identical
+// to the row quantizer of the append kernel: the maximum of the row is exact in any order, everything behind it is the
+// same sequence of IEEE operations per channel.  All 32 lanes of the row call it; `store` is uniform over them.
+__device__ __forceinline__ void quant_store_word256(const KvView& kv, int kvh, int pos, bool isv, uint4 raw, int c, bool store) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+  float x[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) x[e] = __half2float(__ushort_as_half((uint16_t)(w[e >> 1] >> (16 * (e & 1)))));
+  float am = fabsf(x[0]);
+#pragma unroll
+  for (int e = 1; e < 8; ++e) am = fmaxf(am, fabsf(x[e]));
+#pragma unroll
+  for (int o = 1; o < 32; o <<= 1) am = fmaxf(am, __shfl_xor(am, o, 64));
+  float s7 = __fdiv_rn(am, 7.f);
+  if (s7 == 0.f) s7 = 1.f;
+  uint32_t word = 0u;                          // channel 8c + e in bits [28 - 4e, 32 - 4e): the first field on top
+#pragma unroll
+  for (int e = 0; e < 8; ++e) {
+    float q = rintf(__fdiv_rn(x[e], s7));
+    q = fminf(fmaxf(q, -7.f), 7.f);
+    word |= (uint32_t)((int)q + 8) << (28 - 4 * e);
+  }
+  if (store) {
+    const int lp = pos / kPageTok, tp = pos % kPageTok;
+    const int pp = kv.table ? kv.table[lp] : lp;             // rows of one wave may lie in two pages: a load per lane
+    uint8_t* pg = kv.base + (size_t)(pp * kv.n_kv + kvh) * kPage256Bytes;
+    reinterpret_cast<uint32_t*>(pg + (isv ? kP2Vw : kP2Kw))[tp * 32 + c] = word;
+    if (c == 0) reinterpret_cast<float*>(pg + (isv ? kP2Vs : kP2Ks))[tp] = s7;
+  }
+}
+
 }  // namespace
 
 // grid (S, n_kv, ceil(6M / 128)), block 512; wave w owns rows [16 w, 16 (w+1)) of the block
@@ -155,6 +188,40 @@ __global__ void __launch_bounds__(NT, 1) attend256_wide_kernel(AttnArgs A) {
   const int maxlen = min(pos + maxdep + 1, A.kv.max_ctx), minlen = min(pos + mindep + 1, A.kv.max_ctx);
   const int ntiles = (maxlen + 31) >> 5, tps = (ntiles + A.S - 1) / A.S;
   const int tile0 = split * tps, tile1 = min(ntiles, tile0 + tps);
+
+  // ---- fused quantize-on-append (a slice of at most 64 tokens): a workgroup stores the rows of this pass that lie in
+  //      the tiles of its own range before it reads them, so no workgroup reads a row another one has to store.  Row
+  //      blocks of one kv head write identical bytes where their ranges overlap.  A row past the last tile of the last
+  //      row block (no query row of the pass sees it: a depth table may say so) is stored by that block's last split.
+  //      Writer and readers are waves of one CU and one write-through L1: workgroup-scope fences order the stores.
+  //      Every condition that guards the barrier is uniform over the workgroup. ----
+  if (A.k16) {
+    static_assert(kMaxSlice <= 64, "8 steps of 16 rows cover K and V of a slice");
+    const int r0 = pos + A.tok0;
+    const int Tn0 = r0 >> 5, Tn1 = (r0 + A.M - 1) >> 5;
+    const bool last_wg = split == A.S - 1 && rb == (int)gridDim.z - 1;
+    if ((Tn0 < tile1 && Tn1 >= tile0) || (last_wg && Tn1 >= ntiles)) {
+      const int slot = tid >> 5, c = tid & 31;
+      uint4 rawv[8];
+      bool mine[8];
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const int hh = it * 16 + slot, t = hh >> 1, r = r0 + t, T = r >> 5;
+        mine[it] = t < A.M && r >= 0 && r < A.kv.max_ctx && ((T >= tile0 && T < tile1) || (last_wg && T >= ntiles));
+        const uint16_t* src = ((hh & 1) ? A.v16 : A.k16) + ((size_t)(A.tok0 + t) * A.kv.n_kv + kvh) * kD2 + 8 * c;
+        rawv[it] = mine[it] ? *reinterpret_cast<const uint4*>(src) : make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int it = 0; it < 8; ++it) {
+        const int hh = it * 16 + slot;
+        quant_store_word256(A.kv, kvh, r0 + (hh >> 1), hh & 1, rawv[it], c, mine[it]);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      __syncthreads();
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+      asm volatile("" ::: "memory");           // the tile loads below are instructions the compiler does not see as loads
+    }
+  }
 
   const float sc_log2 = kLog2e * 0.0625f;      // log2(e) / sqrt(256)
   float m_run = -1e30f, l_run = 0.f;           // m_run in log2 units, shared by the four lanes of a row
