@@ -153,6 +153,33 @@ def test_windows_store_their_own_rows(native, oracle, case, paged):
     assert_attn_close(out, ref.attend_f32(q, ctx, depth=depth, threads=8), case)
 
 
+def test_seeded_sweep_of_windows(native, oracle):
+    """40 seeded cases: context lengths around tile and page boundaries, 1..64 rows, a random depth table (row t sees up
+    to t rows of the pass) or none, paged or contiguous: stored rows bit-exact, outputs within the attention bars."""
+    rng = np.random.default_rng(4256)
+    for case in range(40):
+        ctx = int(rng.choice([0, 1, 31, 32, 33, 255, 256, 257, 511, int(rng.integers(0, 2200)), int(rng.integers(0, 2200))]))
+        M = int(rng.choice([1, 2, 3, 5, 16, 21, 22, 23, 43, 64, int(rng.integers(1, 65))]))
+        depth = None
+        if rng.random() < 0.5:
+            depth = np.array([int(rng.integers(0, t + 1)) for t in range(M)], np.uint8)
+        paged = bool(rng.random() < 0.5)
+        max_ctx = ((ctx + M + 255) // 256 + int(rng.integers(0, 2))) * 256
+        what = f"case {case}: ctx={ctx} M={M} depth={'yes' if depth is not None else 'no'} paged={paged} max_ctx={max_ctx}"
+        print(what, flush=True)
+        q, k, v = _inputs(5000 + case, ctx, M)
+        ref = oracle.Cache(max_ctx, NH, KVH, D)
+        with native.KvCache(head_dim=D, max_ctx=max_ctx, paged=paged) as kv:
+            if paged:
+                kv.set_page_table(rng.permutation(max_ctx // 256).astype(np.int32))
+            _fill(kv, ref, k, v, ctx)
+            out = kv.layer_call(0, q, k[ctx:], v[ctx:], ctx, depth=depth)
+            got = kv.export_rows(0, ctx, M)
+        ref.append(k[ctx:], v[ctx:], ctx)
+        _rows_bit_exact(got, ref, ctx, M, what)
+        assert_attn_close(out, ref.attend_f32(q, ctx, depth=depth, threads=8), what)
+
+
 def test_entry_points_of_the_other_format_refuse(native):
     with native.KvCache(head_dim=D, max_ctx=256) as kv:
         with pytest.raises(native.YkaError, match="128"):
