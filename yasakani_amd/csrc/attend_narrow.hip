@@ -482,8 +482,9 @@ void launch_attend_narrow(const AttnArgs& A, hipStream_t st) {
 // combiner (reference: src/attention_kv4q.cu:325-332): M2 = max pm; w_s = pm_s > -1e29 ? 2^(pm_s - M2) * pl_s : 0;
 // y = sum w_s * (acc_s / l_s) / sum w_s.  grid (n_heads, M), block 256: 16 lanes x 8 channels cover a row, 16 split
 // lanes run in parallel and are summed through LDS.  S <= 256.
-// kInFlight = partial rows a split lane requests before it uses any: 16 covers 256 splits in one memory round trip (few,
-// long workgroups: decode); 4 keeps the register count low where thousands of workgroups run (wide windows).
+// kInFlight = partial rows a split lane requests before it uses any: 16 covers 256 splits in one memory round trip, 8
+// covers the 128 splits of decode over long contexts (few, long workgroups); 4 keeps the register count low where
+// thousands of workgroups run (wide windows).
 template <int kInFlight>
 __global__ void __launch_bounds__(256) combine_kernel(CombineArgs A) {
   __shared__ float s_w[256];
@@ -604,7 +605,8 @@ __global__ void __launch_bounds__(256) combine_rows_kernel(CombineArgs A) {
 }
 void launch_combine(const CombineArgs& A, hipStream_t st) {
   if (A.S <= 32 && !A.unrot && A.M >= 8) { hipLaunchKernelGGL(combine_rows_kernel, dim3((A.M * A.n_heads + 3) / 4), dim3(256), 0, st, A); return; }
-  if (A.S > 64) hipLaunchKernelGGL(combine_kernel<16>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);    // S <= 256
+  if (A.S > 128) hipLaunchKernelGGL(combine_kernel<16>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);   // S <= 256
+  else if (A.S > 64) hipLaunchKernelGGL(combine_kernel<8>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
   else hipLaunchKernelGGL(combine_kernel<4>, dim3(A.n_heads, A.M), dim3(256), 0, st, A);
 }
 
